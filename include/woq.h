@@ -1,0 +1,207 @@
+/*
+ * libwoq — MI355X (gfx950) weight-only quantized matmul, C ABI.
+ *
+ * This is the drop-in boundary for the computation behind TensorRT-LLM's
+ * WeightOnlyQuantMatmulPlugin and WeightOnlyGroupwiseQuantMatmulPlugin.  TensorRT does not
+ * exist on ROCm, so the boundary sits one level under the plugins' `enqueue`: at the pair
+ *   weight_only::kernel_launcher(arch, Params&, stream)          (small-M kernel) and
+ *   CutlassFpAIntBGemmRunner::gemm(A, B, scales, zeros, bias, alpha, C, m, n, k, group, ...)
+ * and at the torch custom ops that prepare weights.  Every entry point below names the
+ * reference interface it replaces (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - plain C types only; all device pointers are HIP device pointers; `stream` is a hipStream_t
+ *     passed as void* (NULL = the default stream);
+ *   - every function returns 0 on success or a negative woq_status; the message of the last
+ *     failure on the calling thread is available from woq_last_error();
+ *   - nothing is thrown across the boundary, nothing is allocated on the device by woq_matmul
+ *     (the caller supplies the workspace), the library keeps no per-call state, and calls on
+ *     different streams may run concurrently.
+ */
+#ifndef WOQ_H_
+#define WOQ_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define WOQ_ABI_VERSION 1
+/* tag of the preprocessed-weight byte layout (gfx950 tile layout, see woq_preprocess_weights) */
+#define WOQ_LAYOUT_VERSION 1
+
+typedef enum woq_status
+{
+    WOQ_OK = 0,
+    WOQ_ERR_INVALID_ARGUMENT = -1, /* null pointer, bad enum, inconsistent optional inputs */
+    WOQ_ERR_BAD_SHAPE = -2,        /* m/n/k/group_size violate an alignment rule */
+    WOQ_ERR_UNSUPPORTED = -3,      /* a combination the reference also rejects (e.g. W4A8 with g64) */
+    WOQ_ERR_WORKSPACE = -4,        /* workspace missing or smaller than woq_workspace_bytes() */
+    WOQ_ERR_RUNTIME = -5,          /* a HIP call failed (no device, launch failure) */
+    WOQ_ERR_VALUE = -6             /* data out of range (e.g. an int4 value outside [-8, 7]) */
+} woq_status;
+
+/* element types of activations / scales / outputs
+ * (the plugins' `type_id`: nvinfer1::DataType kHALF / kBF16; fp8 only as a W4A8 activation) */
+typedef enum woq_dtype
+{
+    WOQ_FP16 = 0,
+    WOQ_BF16 = 1,
+    WOQ_FP8_E4M3 = 2, /* OCP e4m3fn */
+    WOQ_FP32 = 3      /* only as a host-side weight/scale type of woq_symmetric_quantize */
+} woq_dtype;
+
+/* cutlass_kernels::QuantType — cpp/tensorrt_llm/kernels/cutlass_kernels/cutlass_preprocessors.h:32-48 */
+typedef enum woq_quant_type
+{
+    WOQ_W8_A16 = 0,
+    WOQ_W4_A16 = 1,
+    WOQ_W4_AFP8 = 2
+} woq_quant_type;
+
+/* quant_algo bit flags of the groupwise plugin —
+ * cpp/tensorrt_llm/plugins/weightOnlyGroupwiseQuantMatmulPlugin/weightOnlyGroupwiseQuantMatmulPlugin.cpp:29-37 */
+#define WOQ_ALGO_BIAS 1
+#define WOQ_ALGO_ZERO 2
+#define WOQ_ALGO_PRE_QUANT_SCALE 4
+#define WOQ_ALGO_FP8_ALPHA 8 /* W4A8: fp8 MFMA path, `alpha` applied in the epilogue */
+#define WOQ_ALGO_INT8_WEIGHT 16
+
+/* which kernel family runs; AUTO follows the M-regime rule of woq_select_regime() */
+typedef enum woq_regime
+{
+    WOQ_REGIME_AUTO = 0,
+    WOQ_REGIME_STREAM = 1, /* weight-streaming kernel (decode GEMV / skinny M) */
+    WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMM (prefill) */
+} woq_regime;
+
+/*
+ * One matmul call.  Replaces weight_only::Params
+ * (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/common.h:63-101) and the argument lists of
+ * CutlassFpAIntBGemmRunnerInterface::gemm
+ * (cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm.h:55-96); field meaning
+ * follows the plugins' enqueue (weightOnlyQuantMatmulPlugin.cpp:283-339,
+ * weightOnlyGroupwiseQuantMatmulPlugin.cpp:407-495):
+ *
+ *   out[m, n] = T( alpha * sum_k  S(act[m, k]) * W[k, n]  + bias[n] )
+ *   W[k, n]   = q[k, n] * scales[g(k), n] + zeros[g(k), n]      (zeros are additive, pre-scaled)
+ *   S(a)      = a * pre_quant_scale[k] when given, else a
+ *
+ *   act              [m, k]            act_dtype (fp16 / bf16; fp8 e4m3 only with FP8_ALPHA)
+ *   pre_quant_scale  [k]               out_dtype, required iff quant_algo & PRE_QUANT_SCALE
+ *   weight           woq_preprocessed_bytes(k, n, quant_type) bytes from woq_preprocess_weights
+ *   scales           [k/group_size, n] or [n] when group_size == 0 (one scale per column);
+ *                    out_dtype, except W4A8 where they hold fp16 whatever out_dtype is
+ *   zeros            same shape/type as scales, required iff quant_algo & ZERO
+ *   bias             [n]               out_dtype, required iff quant_algo & BIAS
+ *   out              [m, n]            out_dtype
+ *   n                LOGICAL number of output columns (the reference plugins receive the packed
+ *                    column count and multiply it back: `real_n`)
+ *   group_size       0 (per-channel, the WeightOnlyQuantMatmul plugin), 64 or 128
+ *   alpha            used only with FP8_ALPHA; otherwise must be 1 or is ignored as in the reference
+ *   workspace        device scratch of at least woq_workspace_bytes(...) bytes (may be NULL when
+ *                    that is 0)
+ */
+typedef struct woq_matmul_args
+{
+    const void* act;
+    const void* pre_quant_scale;
+    const void* weight;
+    const void* scales;
+    const void* zeros;
+    const void* bias;
+    void* out;
+    float alpha;
+    int32_t m;
+    int32_t n;
+    int32_t k;
+    int32_t group_size;
+    int32_t quant_algo; /* WOQ_ALGO_* bits */
+    int32_t act_dtype;  /* woq_dtype of `act` */
+    int32_t out_dtype;  /* woq_dtype of out / scales / zeros / bias / pre_quant_scale: fp16 or bf16 */
+    int32_t regime;     /* woq_regime; 0 = automatic */
+    void* workspace;
+    size_t workspace_bytes;
+} woq_matmul_args;
+
+/* Runs the matmul on `stream`.  m == 0 returns WOQ_OK at once (weightOnlyQuantMatmulPlugin.cpp:303).
+ * Replaces the bodies of both plugins' enqueue(): kernel_launcher(...) for small m and
+ * apply_per_channel_scale + Runner::gemm(...) otherwise. */
+int woq_matmul(const woq_matmul_args* args, void* stream);
+
+/* Validates exactly like woq_matmul but launches nothing (usable without a GPU). */
+int woq_matmul_check(const woq_matmul_args* args);
+
+/* Device scratch woq_matmul needs for this problem.  Replaces
+ * CutlassFpAIntBGemmRunner::getWorkspaceSize (fpA_intB_gemm_template.h:549-582) plus the
+ * plugin's own m*k*sizeof(half) smoothing buffer (weightOnlyGroupwiseQuantMatmulPlugin.cpp:377-379). */
+size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype);
+
+/* The regime AUTO picks for a given m.  Counterpart of the tactic choice
+ * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
+int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
+
+/* ---- host-side weight preparation (CPU buffers) ------------------------------------------- */
+
+/* Bytes of the preprocessed weight of one [k, n] matrix.  Equals k*n*bits/8 whenever k is a
+ * multiple of 128 (int4) / 64 (int8); otherwise K is padded up to that multiple. */
+size_t woq_preprocessed_bytes(int64_t k, int64_t n, int32_t quant_type);
+
+/* Row-major signed [experts, k, n] (int4: two per byte along n, low nibble first) ->
+ * the opaque layout the kernels of THIS library read.  Same contract as
+ * preprocess_weights_for_mixed_gemm (cutlass_preprocessors.cpp:564-615; torch op
+ * trtllm::preprocess_weights_for_mixed_gemm, thop/weightOnlyQuantOp.cpp:123-151): lossless,
+ * arch-specific bytes.  Requires n % 16 == 0 and k % 32 == 0. */
+int woq_preprocess_weights(void* dst, const void* src, int64_t experts, int64_t k, int64_t n, int32_t quant_type);
+
+/* Inverse of woq_preprocess_weights (no reference counterpart: the reference layout is
+ * write-only; provided so the layout is testable and checkpoints can be converted back). */
+int woq_unpreprocess_weights(void* dst_row_major, const void* src, int64_t experts, int64_t k, int64_t n,
+    int32_t quant_type);
+
+/* Decodes a buffer produced by the REFERENCE's preprocess_weights_for_mixed_gemm on SM `arch`
+ * (80..89 / >=100: permute+transpose+interleave+bias; 90: no column interleave) back to
+ * row-major signed, so existing TensorRT-LLM checkpoints can be re-laid-out for gfx950.
+ * Inverts cutlass_preprocessors.cpp:163-615. */
+int woq_import_reference_weights(void* dst_row_major, const void* src_reference_layout, int64_t experts, int64_t k,
+    int64_t n, int32_t quant_type, int32_t arch);
+
+/* Per-column symmetric quantizer + preprocess.  Replaces symmetric_quantize<ComputeType, WeightType>
+ * (cutlass_preprocessors.cpp:652-762) behind trtllm::symmetric_quantize_last_axis_of_batched_matrix
+ * and trtllm::_symmetric_quantize_last_axis_of_batched_matrix (thop/weightOnlyQuantOp.cpp:153-251).
+ * weight [experts, k, n] of weight_dtype (fp32/fp16/bf16); scales [experts, n] of scale_dtype;
+ * `processed` (preprocessed bytes) and `unprocessed` (row-major packed) may each be NULL. */
+int woq_symmetric_quantize(void* processed, void* unprocessed, void* scales, const void* weight, int64_t experts,
+    int64_t k, int64_t n, int32_t quant_type, int32_t weight_dtype, int32_t scale_dtype);
+
+/* trtllm::pack_int8_tensor_to_packed_int4 / trtllm::unpack_int4_packed_tensor_to_int8
+ * (thop/weightOnlyQuantOp.cpp:284-353).  n_unpacked must be even. */
+int woq_pack_int4(void* packed, const void* unpacked_int8, size_t n_unpacked);
+int woq_unpack_int4(void* unpacked_int8, const void* packed, size_t n_packed);
+
+/* ---- device helpers ------------------------------------------------------------------------ */
+
+/* out[m, k] = T_out(T_in(act[m, k] * scale[k])), T_out = T_in or fp8 e4m3.  Replaces
+ * apply_per_channel_scale_kernel_launcher<T_in, T_out> (kernels/preQuantScaleKernel.cu:42-149). */
+int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m, int32_t k,
+    int32_t in_dtype, int32_t out_dtype, void* stream);
+
+/* Materialises W[k, n] = T(q*scale + zero) from preprocessed weights with the same device code
+ * the GEMM main loop uses (counterpart of the identity-activation round trip in
+ * tests/quantization/test_weight_only_quant_matmul.py:147-164).  dtype fp16/bf16, or fp8 e4m3
+ * with fp16 scales (the W4A8 B operand). */
+int woq_dequantize(void* out, const void* weight, const void* scales, const void* zeros, int32_t k, int32_t n,
+    int32_t group_size, int32_t quant_type, int32_t dtype, void* stream);
+
+/* ---- misc ------------------------------------------------------------------------------------ */
+
+const char* woq_last_error(void);
+int woq_abi_version(void);
+int woq_layout_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WOQ_H_ */

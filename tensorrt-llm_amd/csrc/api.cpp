@@ -1,0 +1,232 @@
+// The matmul entry points of libwoq: argument validation, M-regime selection and dispatch to the
+// kernel launchers.  This is the counterpart of the two plugins' enqueue()
+// (cpp/tensorrt_llm/plugins/weightOnlyQuantMatmulPlugin/weightOnlyQuantMatmulPlugin.cpp:283-339,
+// cpp/tensorrt_llm/plugins/weightOnlyGroupwiseQuantMatmulPlugin/weightOnlyGroupwiseQuantMatmulPlugin.cpp:407-495),
+// of the small-M dispatcher (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernelDispatcher.h:30-166)
+// and of the runner's argument checks
+// (cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:129-196).
+#include <cstdlib>
+#include <cstring>
+
+#include "woq_internal.h"
+
+namespace woq
+{
+int launch_stream_BF16_4(MatmulProblem const& p, void* stream);
+int launch_stream_BF16_8(MatmulProblem const& p, void* stream);
+int launch_stream_FP16_4(MatmulProblem const& p, void* stream);
+int launch_stream_FP16_8(MatmulProblem const& p, void* stream);
+
+int launch_stream(MatmulProblem const& p, void* stream)
+{
+    if (p.m > kStreamMaxM)
+        return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
+            p.m);
+    if (p.w4a8)
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 runs on the fp8 MFMA GEMM kernel only");
+    if (p.out_dtype == WOQ_BF16)
+        return p.bits == 4 ? launch_stream_BF16_4(p, stream) : launch_stream_BF16_8(p, stream);
+    return p.bits == 4 ? launch_stream_FP16_4(p, stream) : launch_stream_FP16_8(p, stream);
+}
+
+namespace
+{
+
+// Environment override of the regime, for experiments: WOQ_FORCE_REGIME=stream|gemm
+int env_regime()
+{
+    char const* e = std::getenv("WOQ_FORCE_REGIME");
+    if (!e)
+        return WOQ_REGIME_AUTO;
+    if (!std::strcmp(e, "stream"))
+        return WOQ_REGIME_STREAM;
+    if (!std::strcmp(e, "gemm"))
+        return WOQ_REGIME_GEMM;
+    return WOQ_REGIME_AUTO;
+}
+
+int validate(woq_matmul_args const* a, MatmulProblem& p)
+{
+    if (!a)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "args is NULL");
+    if (a->m < 0 || a->n <= 0 || a->k <= 0)
+        return fail(WOQ_ERR_BAD_SHAPE, "m, n, k must be non-negative / positive (got %d, %d, %d)", a->m, a->n, a->k);
+    if (a->out_dtype != WOQ_FP16 && a->out_dtype != WOQ_BF16)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "No valid weightOnlyQuantMatmul configuration: out_dtype must be fp16 or bf16");
+    int const algo = a->quant_algo;
+    if (algo & ~(WOQ_ALGO_BIAS | WOQ_ALGO_ZERO | WOQ_ALGO_PRE_QUANT_SCALE | WOQ_ALGO_FP8_ALPHA | WOQ_ALGO_INT8_WEIGHT))
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown quant_algo bits 0x%x", algo);
+    bool const w4a8 = algo & WOQ_ALGO_FP8_ALPHA;
+    if (w4a8 && (algo & WOQ_ALGO_INT8_WEIGHT))
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A(fp)8 kernel requires INT4 weight!");
+    if (a->act_dtype == WOQ_FP8_E4M3)
+    {
+        if (!w4a8)
+            return fail(WOQ_ERR_INVALID_ARGUMENT, "fp8 activations need quant_algo FP8_ALPHA");
+        if (algo & WOQ_ALGO_PRE_QUANT_SCALE)
+            return fail(WOQ_ERR_INVALID_ARGUMENT, "fp8 activations are already smoothed: PRE_QUANT_SCALE not allowed");
+    }
+    else if (a->act_dtype != a->out_dtype)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "activation dtype must equal out_dtype (or be fp8 for W4A8)");
+    else if (w4a8 && !(algo & WOQ_ALGO_PRE_QUANT_SCALE))
+        return fail(WOQ_ERR_INVALID_ARGUMENT,
+            "W4A8 with fp16/bf16 activations needs PRE_QUANT_SCALE (the smoothing pass is what casts to fp8)");
+    if (a->group_size != 0 && a->group_size != 64 && a->group_size != 128)
+        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 (per-channel), 64 or 128 (got %d)", a->group_size);
+    if (w4a8 && a->group_size != 128)
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 supports group_size 128 only (got %d)", a->group_size);
+    if (!a->act || !a->weight || !a->out)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "act, weight and out must not be NULL");
+    if (!a->scales)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "Weight scales must always be set to a non-null value.");
+    if (a->group_size == 0 && (a->zeros || (algo & WOQ_ALGO_ZERO)))
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "Weight zero pointer must be a nullptr for scale only ops");
+    if (((algo & WOQ_ALGO_ZERO) != 0) != (a->zeros != nullptr))
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "zeros must be given exactly when quant_algo has ZERO");
+    if (((algo & WOQ_ALGO_BIAS) != 0) != (a->bias != nullptr))
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "bias must be given exactly when quant_algo has BIAS");
+    if (((algo & WOQ_ALGO_PRE_QUANT_SCALE) != 0) != (a->pre_quant_scale != nullptr))
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "pre_quant_scale must be given exactly when quant_algo has PRE_QUANT_SCALE");
+    int const k_align = w4a8 ? 128 : 64;
+    if (a->k % k_align)
+        return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of %d (got %d)", k_align, a->k);
+    if (a->group_size && a->k % a->group_size)
+        return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of group_size (got %d, %d)", a->k, a->group_size);
+    if (a->n % kTileN)
+        return fail(WOQ_ERR_BAD_SHAPE, "n must be a multiple of %d (got %d)", kTileN, a->n);
+    if (a->regime != WOQ_REGIME_AUTO && a->regime != WOQ_REGIME_STREAM && a->regime != WOQ_REGIME_GEMM)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", a->regime);
+
+    p.act = a->act;
+    p.pre_quant_scale = a->pre_quant_scale;
+    p.weight = a->weight;
+    p.scales = a->scales;
+    p.zeros = a->zeros;
+    p.bias = a->bias;
+    p.out = a->out;
+    p.alpha = w4a8 ? a->alpha : 1.f;
+    p.m = a->m;
+    p.n = a->n;
+    p.k = a->k;
+    p.group_size = a->group_size;
+    p.bits = (algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
+    p.out_dtype = a->out_dtype;
+    p.act_dtype = a->act_dtype;
+    p.w4a8 = w4a8;
+    p.workspace = a->workspace;
+    p.workspace_bytes = a->workspace_bytes;
+    return WOQ_OK;
+}
+
+int pick_regime(woq_matmul_args const* a)
+{
+    int r = a->regime != WOQ_REGIME_AUTO ? a->regime : env_regime();
+    if (r == WOQ_REGIME_AUTO)
+        r = woq_select_regime(a->m, a->n, a->k, a->quant_algo);
+    return r;
+}
+
+} // namespace
+} // namespace woq
+
+using namespace woq;
+
+extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo)
+{
+    (void) n;
+    (void) k;
+    if (quant_algo & WOQ_ALGO_FP8_ALPHA)
+        return WOQ_REGIME_GEMM;
+    return m <= kStreamMaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
+}
+
+extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype)
+{
+    (void) n;
+    (void) act_dtype;
+    if (m <= 0 || k <= 0)
+        return 0;
+    // the GEMM regime smooths activations into the workspace first (the streaming kernel fuses it)
+    if (quant_algo & WOQ_ALGO_PRE_QUANT_SCALE)
+        return (size_t) m * (size_t) k * 2;
+    return 0;
+}
+
+extern "C" int woq_matmul_check(const woq_matmul_args* args)
+{
+    MatmulProblem p;
+    if (int rc = validate(args, p))
+        return rc;
+    int const regime = pick_regime(args);
+    if (regime == WOQ_REGIME_STREAM && args->m > kStreamMaxM)
+        return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
+            args->m);
+    if (regime == WOQ_REGIME_STREAM && p.w4a8)
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 runs on the fp8 MFMA GEMM kernel only");
+    if (regime == WOQ_REGIME_GEMM && p.pre_quant_scale)
+    {
+        size_t const need = woq_workspace_bytes(p.m, p.n, p.k, args->quant_algo, p.act_dtype);
+        if (p.m > 0 && (!p.workspace || p.workspace_bytes < need))
+            return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
+                p.workspace ? p.workspace_bytes : (size_t) 0);
+    }
+    return WOQ_OK;
+}
+
+extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
+{
+    if (int rc = woq_matmul_check(args))
+        return rc;
+    MatmulProblem p;
+    validate(args, p);
+    if (p.m == 0)
+        return WOQ_OK;
+    if (pick_regime(args) == WOQ_REGIME_STREAM)
+        return launch_stream(p, stream);
+    if (p.pre_quant_scale)
+    {
+        // smoothing pass into the workspace, then the GEMM reads the smoothed activations
+        int const smoothed_dtype = p.w4a8 ? WOQ_FP8_E4M3 : p.out_dtype;
+        if (int rc = launch_prequant(
+                p.workspace, p.act, p.pre_quant_scale, p.m, p.k, p.out_dtype, smoothed_dtype, stream))
+            return rc;
+        p.act = p.workspace;
+        p.act_dtype = smoothed_dtype;
+        p.pre_quant_scale = nullptr;
+    }
+    return launch_gemm(p, stream);
+}
+
+extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,
+    int32_t k, int32_t in_dtype, int32_t out_dtype, void* stream)
+{
+    if (!out || !act || !per_channel_scale)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_apply_per_channel_scale: null pointer");
+    if (in_dtype != WOQ_FP16 && in_dtype != WOQ_BF16)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "input dtype must be fp16 or bf16");
+    if (out_dtype != in_dtype && out_dtype != WOQ_FP8_E4M3)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "output dtype must be the input dtype or fp8 e4m3");
+    if (m < 0 || k <= 0 || k % 8)
+        return fail(WOQ_ERR_BAD_SHAPE, "m >= 0 and k %% 8 == 0 required (got %d, %d)", m, k);
+    if (m == 0)
+        return WOQ_OK;
+    return launch_prequant(out, act, per_channel_scale, m, k, in_dtype, out_dtype, stream);
+}
+
+extern "C" int woq_dequantize(void* out, const void* weight, const void* scales, const void* zeros, int32_t k,
+    int32_t n, int32_t group_size, int32_t quant_type, int32_t dtype, void* stream)
+{
+    if (!out || !weight || !scales)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_dequantize: null pointer");
+    if (quant_type != WOQ_W8_A16 && quant_type != WOQ_W4_A16 && quant_type != WOQ_W4_AFP8)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown quant_type %d", quant_type);
+    if (dtype != WOQ_FP16 && dtype != WOQ_BF16 && dtype != WOQ_FP8_E4M3)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "dtype must be fp16, bf16 or fp8 e4m3");
+    if (k <= 0 || n <= 0 || n % kTileN || k % 32)
+        return fail(WOQ_ERR_BAD_SHAPE, "k %% 32 == 0 and n %% 16 == 0 required (got %d, %d)", k, n);
+    if (group_size != 0 && group_size != 64 && group_size != 128)
+        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0, 64 or 128 (got %d)", group_size);
+    if (group_size && k % group_size)
+        return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of group_size");
+    return launch_dequant(out, weight, scales, zeros, k, n, group_size, bits_of(quant_type), dtype, stream);
+}

@@ -1,0 +1,189 @@
+// Device-side building blocks shared by the gfx950 kernels of libwoq: vector types, 16-bit float
+// helpers, the int4/int8 -> MFMA-operand extractors and the 16x16x32 matrix-core wrappers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../woq_internal.h"
+
+namespace woq
+{
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+template <typename To, typename From>
+__device__ __forceinline__ To bit_cast(From const& v)
+{
+    static_assert(sizeof(To) == sizeof(From), "size mismatch");
+    return __builtin_bit_cast(To, v);
+}
+
+// ---- per-dtype traits ----------------------------------------------------------------------
+// MAGIC4: OR-ed onto an isolated nibble pair it yields two 16-bit floats of value BASE4 + u
+//         (bf16: 0x4300 = 128.0 with ulp 1; fp16: 0x6400 = 1024.0 with ulp 1).
+template <int DT>
+struct Elem;
+
+template <>
+struct Elem<WOQ_BF16>
+{
+    static constexpr uint32_t kMagic4 = 0x43004300u;
+    static constexpr float kBase4 = 128.f;
+    static constexpr uint32_t kOnes = 0x3F803F80u;
+    static constexpr float kBase8 = 0.f; // int8 goes through an exact float conversion: value u
+
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bit_cast<bf16x8>(a), bit_cast<bf16x8>(b), c, 0, 0, 0);
+    }
+
+    static __device__ __forceinline__ float lo(uint32_t pair)
+    {
+        return bit_cast<float>(pair << 16);
+    }
+
+    static __device__ __forceinline__ float hi(uint32_t pair)
+    {
+        return bit_cast<float>(pair & 0xFFFF0000u);
+    }
+
+    static __device__ __forceinline__ uint32_t pack(float a, float b)
+    {
+        bf16x2 r;
+        r[0] = (__bf16) a; // round to nearest even (v_cvt_pk_bf16_f32)
+        r[1] = (__bf16) b;
+        return bit_cast<uint32_t>(r);
+    }
+
+    static __device__ __forceinline__ float load(void const* p, size_t i)
+    {
+        return bit_cast<float>((uint32_t) static_cast<uint16_t const*>(p)[i] << 16);
+    }
+
+    static __device__ __forceinline__ uint16_t store(float v)
+    {
+        return bit_cast<uint16_t>((__bf16) v);
+    }
+
+    // elementwise product of two packed pairs, rounded once to the type
+    static __device__ __forceinline__ uint32_t mul2(uint32_t a, uint32_t b)
+    {
+        return pack(lo(a) * lo(b), hi(a) * hi(b));
+    }
+};
+
+template <>
+struct Elem<WOQ_FP16>
+{
+    static constexpr uint32_t kMagic4 = 0x64006400u;
+    static constexpr float kBase4 = 1024.f;
+    static constexpr uint32_t kOnes = 0x3C003C00u;
+    static constexpr float kBase8 = 1024.f; // int8 uses the byte-permute form 0x6400 | u
+
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<f16x8>(a), bit_cast<f16x8>(b), c, 0, 0, 0);
+    }
+
+    static __device__ __forceinline__ float lo(uint32_t pair)
+    {
+        return (float) bit_cast<f16x2>(pair)[0];
+    }
+
+    static __device__ __forceinline__ float hi(uint32_t pair)
+    {
+        return (float) bit_cast<f16x2>(pair)[1];
+    }
+
+    static __device__ __forceinline__ uint32_t pack(float a, float b)
+    {
+        f16x2 r;
+        r[0] = (_Float16) a;
+        r[1] = (_Float16) b;
+        return bit_cast<uint32_t>(r);
+    }
+
+    static __device__ __forceinline__ float load(void const* p, size_t i)
+    {
+        return (float) static_cast<_Float16 const*>(p)[i];
+    }
+
+    static __device__ __forceinline__ uint16_t store(float v)
+    {
+        return bit_cast<uint16_t>((_Float16) v);
+    }
+
+    static __device__ __forceinline__ uint32_t mul2(uint32_t a, uint32_t b)
+    {
+        return bit_cast<uint32_t>(bit_cast<f16x2>(a) * bit_cast<f16x2>(b));
+    }
+};
+
+// ---- packed weights -> MFMA B operand holding (BASE + u) exactly ---------------------------
+// int4: dword `w` holds elements e at nibble (e even ? e/2 : 4 + e/2); operand register i is
+// the pair (element 2i, element 2i+1).
+template <int DT>
+__device__ __forceinline__ u32x4 expand_int4(uint32_t w)
+{
+    constexpr uint32_t M = Elem<DT>::kMagic4;
+    u32x4 r;
+    r[0] = (w & 0x000F000Fu) | M;
+    r[1] = ((w >> 4) & 0x000F000Fu) | M;
+    r[2] = ((w >> 8) & 0x000F000Fu) | M;
+    r[3] = ((w >> 12) & 0x000F000Fu) | M;
+    return r;
+}
+
+// int8: two dwords hold elements 0..3 and 4..7 as bytes.
+template <int DT>
+__device__ __forceinline__ u32x4 expand_int8(uint32_t w0, uint32_t w1);
+
+template <>
+__device__ __forceinline__ u32x4 expand_int8<WOQ_BF16>(uint32_t w0, uint32_t w1)
+{
+    // 0..255 is exact in bf16 (8 significant bits); v_cvt_f32_ubyteN then a packed bf16 convert
+    u32x4 r;
+    r[0] = Elem<WOQ_BF16>::pack((float) (w0 & 0xFF), (float) ((w0 >> 8) & 0xFF));
+    r[1] = Elem<WOQ_BF16>::pack((float) ((w0 >> 16) & 0xFF), (float) (w0 >> 24));
+    r[2] = Elem<WOQ_BF16>::pack((float) (w1 & 0xFF), (float) ((w1 >> 8) & 0xFF));
+    r[3] = Elem<WOQ_BF16>::pack((float) ((w1 >> 16) & 0xFF), (float) (w1 >> 24));
+    return r;
+}
+
+template <>
+__device__ __forceinline__ u32x4 expand_int8<WOQ_FP16>(uint32_t w0, uint32_t w1)
+{
+    // byte permute builds [u, 0x64] pairs: fp16 1024 + u, exact for u <= 1023
+    constexpr uint32_t K = 0x64646464u;
+    u32x4 r;
+    r[0] = __builtin_amdgcn_perm(K, w0, 0x04010400u);
+    r[1] = __builtin_amdgcn_perm(K, w0, 0x04030402u);
+    r[2] = __builtin_amdgcn_perm(K, w1, 0x04010400u);
+    r[3] = __builtin_amdgcn_perm(K, w1, 0x04030402u);
+    return r;
+}
+
+// additive constant carried by the expanded operand: expanded value = q + kOffset
+template <int DT, int BITS>
+struct Offset
+{
+    static constexpr float value = BITS == 4 ? Elem<DT>::kBase4 + 8.f : Elem<DT>::kBase8 + 128.f;
+};
+
+// Workgroups are handed to the 8 XCDs round-robin.  Mapping block b to
+// strip (b % 8) * strips_per_xcd + b / 8 keeps neighbouring 16-column strips (which share
+// 128-byte lines of the scale / zero rows) on one XCD, hence in one L2.
+__device__ __forceinline__ int xcd_strip(int block, int strips_per_xcd)
+{
+    return (block & 7) * strips_per_xcd + (block >> 3);
+}
+
+} // namespace woq

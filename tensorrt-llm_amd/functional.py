@@ -1,0 +1,123 @@
+"""The two matmul ops of the reference's quantization front end, run eagerly on torch device
+tensors through libwoq's C ABI.
+
+Mirrors tensorrt_llm/quantization/functional.py:216-347 (`weight_only_quant_matmul`,
+`weight_only_groupwise_quant_matmul`): same argument order and meaning; the plugin path of the
+reference is the semantic (zeros AND pre-quant scale both apply).  Weights are the opaque
+tensors made by ops.preprocess_weights_for_mixed_gemm, moved to the GPU.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import lib, check, MatmulArgs
+
+_DTYPES = {"float16": torch.float16, "bfloat16": torch.bfloat16, torch.float16: torch.float16,
+           torch.bfloat16: torch.bfloat16}
+_WOQ_DT = {torch.float16: _lib.FP16, torch.bfloat16: _lib.BF16, torch.float8_e4m3fn: _lib.FP8_E4M3}
+
+# WeightOnlyQuantMatmulPlugin::WeightTypeId
+# (cpp/tensorrt_llm/plugins/weightOnlyQuantMatmulPlugin/weightOnlyQuantMatmulPlugin.h:38-42)
+INT8, INT4 = 1, 2
+# quant_algo flags (plugins/weightOnlyGroupwiseQuantMatmulPlugin/weightOnlyGroupwiseQuantMatmulPlugin.cpp:29-37)
+BIAS, ZERO, PRE_QUANT_SCALE, FP8_ALPHA, INT8_WEIGHT = 1, 2, 4, 8, 16
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream_handle(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and t.device.type != "cuda":
+            raise RuntimeError("weight-only matmul runs on the GPU only (got a %s tensor); "
+                               "there is no CPU path" % t.device.type)
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("tensors must be contiguous")
+
+
+def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int, k: int, group_size: int,
+                   quant_algo: int, alpha: float = 1.0, out_dtype=None, regime: int = 0, workspace=None,
+                   out=None) -> torch.Tensor:
+    """One call of woq_matmul.  `act` is [..., k]; returns [..., n]."""
+    _require_gpu(act, pre_quant_scale, weight, scales, zeros, bias, workspace, out)
+    out_dtype = out_dtype or (act.dtype if act.dtype != torch.float8_e4m3fn else scales.dtype)
+    if act.shape[-1] != k:
+        raise RuntimeError("activation has %d input features, weight expects %d" % (act.shape[-1], k))
+    m = act.numel() // k if k else 0
+    if out is None:
+        out = torch.empty(act.shape[:-1] + (n,), dtype=out_dtype, device=act.device)
+    need = lib.woq_workspace_bytes(m, n, k, quant_algo, _WOQ_DT[act.dtype])
+    if need and workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=act.device)
+    args = MatmulArgs(
+        act=_ptr(act), pre_quant_scale=_ptr(pre_quant_scale), weight=_ptr(weight), scales=_ptr(scales),
+        zeros=_ptr(zeros), bias=_ptr(bias), out=_ptr(out), alpha=float(alpha), m=m, n=n, k=k,
+        group_size=group_size, quant_algo=quant_algo, act_dtype=_WOQ_DT[act.dtype], out_dtype=_WOQ_DT[out_dtype],
+        regime=regime, workspace=_ptr(workspace),
+        workspace_bytes=0 if workspace is None else workspace.numel() * workspace.element_size())
+    check(lib.woq_matmul(ctypes.byref(args), _stream_handle(act.device)))
+    return out
+
+
+def weight_only_quant_matmul(input: torch.Tensor, weights: torch.Tensor, scales: torch.Tensor, weightTypeId: int,
+                             dtype="float16", transa: bool = False, transb: bool = False) -> torch.Tensor:
+    """Per-channel W8A16 / W4A16: input [.., K] x weights [K, N or N/2] (int8 storage, preprocessed),
+    scales [N].  Mirrors functional.py:216-256 + weightOnlyQuantMatmulPlugin.cpp:283-339."""
+    if transa or transb:
+        raise RuntimeError("transa/transb are not supported by the weight-only matmul plugin path")
+    if weightTypeId not in (INT8, INT4):
+        raise RuntimeError("weightTypeId must be 1 (int8) or 2 (int4)")
+    k = input.shape[-1]
+    n = weights.shape[-1] * (2 if weightTypeId == INT4 else 1)  # `real_n`
+    algo = INT8_WEIGHT if weightTypeId == INT8 else 0
+    return woq_matmul_raw(input, None, weights, scales, None, None, n=n, k=k, group_size=0, quant_algo=algo,
+                          out_dtype=_DTYPES[dtype])
+
+
+def weight_only_groupwise_quant_matmul(input: torch.Tensor, pre_quant_scale, weights: torch.Tensor,
+                                       scales: torch.Tensor, zeros, biases, alpha, quant_algo: int, group_size: int,
+                                       dtype="float16") -> torch.Tensor:
+    """Groupwise W4A16 / W8A16 / W4A8.  Mirrors functional.py:259-347 +
+    weightOnlyGroupwiseQuantMatmulPlugin.cpp:407-495.  `weights` is the preprocessed tensor; the
+    reference types it as the activation dtype ([K, N/4] halfs for int4, [K, N/2] for int8), a
+    plain int8 [K, N/2] / [K, N] tensor is accepted as well."""
+    out_dtype = _DTYPES[dtype]
+    k = input.shape[-1]
+    bits = 8 if quant_algo & INT8_WEIGHT else 4
+    n = weights.shape[-1] * weights.element_size() * 8 // bits
+    a = 1.0
+    if quant_algo & FP8_ALPHA:
+        a = float(alpha) if not hasattr(alpha, "raw_value") else float(alpha.raw_value[0])
+    return woq_matmul_raw(
+        input, pre_quant_scale if quant_algo & PRE_QUANT_SCALE else None, weights, scales,
+        zeros if quant_algo & ZERO else None, biases if quant_algo & BIAS else None,
+        n=n, k=k, group_size=group_size, quant_algo=quant_algo, alpha=a, out_dtype=out_dtype)
+
+
+def apply_per_channel_scale(act: torch.Tensor, per_channel_scale: torch.Tensor, out_dtype=None) -> torch.Tensor:
+    """kernels/preQuantScaleKernel.cu:42-149: act * scale, optionally cast to fp8 e4m3."""
+    _require_gpu(act, per_channel_scale)
+    out_dtype = out_dtype or act.dtype
+    k = act.shape[-1]
+    out = torch.empty(act.shape, dtype=out_dtype, device=act.device)
+    check(lib.woq_apply_per_channel_scale(_ptr(out), _ptr(act), _ptr(per_channel_scale), act.numel() // k, k,
+                                          _WOQ_DT[act.dtype], _WOQ_DT[out_dtype], _stream_handle(act.device)))
+    return out
+
+
+def dequantize_weights(weights: torch.Tensor, scales: torch.Tensor, zeros, *, k: int, n: int, group_size: int,
+                       quant_type: int, dtype: torch.dtype) -> torch.Tensor:
+    """W[k, n] = dtype(q * scale + zero) from preprocessed weights (woq_dequantize)."""
+    _require_gpu(weights, scales, zeros)
+    out = torch.empty((k, n), dtype=dtype, device=weights.device)
+    check(lib.woq_dequantize(_ptr(out), _ptr(weights), _ptr(scales), _ptr(zeros), k, n, group_size, quant_type,
+                             _WOQ_DT[dtype], _stream_handle(weights.device)))
+    return out

@@ -1,0 +1,116 @@
+"""Argument validation and regime selection of woq_matmul, exercised without a GPU through
+woq_matmul_check (same checks, no launch).  Error behaviour follows the reference's
+TLLM_CHECK / runtime_error sites (fpA_intB_gemm_template.h:129-196, kernelDispatcher.h:30-166)."""
+import ctypes
+
+import pytest
+
+
+def make_args(L, **kw):
+    a = L.MatmulArgs()
+    base = dict(act=0x1000, pre_quant_scale=None, weight=0x2000, scales=0x3000, zeros=None, bias=None, out=0x4000,
+                alpha=1.0, m=4, n=256, k=512, group_size=128, quant_algo=0, act_dtype=L.BF16, out_dtype=L.BF16,
+                regime=0, workspace=None, workspace_bytes=0)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(a, k, v)
+    return a
+
+
+def status(pkg, **kw):
+    L = pkg._lib
+    return L.lib.woq_matmul_check(ctypes.byref(make_args(L, **kw))), (L.lib.woq_last_error() or b"").decode()
+
+
+def test_valid_combinations(pkg):
+    L = pkg._lib
+    assert status(pkg)[0] == 0
+    assert status(pkg, zeros=0x5000, quant_algo=L.ALGO_ZERO)[0] == 0
+    assert status(pkg, bias=0x5000, quant_algo=L.ALGO_BIAS, group_size=64)[0] == 0
+    assert status(pkg, pre_quant_scale=0x5000, quant_algo=L.ALGO_PRE_QUANT_SCALE)[0] == 0
+    assert status(pkg, group_size=0, quant_algo=L.ALGO_INT8_WEIGHT, act_dtype=L.FP16, out_dtype=L.FP16)[0] == 0
+    assert status(pkg, m=0)[0] == 0                                     # m == 0 is a no-op, not an error
+    assert status(pkg, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, alpha=0.5)[0] == 0
+
+
+@pytest.mark.parametrize("kw,code,text", [
+    (dict(scales=None), -1, "scales"),
+    (dict(act=None), -1, "NULL"),
+    (dict(group_size=32), -3, "group_size"),
+    (dict(k=96), -2, "multiple of 64"),
+    (dict(k=576, group_size=128), -2, "group_size"),
+    (dict(n=250), -2, "multiple of 16"),
+    (dict(zeros=0x5000), -1, "ZERO"),
+    (dict(quant_algo=2), -1, "ZERO"),
+    (dict(quant_algo=1), -1, "BIAS"),
+    (dict(quant_algo=4), -1, "PRE_QUANT_SCALE"),
+    (dict(group_size=0, zeros=0x5000, quant_algo=2), -1, "scale only"),
+    (dict(out_dtype=2), -1, "out_dtype"),
+    (dict(act_dtype=0), -1, "activation dtype"),
+    (dict(quant_algo=8 | 16, act_dtype=2), -3, "INT4"),
+    (dict(quant_algo=8, act_dtype=2, group_size=64), -3, "128"),
+    (dict(quant_algo=8, act_dtype=2, k=192, group_size=64), -3, "128"),
+    (dict(quant_algo=8), -1, "PRE_QUANT_SCALE"),
+    (dict(act_dtype=2), -1, "FP8_ALPHA"),
+    (dict(regime=1, m=129), -3, "unsupported m"),
+    (dict(regime=7), -1, "regime"),
+    (dict(m=-1), -2, "non-negative"),
+    (dict(quant_algo=64), -1, "quant_algo"),
+])
+def test_rejections(pkg, kw, code, text):
+    rc, msg = status(pkg, **kw)
+    assert rc == code, msg
+    assert text.lower() in msg.lower()
+
+
+def test_null_args(pkg):
+    assert pkg._lib.lib.woq_matmul_check(None) == -1
+
+
+def test_workspace_rule(pkg):
+    L = pkg._lib
+    lib = L.lib
+    algo = L.ALGO_PRE_QUANT_SCALE
+    assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2
+    assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == 0
+    # GEMM regime with smoothing needs the workspace; the streaming regime fuses it
+    rc, msg = status(pkg, m=512, pre_quant_scale=0x5000, quant_algo=algo)
+    assert rc == -4 and "workspace" in msg
+    assert status(pkg, m=512, pre_quant_scale=0x5000, quant_algo=algo, workspace=0x9000,
+                  workspace_bytes=512 * 512 * 2)[0] == 0
+    assert status(pkg, m=8, pre_quant_scale=0x5000, quant_algo=algo)[0] == 0
+
+
+def test_regime_table(pkg):
+    L = pkg._lib
+    sel = L.lib.woq_select_regime
+    for m in (1, 2, 4, 15, 16, 64, 128):
+        assert sel(m, 4096, 4096, 0) == L.REGIME_STREAM
+    for m in (129, 256, 4096, 8192):
+        assert sel(m, 4096, 4096, 0) == L.REGIME_GEMM
+    assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
+
+
+def test_python_wrappers_refuse_cpu_tensors(pkg):
+    import torch
+    a = torch.zeros(1, 128, dtype=torch.bfloat16)
+    w = torch.zeros(128, 8, dtype=torch.int8)
+    s = torch.zeros(1, 16, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        pkg.functional.weight_only_groupwise_quant_matmul(a, None, w, s, None, None, None, 0, 128, "bfloat16")
+
+
+def test_last_error_is_per_thread(pkg):
+    import threading
+    L = pkg._lib
+    status(pkg, group_size=32)
+    seen = {}
+
+    def other():
+        seen["msg"] = (L.lib.woq_last_error() or b"").decode()
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen["msg"] == ""
+    assert "group_size" in (L.lib.woq_last_error() or b"").decode()

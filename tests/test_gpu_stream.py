@@ -1,0 +1,130 @@
+"""GPU parity of the weight-streaming kernel (decode GEMV / skinny M) against the CPU oracle,
+through the C ABI.  Tolerance: max|out - ref| / max|ref| <= 1e-2 against the float64-accumulated
+dequantize-then-matmul reference (the bar the benchmark definition states); observed errors are
+~1e-3 (one rounding of the output to fp16/bf16)."""
+import numpy as np
+import pytest
+import torch
+
+from _util import random_problem, reference, run_product, preprocess, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+STREAM = 1
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("group", [0, 64, 128])
+@pytest.mark.parametrize("M", [1, 3, 16])
+def test_stream_basic(pkg, oracle, dev, dtype, bits, group, M):
+    p = random_problem(oracle, M, 512, 128, bits, group, dtype, seed=M + bits + group)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("zero,bias,pqs", [(1, 0, 0), (0, 1, 0), (0, 0, 1), (1, 1, 0), (1, 0, 1), (0, 1, 1), (1, 1, 1)])
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 64), (8, 128)])
+def test_stream_optional_inputs(pkg, oracle, dev, dtype, zero, bias, pqs, bits, group):
+    """The eight (act_scale, zero, bias) variants of the reference dispatcher (kernelDispatcher.h:101-143)."""
+    p = random_problem(oracle, 5, 1024, 256, bits, group, dtype, zero, bias, pqs, seed=zero * 4 + bias * 2 + pqs)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 7, 8, 15, 16, 17, 32, 33, 64, 100, 128])
+def test_stream_m_sweep(pkg, oracle, dev, M):
+    p = random_problem(oracle, M, 1024, 1024, 4, 128, "bf16", zero=True, seed=M)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("K,N", [(64, 1024), (128, 16), (192, 48), (320, 2048), (1024, 1040), (4096, 4096)])
+def test_stream_ragged_shapes(pkg, oracle, dev, K, N):
+    """K that is not a multiple of the 128-row weight tile (padded tail), N not a multiple of 128
+    (partly empty XCD chunks), and the reference's own small test shapes."""
+    for bits, group in [(4, 64), (8, 64), (4, 0)]:
+        p = random_problem(oracle, 3, K, N, bits, group, "bf16", zero=group != 0, seed=K + N)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        assert err < TOL, (bits, group, err)
+
+
+def test_stream_identity_recovers_weight(pkg, oracle, dev):
+    """The reference's conversion test (test_weight_only_quant_matmul.py:147-164): an identity
+    activation pulls the dequantized weight out of the kernel.  Here the result must equal the
+    oracle's dequantize to within one output rounding of q*s+z computed in float32."""
+    K, N = 128, 64
+    p = random_problem(oracle, K, K, N, 4, 128, "bf16", zero=True, seed=3)
+    p["act"] = np.eye(K, dtype=np.float32)
+    out = run_product(pkg, oracle, dev, p, STREAM)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")
+    assert oracle.max_rel_err(out, w) < 4e-3
+
+
+def test_stream_all_ones_and_zeros(pkg, oracle, dev):
+    p = random_problem(oracle, 2, 512, 128, 4, 128, "bf16", zero=True, seed=8)
+    p["act"] = np.stack([np.ones(512, np.float32), np.zeros(512, np.float32)])
+    out = run_product(pkg, oracle, dev, p, STREAM)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16").astype(np.float64)
+    assert oracle.max_rel_err(out[0], w.sum(0)) < TOL
+    assert (out[1] == 0).all()
+
+
+def test_stream_zero_none_equals_zero_zero_and_is_deterministic(pkg, oracle, dev):
+    p = random_problem(oracle, 4, 1024, 256, 4, 128, "bf16", seed=11)
+    a = run_product(pkg, oracle, dev, p, STREAM)
+    p2 = dict(p, zeros=np.zeros_like(p["scales"]))
+    b = run_product(pkg, oracle, dev, p2, STREAM)
+    assert (a == b).all()
+    assert (a == run_product(pkg, oracle, dev, p, STREAM)).all()       # fixed reduction order
+
+
+def test_stream_large_activations_offset_cancellation(pkg, oracle, dev):
+    """The kernel removes the (BASE + 8) operand offset with activation row sums; activations
+    with a large common mean stress that cancellation."""
+    for dtype in ("bf16", "fp16"):
+        for bits, group in [(4, 128), (8, 0)]:
+            p = random_problem(oracle, 2, 4096, 64, bits, group, dtype, seed=5)
+            p["act"] = oracle.round_to(p["act"] + 3.0, dtype)
+            err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+            assert err < TOL, (dtype, bits, err)
+
+
+def test_m_zero_is_a_noop(pkg, dev):
+    F = pkg.functional
+    act = torch.zeros((0, 128), dtype=torch.bfloat16, device=dev)
+    w = torch.zeros((128, 8), dtype=torch.int8, device=dev)
+    s = torch.ones((1, 16), dtype=torch.bfloat16, device=dev)
+    out = F.weight_only_groupwise_quant_matmul(act, None, w, s, None, None, None, 0, 128, "bfloat16")
+    assert out.shape == (0, 16)
+
+
+def test_functional_and_plugin_mirrors(pkg, oracle, dev):
+    """Per-channel op + both plugin wrappers give the same numbers as the raw call."""
+    F, P = pkg.functional, pkg.plugin
+    p = random_problem(oracle, 4, 512, 256, 8, 0, "fp16", seed=21)
+    w = preprocess(pkg, oracle, p["q"], 8, torch.float16).to(dev)
+    act, s = to_dev(p["act"], "fp16", dev), to_dev(p["scales"], "fp16", dev)
+    out = F.weight_only_quant_matmul(act, w, s, F.INT8, "float16")
+    assert oracle.max_rel_err(out.float().cpu().numpy(), reference(oracle, p)) < TOL
+    out2 = torch.empty_like(out)
+    assert P.WeightOnlyQuantMatmulPlugin(torch.float16, F.INT8).enqueue([act, w, s], [out2]) == 0
+    assert (out2 == out).all()
+    # int4: the plugin receives N/2 packed columns and doubles them
+    p4 = random_problem(oracle, 4, 512, 256, 4, 0, "fp16", seed=22)
+    w4 = preprocess(pkg, oracle, p4["q"], 4, torch.float16).to(dev)
+    out4 = F.weight_only_quant_matmul(to_dev(p4["act"], "fp16", dev), w4, to_dev(p4["scales"], "fp16", dev), F.INT4)
+    assert out4.shape == (4, 256)
+    assert oracle.max_rel_err(out4.float().cpu().numpy(), reference(oracle, p4)) < TOL
+    # groupwise plugin: inputs in plugin order, weight typed as the activation dtype ([K, N/4] halfs)
+    pg = random_problem(oracle, 3, 512, 256, 4, 128, "bf16", zero=True, bias=True, pqs=True, seed=23)
+    wg = preprocess(pkg, oracle, pg["q"], 4).to(dev).view(torch.bfloat16)
+    assert wg.shape == (512, 64)
+    plug = P.WeightOnlyGroupwiseQuantMatmulPlugin(torch.bfloat16, F.BIAS | F.ZERO | F.PRE_QUANT_SCALE, 128)
+    outg = torch.empty((3, 256), dtype=torch.bfloat16, device=dev)
+    ins = [to_dev(pg[k], "bf16", dev) for k in ("act", "pqs")] + [wg] + [to_dev(pg[k], "bf16", dev) for k in
+                                                                         ("scales", "zeros", "bias")]
+    assert plug.enqueue(ins, [outg]) == 0
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err(outg.float().cpu().numpy(), reference(oracle, pg)) < TOL
