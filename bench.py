@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-only quantized matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep]
+
+Workload (the configuration the headline metric is quoted on): W4A16, group 128, bf16
+activations/scales/zeros, M = 1 — the four linear layers of one Llama-3-8B decoder layer
+(qkv K=4096 N=6144, o K=4096 N=4096, gate_up K=4096 N=28672, down K=14336 N=4096).  One "step" is
+one pass over those four matmuls.  Steps rotate over several distinct copies of the weights
+(more than the 256 MB last-level cache), so weights always come from HBM.  The timed K steps are
+captured in one HIP graph and replayed, so launches are back to back with no Python in between.
+
+`value` = algorithmic bytes of a step / time of a step (inputs resident in HBM).  `roofline`
+describes the dominant kernel (the gate_up GEMV), timed on its own with HIP events on the launch
+stream.  `cpu_baseline` times the reference's CPU path (torch dequantize + float32 matmul) on the
+host cores for the same step.  `gemm` (extra field) reports the prefill regime at M = 4096.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import torch
+
+from __graft_entry__ import import_package
+
+METRIC = "W4A16 g128 GEMM: HBM GB/s at M=1, TFLOP/s at M=4096 (Llama-3-8B shapes)"
+SHAPES_8B = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+GROUP = 128
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
+
+
+def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
+    """Every operand once: packed weights + scales(+zeros) + activations + output."""
+    sz = (k // group) * n * 2 * n_sz if group else n * 2
+    return k * n * bits // 8 + sz + m * k * act_bytes + m * n * 2
+
+
+def make_layer(pkg, dev, k, n, seed):
+    """Synthetic tensors of the benchmark configuration: W ~ N(0, 0.02) quantized to uint4 with
+    group 128 along K (asymmetric min/max), bf16 scales, bf16 zeros = (8 - zp) * scale."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    w = torch.randn((k, n), generator=g, device=dev, dtype=torch.float32) * 0.02
+    wg = w.view(k // GROUP, GROUP, n)
+    mx, mn = wg.amax(1), wg.amin(1)
+    scale = ((mx - mn).clamp_min(1e-8) / 15.0).to(torch.bfloat16)
+    sf = scale.float()
+    zp = torch.round(-mn / sf).clamp(0, 15)
+    qu = (torch.round(wg / sf[:, None, :]) + zp[:, None, :]).clamp(0, 15)
+    q = (qu - 8).to(torch.int8).view(k, n)
+    zeros = ((8.0 - zp) * sf).to(torch.bfloat16)
+    packed = ((q[:, 0::2] & 0xF) | (q[:, 1::2] << 4)).to(torch.int8).cpu().contiguous()
+    wq = pkg.ops.preprocess_weights_for_mixed_gemm(packed, torch.quint4x2, torch.bfloat16).to(dev)
+    return dict(k=k, n=n, q=q, weight=wq, scales=scale.contiguous(), zeros=zeros.contiguous())
+
+
+def rotated_copies(layer, copies):
+    """Distinct device buffers holding the same tiles in rolled order: different addresses for
+    the caches, still valid weights (any byte pattern is)."""
+    out = [layer]
+    tiles = layer["weight"].view(-1, 1024)
+    for r in range(1, copies):
+        c = dict(layer)
+        c["weight"] = tiles.roll(977 * r + 1, 0).contiguous().view_as(layer["weight"])
+        c["scales"] = layer["scales"].roll(r, 0).contiguous()
+        c["zeros"] = layer["zeros"].roll(r, 0).contiguous()
+        out.append(c)
+    return out
+
+
+def launch(pkg, act, layer, out, regime=0):
+    F = pkg.functional
+    F.woq_matmul_raw(act, None, layer["weight"], layer["scales"], layer["zeros"], None, n=layer["n"], k=layer["k"],
+                     group_size=GROUP, quant_algo=F.ZERO, out_dtype=torch.bfloat16, out=out, regime=regime)
+
+
+def time_graph(fn_body, launches):
+    """Captures fn_body() (which issues `launches` kernels) in a HIP graph, replays it once
+    untimed, then times one replay with HIP events on the replay stream and with the host clock."""
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            fn_body()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    return (t1 - t0), e0.elapsed_time(e1) * 1e-3, launches
+
+
+def bench_decode(pkg, dev, steps, warmup, m=1):
+    per_step_bytes = sum(algorithmic_bytes(m, k, n) for _, k, n in SHAPES_8B)
+    weight_bytes = sum(k * n // 2 for _, k, n in SHAPES_8B)
+    copies = max(2, -(-3 * CACHE_BYTES // weight_bytes))  # >= 3x the cache
+    layers = [rotated_copies(make_layer(pkg, dev, k, n, 2000 + i), copies) for i, (_, k, n) in enumerate(SHAPES_8B)]
+    g = torch.Generator(device=dev).manual_seed(2999)
+    acts = {k: torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16) for k in (4096, 14336)}
+    outs = [torch.empty((m, n), dtype=torch.bfloat16, device=dev) for _, _, n in SHAPES_8B]
+
+    def step(s):
+        for i, (_, k, _) in enumerate(SHAPES_8B):
+            launch(pkg, acts[k], layers[i][s % copies], outs[i])
+
+    for s in range(warmup):
+        step(s)
+    torch.cuda.synchronize()
+    host_s, ev_s, _ = time_graph(lambda: [step(s) for s in range(steps)], steps * len(SHAPES_8B))
+
+    # dominant kernel on its own: the gate_up GEMV
+    gi = 2
+    _, gk, gn = SHAPES_8B[gi]
+    reps = max(steps, 50)
+    _, dom_s, dom_launches = time_graph(
+        lambda: [launch(pkg, acts[gk], layers[gi][r % copies], outs[gi]) for r in range(reps)], reps)
+    dom_bytes = algorithmic_bytes(m, gk, gn)
+    dom_dur = dom_s / dom_launches
+    per_shape = {}
+    for i, (name, k, n) in enumerate(SHAPES_8B):
+        _, s_s, s_l = time_graph(lambda: [launch(pkg, acts[k], layers[i][r % copies], outs[i]) for r in range(reps)],
+                                 reps)
+        per_shape[name] = dict(us=round(s_s / s_l * 1e6, 3), gbs=round(algorithmic_bytes(m, k, n) / (s_s / s_l) / 1e9, 1))
+    return dict(host_s=host_s, ev_s=ev_s, per_step_bytes=per_step_bytes, copies=copies, dom_dur=dom_dur,
+                dom_bytes=dom_bytes, per_shape=per_shape, layers=layers, acts=acts)
+
+
+def bench_cpu_baseline(layers, acts, m=1, budget_s=15.0):
+    """The reference's CPU path (tensorrt_llm/quantization/functional.py:269-290 semantics):
+    dequantize with torch, then a float32 matmul, on the host cores."""
+    from __graft_entry__ import import_oracle
+    o = import_oracle()
+    host = []
+    for i, (_, k, n) in enumerate(SHAPES_8B):
+        l = layers[i][0]
+        host.append((acts[k].float().cpu(), l["q"].cpu(), l["scales"].float().cpu(), l["zeros"].float().cpu()))
+    per_step_bytes = sum(algorithmic_bytes(m, k, n) for _, k, n in SHAPES_8B)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+        t0 = time.perf_counter()
+        for a, q, s, z in host:
+            o.torch_cpu_dequant_matmul(a, q, s, z, GROUP)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return dict(value=round(per_step_bytes / med / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                sample="%d passes over the same 4-matmul step (torch dequant + fp32 matmul), median %.1f ms"
+                       % (len(times), med * 1e3))
+
+
+def bench_gemm(pkg, dev, m=4096, reps=5):
+    """Prefill regime, largest shape (gate_up): TFLOP/s at M = 4096."""
+    try:
+        name, k, n = SHAPES_8B[2]
+        layer = make_layer(pkg, dev, k, n, 3000)
+        g = torch.Generator(device=dev).manual_seed(3999)
+        act = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        launch(pkg, act, layer, out)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            launch(pkg, act, layer, out)
+        e1.record()
+        torch.cuda.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / reps
+        tf = 2.0 * m * n * k / sec / 1e12
+        return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
+                    frac_of_bf16_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
+    except Exception as e:  # the decode line is still valid without the prefill extra
+        return dict(error=str(e)[:200])
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "
+                 "communication inside it, see DESIGN.md")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the matmul has no CPU path")
+    pkg = import_package()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    r = bench_decode(pkg, dev, args.steps, args.warmup)
+    sec_per_step = r["host_s"] / args.steps
+    value = r["per_step_bytes"] / sec_per_step / 1e9
+    achieved = r["dom_bytes"] / r["dom_dur"] / 1e9
+    line = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B decoder-layer linears (qkv, o_proj, gate_up, down), W4A16 g128 "
+                               "bf16 scales+zeros, decode GEMV M=1; %d rotating weight copies" % r["copies"],
+                   "m": 1, "group_size": GROUP, "weight_bits": 4},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "stream_kernel<bf16,int4,g128,MT=1> on gate_up K=4096 N=28672",
+                     "bytes_per_launch": r["dom_bytes"], "us_per_launch": round(r["dom_dur"] * 1e6, 3)},
+        "per_shape": r["per_shape"],
+        "event_ms_per_step": round(r["ev_s"] / args.steps * 1e3, 5),
+    }
+    if not args.no_gemm:
+        line["gemm"] = bench_gemm(pkg, dev)
+    if not args.no_cpu:
+        line["cpu_baseline"] = bench_cpu_baseline(r["layers"], r["acts"])
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -75,7 +75,8 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
         return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 (per-channel), 64 or 128 (got %d)", a->group_size);
     if (w4a8 && a->group_size != 128)
         return fail(WOQ_ERR_UNSUPPORTED, "W4A8 supports group_size 128 only (got %d)", a->group_size);
-    if (!a->act || !a->weight || !a->out)
+    // m == 0 is a no-op (weightOnlyQuantMatmulPlugin.cpp:303): empty tensors may carry null pointers
+    if (a->m > 0 && (!a->act || !a->weight || !a->out))
         return fail(WOQ_ERR_INVALID_ARGUMENT, "act, weight and out must not be NULL");
     if (!a->scales)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "Weight scales must always be set to a non-null value.");
