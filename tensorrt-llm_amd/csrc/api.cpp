@@ -5,6 +5,7 @@
 // of the small-M dispatcher (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernelDispatcher.h:30-166)
 // and of the runner's argument checks
 // (cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:129-196).
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -27,6 +28,38 @@ int launch_stream(MatmulProblem const& p, void* stream)
     if (p.out_dtype == WOQ_BF16)
         return p.bits == 4 ? launch_stream_BF16_4(p, stream) : launch_stream_BF16_8(p, stream);
     return p.bits == 4 ? launch_stream_FP16_4(p, stream) : launch_stream_FP16_8(p, stream);
+}
+
+// Launch shape of the streaming kernel.  More strips per wavefront amortise the activation
+// fragments and the row-sum MFMA; more wavefronts per workgroup split K further so that small
+// problems still fill 256 CUs.
+struct StreamShape
+{
+    int ns, waves, pf;
+};
+
+StreamShape pick_stream_shape(int mt, int strips, int k_tiles)
+{
+    if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
+    {
+        StreamShape sh{0, 0, 0};
+        if (std::sscanf(e, "%d,%d,%d", &sh.ns, &sh.waves, &sh.pf) == 3)
+            return sh;
+    }
+    (void) k_tiles;
+    if (mt == 1)
+    {
+        if (strips >= 1024)
+            return {4, 4, 2};
+        if (strips >= 384)
+            return {2, 8, 2};
+        return {1, 8, 4};
+    }
+    if (mt == 2)
+        return {strips >= 1024 ? 2 : 1, 8, 2};
+    if (mt == 4)
+        return {strips >= 1024 ? 2 : 1, 8, 1};
+    return {1, 8, 1};
 }
 
 namespace

@@ -73,6 +73,11 @@ struct Elem<WOQ_BF16>
         return bit_cast<uint16_t>((__bf16) v);
     }
 
+    static __device__ __forceinline__ float from_bits(uint16_t b)
+    {
+        return bit_cast<float>((uint32_t) b << 16);
+    }
+
     // elementwise product of two packed pairs, rounded once to the type
     static __device__ __forceinline__ uint32_t mul2(uint32_t a, uint32_t b)
     {
@@ -119,6 +124,11 @@ struct Elem<WOQ_FP16>
     static __device__ __forceinline__ uint16_t store(float v)
     {
         return bit_cast<uint16_t>((_Float16) v);
+    }
+
+    static __device__ __forceinline__ float from_bits(uint16_t b)
+    {
+        return (float) bit_cast<_Float16>(b);
     }
 
     static __device__ __forceinline__ uint32_t mul2(uint32_t a, uint32_t b)
@@ -177,6 +187,23 @@ struct Offset
 {
     static constexpr float value = BITS == 4 ? Elem<DT>::kBase4 + 8.f : Elem<DT>::kBase8 + 128.f;
 };
+
+// ---- buffer (descriptor-based) loads: out-of-range accesses return 0 ---------------------------
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(void const* base, uint32_t bytes)
+{
+    // raw buffer (stride 0): num_records counts bytes; 0x00020000 = 32-bit untyped data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int) bytes, 0x00020000);
+}
+
+__device__ __forceinline__ u32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) byte_offset, 0, 0);
+}
+
+__device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int) byte_offset, 0, 0);
+}
 
 // Workgroups are handed to the 8 XCDs round-robin.  Mapping block b to
 // strip (b % 8) * strips_per_xcd + b / 8 keeps neighbouring 16-column strips (which share

@@ -34,173 +34,308 @@ struct StreamParams
     int m, n, k;
     int k_tiles;        // ceil(k / TILE_K)
     int strips;         // n / 16
-    int strips_per_xcd; // ceil(strips / 8)
+    int groups;         // ceil(strips / NS): column groups, one workgroup each
+    int groups_per_xcd; // ceil(groups / 8)
 };
 
-template <int DT, int BITS, int GROUP, bool PQS, int MT, int WAVES>
+// Everything one wavefront needs for one tile row (NS tiles side by side), fetched together so
+// that no load sits in the dependent chain of the compute that follows.
+template <int NS, int SLABS, int SEGS, int MT, bool PQS>
+struct StreamStage
+{
+    u32x4 w[NS];               // packed weights: this lane's 16 bytes of each tile
+    u32x4 a[SLABS][MT];        // activation fragments (A operands), zero outside m / k
+    u32x4 sm[PQS ? SLABS : 1]; // pre-quant scale fragments
+    uint16_t s[NS][SEGS];      // raw scale / zero of each segment of each tile (this lane's column)
+    uint16_t z[NS][SEGS];
+};
+
+// NS    strips (16 columns each) one wavefront covers; they share the activation fragments and
+//       the row-sum MFMA
+// WAVES wavefronts per workgroup; they split K (tile row kt goes to wave kt % WAVES)
+// PF    tile rows in flight per wavefront
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF>
 __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 {
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
+    constexpr int SLABS = TK / 32;
     constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows that share one scale inside a tile
     constexpr int SEG_SLABS = SEG / 32;
     constexpr int SEGS = TK / SEG;
-    constexpr int PF = 4; // weight tiles in flight per wavefront
     constexpr float OFF = Offset<DT, BITS>::value;
+    using Stage = StreamStage<NS, SLABS, SEGS, MT, PQS>;
 
-    int const strip = xcd_strip(blockIdx.x, p.strips_per_xcd);
-    if (strip >= p.strips)
+    int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
+    if (group >= p.groups)
         return; // whole workgroup leaves together
 
     int const lane = threadIdx.x & 63;
-    int const wave = threadIdx.x >> 6;
+    // the wavefront index is wave-uniform: keep it (and everything derived from it) in SGPRs so
+    // that the K loop is straight scalar control flow
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const c = lane & 15;  // column inside the strip (B operand) / row inside the M-tile (A operand)
     int const kg = lane >> 4; // which 8 of a slab's 32 rows this lane holds
-    int const col = strip * 16 + c;
     int const K = p.k;
     int const KT = p.k_tiles;
+    int const strip0 = group * NS;
 
     u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
     f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
 
-    f32x4 acc_out[MT], acc_p[MT], acc_s[MT];
+    f32x4 acc_out[NS][MT], acc_p[NS][MT], acc_s[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-        acc_out[mt] = acc_p[mt] = acc_s[mt] = zero4;
-
-    u32x4 const* wbase = static_cast<u32x4 const*>(p.weight) + (size_t) strip * KT * 64 + lane;
-    uint16_t const* act16 = static_cast<uint16_t const*>(p.act);
-
-    u32x4 buf[PF];
-#pragma unroll
-    for (int i = 0; i < PF; ++i)
     {
-        int kt = wave + i * WAVES;
-        buf[i] = kt < KT ? wbase[(size_t) kt * 64] : u32x4{0, 0, 0, 0};
+        acc_s[mt] = zero4;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            acc_out[s][mt] = acc_p[s][mt] = zero4;
     }
 
-    for (int kt0 = wave; kt0 < KT; kt0 += WAVES * PF)
-    {
-#pragma unroll
-        for (int i = 0; i < PF; ++i)
-        {
-            int const kt = kt0 + i * WAVES;
-            if (kt >= KT)
-                break; // wave-uniform
-            u32x4 const w = buf[i];
-            int const ktn = kt + PF * WAVES;
-            if (ktn < KT)
-                buf[i] = wbase[(size_t) ktn * 64];
+    // Buffer descriptors: an access past num_records returns 0, which is exactly what rows >= m,
+    // the padded tail of K and the scale rows of that tail must contribute - no branches needed.
+    constexpr uint32_t kOob = 0x7FFFFFF0u;
+    auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
+    auto const pqs_rsrc = make_rsrc(PQS ? p.pqs : p.act, (uint32_t) K * 2u);
+    uint32_t const sz_bytes = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
+    auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
 
+    // weights too go through a descriptor: a prefetch past the last tile row is given an
+    // out-of-range offset and costs no memory traffic, so the K loop needs no conditional loads
+    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+    // strips past the end of N (last group only) are clamped for loads and skipped at the store
+    int strip_of[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+
+    uint32_t wlane[NS]; // byte offset of this lane's 16 bytes in tile row 0 of each strip
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+
+    auto fetch = [&](Stage& st, int kt)
+    {
+        uint32_t const tile_off = kt < KT ? (uint32_t) kt * 1024u : 0x80000000u; // scalar select
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+        {
+            int const kk = kt * TK + j * 32 + kg * 8; // this lane's 8 rows of the slab
+            bool const k_ok = kk < K;
+            if constexpr (PQS)
+                st.sm[j] = buffer_load_x4(pqs_rsrc, (uint32_t) kk * 2u);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+            {
+                uint32_t const row = mt * 16 + c;
+                st.a[j][mt] = buffer_load_x4(act_rsrc, k_ok ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob);
+            }
+        }
+        if constexpr (GROUP != 0)
+        {
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
             {
-                int const krow0 = kt * TK + seg * SEG; // first row of this segment
-                if (krow0 >= K)
-                    break; // padded tail of K: wave-uniform
+                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
 #pragma unroll
-                for (int js = 0; js < SEG_SLABS; ++js)
+                for (int s = 0; s < NS; ++s)
                 {
-                    int const j = seg * SEG_SLABS + js;
+                    uint32_t const off = (grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u;
+                    st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
+                    if constexpr (ZERO)
+                        st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
+                }
+            }
+        }
+    };
+
+    auto compute = [&](Stage const& st)
+    {
+#pragma unroll
+        for (int seg = 0; seg < SEGS; ++seg)
+        {
+#pragma unroll
+            for (int js = 0; js < SEG_SLABS; ++js)
+            {
+                int const j = seg * SEG_SLABS + js;
+                u32x4 a[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                {
+                    a[mt] = st.a[j][mt];
+                    if constexpr (PQS)
+                    {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            a[mt][r] = E::mul2(a[mt][r], st.sm[j][r]);
+                    }
+                    acc_s[mt] = E::mma(a[mt], ones, acc_s[mt]);
+                }
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
                     u32x4 b;
                     if constexpr (BITS == 4)
-                        b = expand_int4<DT>(w[j]);
+                        b = expand_int4<DT>(st.w[s][j]);
                     else
-                        b = expand_int8<DT>(w[2 * j], w[2 * j + 1]);
-                    int const kk = kt * TK + j * 32 + kg * 8; // this lane's 8 rows of the slab
-                    bool const k_ok = kk < K;
-                    u32x4 sm = {0, 0, 0, 0};
-                    if constexpr (PQS)
-                        if (k_ok)
-                            sm = *reinterpret_cast<u32x4 const*>(static_cast<uint16_t const*>(p.pqs) + kk);
+                        b = expand_int8<DT>(st.w[s][2 * j], st.w[s][2 * j + 1]);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
-                    {
-                        int const row = mt * 16 + c;
-                        u32x4 a = {0, 0, 0, 0};
-                        if (k_ok && row < p.m)
-                            a = *reinterpret_cast<u32x4 const*>(act16 + (size_t) row * K + kk);
-                        if constexpr (PQS)
-                        {
-#pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                a[r] = E::mul2(a[r], sm[r]);
-                        }
-                        acc_p[mt] = E::mma(a, b, acc_p[mt]);
-                        acc_s[mt] = E::mma(a, ones, acc_s[mt]);
-                    }
+                        acc_p[s][mt] = E::mma(a[mt], b, acc_p[s][mt]);
                 }
-                if constexpr (GROUP != 0)
+            }
+            if constexpr (GROUP != 0)
+            {
+                // a segment past the end of K carries zero activations, scale 0 and zero 0
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
                 {
-                    size_t const gi = (size_t) (krow0 / GROUP) * p.n + col;
-                    float const s = E::load(p.scales, gi);
-                    float const z = p.zeros ? E::load(p.zeros, gi) : 0.f;
-                    float const cc = z - OFF * s;
+                    float const sc = E::from_bits(st.s[s][seg]);
+                    float const cc = (ZERO ? E::from_bits(st.z[s][seg]) : 0.f) - OFF * sc;
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                     {
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            acc_out[mt][r] += s * acc_p[mt][r] + cc * acc_s[mt][r];
-                        acc_p[mt] = zero4;
-                        acc_s[mt] = zero4;
+                            acc_out[s][mt][r] += sc * acc_p[s][mt][r] + cc * acc_s[mt][r];
+                        acc_p[s][mt] = zero4;
                     }
                 }
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc_s[mt] = zero4;
             }
+        }
+    };
+
+    // tile rows of this wavefront: kt = wave + it * WAVES, it = 0 .. n_my-1 (all scalar).
+    // Every load tolerates kt >= KT (returns zeros), so prologue and loop are unconditional and
+    // the compiler's wait-count tracking stays exact: compute(st[i]) waits only for its own
+    // stage while the PF-1 younger stages stay in flight.  The scheduling barriers keep the
+    // compiler from sinking the prefetch below the compute (it would, to save registers).
+    int const n_my = (KT - wave + WAVES - 1) / WAVES;
+    Stage st[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i)
+        fetch(st[i], wave + i * WAVES);
+    __builtin_amdgcn_sched_barrier(0);
+
+    for (int it = 0; it < n_my; it += PF)
+    {
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+        {
+            if (it + i < n_my)
+                compute(st[i]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(st[i], wave + (it + i + PF) * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
     if constexpr (GROUP == 0)
     {
-        float const s = E::load(p.scales, col);
-        float const z = p.zeros ? E::load(p.zeros, col) : 0.f;
-        float const cc = z - OFF * s;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            int const col = strip_of[s] * 16 + c;
+            float const sc = E::load(p.scales, col);
+            float const cc = (ZERO ? E::load(p.zeros, col) : 0.f) - OFF * sc;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc_out[s][mt][r] = sc * acc_p[s][mt][r] + cc * acc_s[mt][r];
+        }
+    }
+
+    // ---- cross-wavefront reduction (fixed order) and epilogue -------------------------------
+    constexpr int SLOTS = NS * MT * 4;
+    __shared__ float red[WAVES][SLOTS][64];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                acc_out[mt][r] = s * acc_p[mt][r] + cc * acc_s[mt][r];
-    }
-
-    // ---- cross-wavefront reduction (fixed order) and epilogue -------------------------------
-    __shared__ float red[WAVES][MT * 4][64];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            red[wave][mt * 4 + r][lane] = acc_out[mt][r];
+                if (mt * 16 + kg * 4 + r < p.m)
+                    red[wave][(s * MT + mt) * 4 + r][lane] = acc_out[s][mt][r];
     __syncthreads();
 
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
-    for (int e = threadIdx.x; e < MT * 4 * 64; e += WAVES * 64)
+    for (int e = threadIdx.x; e < SLOTS * 64; e += WAVES * 64)
     {
         int const slot = e >> 6, ln = e & 63;
+        int const s = slot / (MT * 4), mt = (slot >> 2) % MT, r = slot & 3;
+        int const row = mt * 16 + (ln >> 4) * 4 + r;
+        if (row >= p.m || strip0 + s >= p.strips)
+            continue;
         float sum = 0.f;
 #pragma unroll
         for (int w2 = 0; w2 < WAVES; ++w2)
             sum += red[w2][slot][ln];
-        int const row = (slot >> 2) * 16 + (ln >> 4) * 4 + (slot & 3);
-        int const ocol = strip * 16 + (ln & 15);
-        if (row < p.m)
-        {
-            float v = p.alpha * sum;
-            if (p.bias)
-                v += E::load(p.bias, ocol);
-            out16[(size_t) row * p.n + ocol] = E::store(v);
-        }
+        int const ocol = (strip0 + s) * 16 + (ln & 15);
+        float v = p.alpha * sum;
+        if (p.bias)
+            v += E::load(p.bias, ocol);
+        out16[(size_t) row * p.n + ocol] = E::store(v);
     }
 }
 
-template <int DT, int BITS, int GROUP, bool PQS, int MT>
-int launch_stream_variant(StreamParams const& sp, hipStream_t stream)
+// launch shape: NS strips per wavefront, WAVES wavefronts per workgroup, PF tile rows in flight
+struct StreamShape
 {
-    constexpr int WAVES = MT >= 8 ? 4 : 8;
-    dim3 grid(sp.strips_per_xcd * 8), block(WAVES * 64);
-    hipLaunchKernelGGL((stream_kernel<DT, BITS, GROUP, PQS, MT, WAVES>), grid, block, 0, stream, sp);
+    int ns, waves, pf;
+};
+
+// WOQ_STREAM_SHAPE="ns,waves,pf" overrides the heuristic (for tuning sweeps)
+StreamShape pick_stream_shape(int mt, int strips, int k_tiles);
+
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF>
+int launch_stream_variant(StreamParams sp, hipStream_t stream)
+{
+    sp.groups = (sp.strips + NS - 1) / NS;
+    sp.groups_per_xcd = (sp.groups + 7) / 8;
+    dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    hipLaunchKernelGGL((stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF>), grid, block, 0, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "stream kernel launch failed: %s", hipGetErrorString(err));
     return WOQ_OK;
+}
+
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
+int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
+{
+    StreamShape const sh = pick_stream_shape(mt, sp.strips, sp.k_tiles);
+#define WOQ_SHAPE(MT_, NS_, WAVES_, PF_)                                                                               \
+    if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_)                                               \
+        return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, MT_, NS_, WAVES_, PF_>(sp, s);
+    // decode (M <= 16)
+    WOQ_SHAPE(1, 1, 8, 4)
+    WOQ_SHAPE(1, 1, 4, 4)
+    WOQ_SHAPE(1, 2, 8, 2)
+    WOQ_SHAPE(1, 2, 8, 3)
+    WOQ_SHAPE(1, 2, 4, 4)
+    WOQ_SHAPE(1, 4, 4, 2)
+    WOQ_SHAPE(1, 4, 4, 3)
+    WOQ_SHAPE(1, 4, 8, 2)
+    WOQ_SHAPE(1, 4, 8, 3)
+    // skinny M
+    WOQ_SHAPE(2, 2, 8, 2)
+    WOQ_SHAPE(2, 1, 8, 2)
+    WOQ_SHAPE(4, 1, 8, 1)
+    WOQ_SHAPE(4, 2, 8, 1)
+    WOQ_SHAPE(8, 1, 4, 1)
+    WOQ_SHAPE(8, 1, 8, 1)
+#undef WOQ_SHAPE
+    return fail(WOQ_ERR_UNSUPPORTED, "stream shape mt=%d ns=%d waves=%d pf=%d is not instantiated", mt, sh.ns,
+        sh.waves, sh.pf);
 }
 
 template <int DT, int BITS>
@@ -221,37 +356,29 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.k = p.k;
     sp.k_tiles = (p.k + TK - 1) / TK;
     sp.strips = p.n / kTileN;
-    sp.strips_per_xcd = (sp.strips + 7) / 8;
+    sp.groups = sp.groups_per_xcd = 0;
     auto s = static_cast<hipStream_t>(stream);
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;
+    bool const zero = p.zeros != nullptr;
 
-#define WOQ_STREAM_MT(G, Q)                                                                                            \
-    switch (mt)                                                                                                        \
-    {                                                                                                                  \
-    case 1: return launch_stream_variant<DT, BITS, G, Q, 1>(sp, s);                                                    \
-    case 2: return launch_stream_variant<DT, BITS, G, Q, 2>(sp, s);                                                    \
-    case 4: return launch_stream_variant<DT, BITS, G, Q, 4>(sp, s);                                                    \
-    default: return launch_stream_variant<DT, BITS, G, Q, 8>(sp, s);                                                   \
-    }
 #define WOQ_STREAM_PQS(G)                                                                                              \
     if (pqs)                                                                                                           \
-    {                                                                                                                  \
-        WOQ_STREAM_MT(G, true)                                                                                         \
-    }                                                                                                                  \
-    else                                                                                                               \
-    {                                                                                                                  \
-        WOQ_STREAM_MT(G, false)                                                                                        \
-    }
+        return zero ? launch_stream_shaped<DT, BITS, G, true, true>(sp, mt, s)                                         \
+                    : launch_stream_shaped<DT, BITS, G, true, false>(sp, mt, s);                                       \
+    return zero ? launch_stream_shaped<DT, BITS, G, false, true>(sp, mt, s)                                            \
+                : launch_stream_shaped<DT, BITS, G, false, false>(sp, mt, s);
     switch (p.group_size)
     {
-    case 0: WOQ_STREAM_PQS(0)
+    case 0:
+        if (pqs)
+            return launch_stream_shaped<DT, BITS, 0, true, false>(sp, mt, s);
+        return launch_stream_shaped<DT, BITS, 0, false, false>(sp, mt, s);
     case 64: WOQ_STREAM_PQS(64)
     case 128: WOQ_STREAM_PQS(128)
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 #undef WOQ_STREAM_PQS
-#undef WOQ_STREAM_MT
 }
 
 } // namespace woq
