@@ -35,31 +35,41 @@ int launch_stream(MatmulProblem const& p, void* stream)
 // problems still fill 256 CUs.
 struct StreamShape
 {
-    int ns, waves, pf;
+    int ns, waves, pf, lds;
 };
 
-StreamShape pick_stream_shape(int mt, int strips, int k_tiles)
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k)
 {
     if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
     {
-        StreamShape sh{0, 0, 0};
-        if (std::sscanf(e, "%d,%d,%d", &sh.ns, &sh.waves, &sh.pf) == 3)
+        StreamShape sh{0, 0, 0, 0};
+        if (std::sscanf(e, "%d,%d,%d,%d", &sh.ns, &sh.waves, &sh.pf, &sh.lds) == 4)
             return sh;
     }
     (void) k_tiles;
     if (mt == 1)
     {
+        int const rows = m < 16 ? m : 16;
+        size_t const act_lds = (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
+        if (act_lds <= 96 * 1024)
+        {
+            if (strips >= 1024)
+                return {4, 8, 2, 1};
+            if (strips >= 384)
+                return {2, 8, 4, 1};
+            return {1, 8, 4, 1};
+        }
         if (strips >= 1024)
-            return {4, 4, 2};
+            return {4, 4, 2, 0};
         if (strips >= 384)
-            return {2, 8, 2};
-        return {1, 8, 4};
+            return {2, 8, 2, 0};
+        return {1, 8, 4, 0};
     }
     if (mt == 2)
-        return {strips >= 1024 ? 2 : 1, 8, 2};
+        return {strips >= 1024 ? 2 : 1, 8, 2, 0};
     if (mt == 4)
-        return {strips >= 1024 ? 2 : 1, 8, 1};
-    return {1, 8, 1};
+        return {strips >= 1024 ? 2 : 1, 8, 1, 0};
+    return {1, 8, 1, 0};
 }
 
 namespace

@@ -140,15 +140,36 @@ struct Elem<WOQ_FP16>
 // ---- packed weights -> MFMA B operand holding (BASE + u) exactly ---------------------------
 // int4: dword `w` holds elements e at nibble (e even ? e/2 : 4 + e/2); operand register i is
 // the pair (element 2i, element 2i+1).
-template <int DT>
-__device__ __forceinline__ u32x4 expand_int4(uint32_t w)
+// The nibble mask and the exponent pattern as values the compiler cannot see through.  With
+// literal constants it emits v_and + v_or (a VOP3 encoding cannot carry 32-bit literals on gfx9);
+// with the mask in an SGPR and the pattern in a VGPR it selects the fused v_and_or_b32 itself,
+// and - unlike hand-written asm in the data path - still sees every VALU->MFMA dependency it has
+// to schedule around.
+struct NibbleConsts
 {
-    constexpr uint32_t M = Elem<DT>::kMagic4;
+    uint32_t mask;  // 0x000F000F, in an SGPR
+    uint32_t magic; // Elem<DT>::kMagic4, in a VGPR
+};
+
+template <int DT>
+__device__ __forceinline__ NibbleConsts nibble_consts()
+{
+    NibbleConsts c;
+    c.mask = 0x000F000Fu;
+    c.magic = Elem<DT>::kMagic4;
+    asm volatile("" : "+s"(c.mask));
+    asm volatile("" : "+v"(c.magic));
+    return c;
+}
+
+template <int DT>
+__device__ __forceinline__ u32x4 expand_int4(uint32_t w, NibbleConsts const& c)
+{
     u32x4 r;
-    r[0] = (w & 0x000F000Fu) | M;
-    r[1] = ((w >> 4) & 0x000F000Fu) | M;
-    r[2] = ((w >> 8) & 0x000F000Fu) | M;
-    r[3] = ((w >> 12) & 0x000F000Fu) | M;
+    r[0] = (w & c.mask) | c.magic;
+    r[1] = ((w >> 4) & c.mask) | c.magic;
+    r[2] = ((w >> 8) & c.mask) | c.magic;
+    r[3] = ((w >> 12) & c.mask) | c.magic;
     return r;
 }
 

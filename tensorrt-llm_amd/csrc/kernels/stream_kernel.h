@@ -13,8 +13,14 @@
 //     BASE + 2^(bits-1) offset and carry the additive zeros:
 //         out += s * P + (z - OFFSET * s) * S,   P = sum a * (q + OFFSET),   S = sum a;
 //   * the wavefronts of a workgroup split K and are reduced through LDS in a fixed order
-//     (results are bit-reproducible from run to run).
+//     (results are bit-reproducible from run to run);
+//   * for decode-sized activations (M rows x K fit in LDS) the workgroup stages the - already
+//     smoothed - activations in LDS once and reads A fragments from there, so a pipeline stage
+//     holds nothing but packed weights and their scales: few registers per byte in flight,
+//     hence many wavefronts and many bytes in flight per CU, which is what HBM needs.
 #pragma once
+
+#include <type_traits>
 
 #include "device_common.h"
 
@@ -40,13 +46,13 @@ struct StreamParams
 
 // Everything one wavefront needs for one tile row (NS tiles side by side), fetched together so
 // that no load sits in the dependent chain of the compute that follows.
-template <int NS, int SLABS, int SEGS, int MT, bool PQS>
+template <int NS, int SLABS, int SEGS, int MT, bool PQS, bool ALDS>
 struct StreamStage
 {
-    u32x4 w[NS];               // packed weights: this lane's 16 bytes of each tile
-    u32x4 a[SLABS][MT];        // activation fragments (A operands), zero outside m / k
-    u32x4 sm[PQS ? SLABS : 1]; // pre-quant scale fragments
-    uint16_t s[NS][SEGS];      // raw scale / zero of each segment of each tile (this lane's column)
+    u32x4 w[NS];                          // packed weights: this lane's 16 bytes of each tile
+    u32x4 a[ALDS ? 1 : SLABS][ALDS ? 1 : MT]; // activation fragments (unused when they live in LDS)
+    u32x4 sm[(PQS && !ALDS) ? SLABS : 1]; // pre-quant scale fragments
+    uint16_t s[NS][SEGS];                 // raw scale / zero of each segment of each tile (this lane's column)
     uint16_t z[NS][SEGS];
 };
 
@@ -54,9 +60,11 @@ struct StreamStage
 //       the row-sum MFMA
 // WAVES wavefronts per workgroup; they split K (tile row kt goes to wave kt % WAVES)
 // PF    tile rows in flight per wavefront
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF>
+// ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
 __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 {
+    static_assert(!ALDS || MT == 1, "LDS-staged activations are for M <= 16");
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
@@ -64,7 +72,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
     constexpr int SEG_SLABS = SEG / 32;
     constexpr int SEGS = TK / SEG;
     constexpr float OFF = Offset<DT, BITS>::value;
-    using Stage = StreamStage<NS, SLABS, SEGS, MT, PQS>;
+    using Stage = StreamStage<NS, SLABS, SEGS, MT, PQS, ALDS>;
+    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (KT*TK*2 + 16) bytes
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
     if (group >= p.groups)
@@ -81,6 +90,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
     int const strip0 = group * NS;
 
     u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
+    NibbleConsts const nib = nibble_consts<DT>();
     f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
 
     f32x4 acc_out[NS][MT], acc_p[NS][MT], acc_s[MT];
@@ -98,23 +108,29 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
     constexpr uint32_t kOob = 0x7FFFFFF0u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
     auto const pqs_rsrc = make_rsrc(PQS ? p.pqs : p.act, (uint32_t) K * 2u);
-    uint32_t const sz_bytes = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes
+        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
-
     // weights too go through a descriptor: a prefetch past the last tile row is given an
     // out-of-range offset and costs no memory traffic, so the K loop needs no conditional loads
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+
     // strips past the end of N (last group only) are clamped for loads and skipped at the store
     int strip_of[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s)
-        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
-
     uint32_t wlane[NS]; // byte offset of this lane's 16 bytes in tile row 0 of each strip
 #pragma unroll
     for (int s = 0; s < NS; ++s)
+    {
+        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
         wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+    }
+
+    // LDS-staged activations: row r of the M-tile at byte r * lds_row; rows >= m read row m-1
+    // (their products land in output rows that are never stored)
+    uint32_t const lds_row = (uint32_t) KT * TK * 2u + 16u; // +16: rows start in different banks
+    int const a_row = c < p.m ? c : p.m - 1;
+    char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
 
     auto fetch = [&](Stage& st, int kt)
     {
@@ -122,18 +138,22 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 #pragma unroll
         for (int s = 0; s < NS; ++s)
             st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
-#pragma unroll
-        for (int j = 0; j < SLABS; ++j)
+        if constexpr (!ALDS)
         {
-            int const kk = kt * TK + j * 32 + kg * 8; // this lane's 8 rows of the slab
-            bool const k_ok = kk < K;
-            if constexpr (PQS)
-                st.sm[j] = buffer_load_x4(pqs_rsrc, (uint32_t) kk * 2u);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int j = 0; j < SLABS; ++j)
             {
-                uint32_t const row = mt * 16 + c;
-                st.a[j][mt] = buffer_load_x4(act_rsrc, k_ok ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob);
+                int const kk = kt * TK + j * 32 + kg * 8; // this lane's 8 rows of the slab
+                bool const k_ok = kk < K;
+                if constexpr (PQS)
+                    st.sm[j] = buffer_load_x4(pqs_rsrc, (uint32_t) kk * 2u);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                {
+                    uint32_t const row = mt * 16 + c;
+                    st.a[j][mt]
+                        = buffer_load_x4(act_rsrc, k_ok ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob);
+                }
             }
         }
         if constexpr (GROUP != 0)
@@ -154,7 +174,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
         }
     };
 
-    auto compute = [&](Stage const& st)
+    auto compute = [&](Stage const& st, int kt)
     {
 #pragma unroll
         for (int seg = 0; seg < SEGS; ++seg)
@@ -167,12 +187,17 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                 {
-                    a[mt] = st.a[j][mt];
-                    if constexpr (PQS)
+                    if constexpr (ALDS)
+                        a[mt] = *reinterpret_cast<u32x4 const*>(a_lds + (uint32_t) (kt * TK + j * 32) * 2u);
+                    else
                     {
+                        a[mt] = st.a[j][mt];
+                        if constexpr (PQS)
+                        {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            a[mt][r] = E::mul2(a[mt][r], st.sm[j][r]);
+                            for (int r = 0; r < 4; ++r)
+                                a[mt][r] = E::mul2(a[mt][r], st.sm[j][r]);
+                        }
                     }
                     acc_s[mt] = E::mma(a[mt], ones, acc_s[mt]);
                 }
@@ -181,7 +206,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
                 {
                     u32x4 b;
                     if constexpr (BITS == 4)
-                        b = expand_int4<DT>(st.w[s][j]);
+                        b = expand_int4<DT>(st.w[s][j], nib);
                     else
                         b = expand_int8<DT>(st.w[s][2 * j], st.w[s][2 * j + 1]);
 #pragma unroll
@@ -191,21 +216,32 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
             }
             if constexpr (GROUP != 0)
             {
-                // a segment past the end of K carries zero activations, scale 0 and zero 0
-#pragma unroll
-                for (int s = 0; s < NS; ++s)
+                // a segment past the end of K carries zero activations, scale 0 and zero 0.
+                // Lane (kg, c) register r is output row kg*4 + r: with a single row (decode,
+                // m == 1) only r == 0 is ever stored, so the other three are not scaled.
+                auto scale_rows = [&](auto rows_tag)
                 {
-                    float const sc = E::from_bits(st.s[s][seg]);
-                    float const cc = (ZERO ? E::from_bits(st.z[s][seg]) : 0.f) - OFF * sc;
+                    constexpr int ROWS = decltype(rows_tag)::value;
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
+                    for (int s = 0; s < NS; ++s)
                     {
+                        float const sc = E::from_bits(st.s[s][seg]);
+                        float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits(st.z[s][seg]) : 0.f);
 #pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            acc_out[s][mt][r] += sc * acc_p[s][mt][r] + cc * acc_s[mt][r];
-                        acc_p[s][mt] = zero4;
+                        for (int mt = 0; mt < MT; ++mt)
+                        {
+#pragma unroll
+                            for (int r = 0; r < ROWS; ++r)
+                                acc_out[s][mt][r] = __builtin_fmaf(
+                                    sc, acc_p[s][mt][r], __builtin_fmaf(cc, acc_s[mt][r], acc_out[s][mt][r]));
+                            acc_p[s][mt] = zero4;
+                        }
                     }
-                }
+                };
+                if (MT == 1 && p.m == 1)
+                    scale_rows(std::integral_constant<int, 1>{});
+                else
+                    scale_rows(std::integral_constant<int, 4>{});
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc_s[mt] = zero4;
@@ -225,13 +261,37 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
         fetch(st[i], wave + i * WAVES);
     __builtin_amdgcn_sched_barrier(0);
 
+    if constexpr (ALDS)
+    {
+        // Stage the activations (smoothed if a pre-quant scale is given) behind the first weight
+        // prefetches: both are in flight together, the activations come from L2 and land first.
+        int const rows = p.m < 16 ? p.m : 16;
+        int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
+        for (int idx = threadIdx.x; idx < rows * chunks_per_row; idx += WAVES * 64)
+        {
+            int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
+            bool const k_ok = ch * 8 < K;
+            u32x4 v = buffer_load_x4(act_rsrc, k_ok ? ((uint32_t) row * (uint32_t) K + (uint32_t) ch * 8u) * 2u : kOob);
+            if constexpr (PQS)
+            {
+                u32x4 const sm = buffer_load_x4(pqs_rsrc, (uint32_t) ch * 16u);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    v[r] = E::mul2(v[r], sm[r]);
+            }
+            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + (uint32_t) row * lds_row + (uint32_t) ch * 16u) = v;
+        }
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
     for (int it = 0; it < n_my; it += PF)
     {
 #pragma unroll
         for (int i = 0; i < PF; ++i)
         {
             if (it + i < n_my)
-                compute(st[i]);
+                compute(st[i], wave + (it + i) * WAVES);
             __builtin_amdgcn_sched_barrier(0);
             fetch(st[i], wave + (it + i + PF) * WAVES);
             __builtin_amdgcn_sched_barrier(0);
@@ -250,7 +310,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    acc_out[s][mt][r] = sc * acc_p[s][mt][r] + cc * acc_s[mt][r];
+                    acc_out[s][mt][r] = __builtin_fmaf(sc, acc_p[s][mt][r], cc * acc_s[mt][r]);
         }
     }
 
@@ -287,22 +347,50 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
     }
 }
 
-// launch shape: NS strips per wavefront, WAVES wavefronts per workgroup, PF tile rows in flight
+// launch shape: NS strips per wavefront, WAVES wavefronts per workgroup, PF tile rows in flight,
+// lds != 0: activations staged in LDS
 struct StreamShape
 {
-    int ns, waves, pf;
+    int ns, waves, pf, lds;
 };
 
-// WOQ_STREAM_SHAPE="ns,waves,pf" overrides the heuristic (for tuning sweeps)
-StreamShape pick_stream_shape(int mt, int strips, int k_tiles);
+// bytes of LDS the staged activations of an m x k problem take (tile_k = 128 int4 / 64 int8)
+inline size_t stream_act_lds_bytes(int m, int k, int tile_k)
+{
+    int const rows = m < 16 ? m : 16;
+    return (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
+}
 
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF>
+constexpr size_t kStreamMaxActLds = 96 * 1024;
+
+// WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k);
+
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
 int launch_stream_variant(StreamParams sp, hipStream_t stream)
 {
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    auto kernel = stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>;
+    size_t lds = 0;
+    if constexpr (ALDS)
+    {
+        lds = stream_act_lds_bytes(sp.m, sp.k, TK);
+        if (lds > kStreamMaxActLds)
+            return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
+        static bool raised = false; // benign race: the attribute call is idempotent
+        if (lds > 32 * 1024 && !raised)
+        {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kStreamMaxActLds);
+            if (e != hipSuccess)
+                return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
-    hipLaunchKernelGGL((stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF>), grid, block, 0, stream, sp);
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "stream kernel launch failed: %s", hipGetErrorString(err));
@@ -312,30 +400,34 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 {
-    StreamShape const sh = pick_stream_shape(mt, sp.strips, sp.k_tiles);
-#define WOQ_SHAPE(MT_, NS_, WAVES_, PF_)                                                                               \
-    if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_)                                               \
-        return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, MT_, NS_, WAVES_, PF_>(sp, s);
-    // decode (M <= 16)
-    WOQ_SHAPE(1, 1, 8, 4)
-    WOQ_SHAPE(1, 1, 4, 4)
-    WOQ_SHAPE(1, 2, 8, 2)
-    WOQ_SHAPE(1, 2, 8, 3)
-    WOQ_SHAPE(1, 2, 4, 4)
-    WOQ_SHAPE(1, 4, 4, 2)
-    WOQ_SHAPE(1, 4, 4, 3)
-    WOQ_SHAPE(1, 4, 8, 2)
-    WOQ_SHAPE(1, 4, 8, 3)
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    StreamShape const sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK);
+#define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
+    if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                      \
+        return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, MT_, NS_, WAVES_, PF_, LDS_>(sp, s);
+    // decode (M <= 16), activations in LDS
+    WOQ_SHAPE(1, 1, 8, 4, true)
+    WOQ_SHAPE(1, 1, 8, 6, true)
+    WOQ_SHAPE(1, 1, 16, 4, true)
+    WOQ_SHAPE(1, 2, 8, 4, true)
+    WOQ_SHAPE(1, 2, 4, 4, true)
+    WOQ_SHAPE(1, 4, 4, 2, true)
+    WOQ_SHAPE(1, 4, 4, 4, true)
+    WOQ_SHAPE(1, 4, 8, 2, true)
+    // decode, activations in registers (M x K too large for LDS)
+    WOQ_SHAPE(1, 1, 8, 4, false)
+    WOQ_SHAPE(1, 2, 8, 2, false)
+    WOQ_SHAPE(1, 4, 4, 2, false)
     // skinny M
-    WOQ_SHAPE(2, 2, 8, 2)
-    WOQ_SHAPE(2, 1, 8, 2)
-    WOQ_SHAPE(4, 1, 8, 1)
-    WOQ_SHAPE(4, 2, 8, 1)
-    WOQ_SHAPE(8, 1, 4, 1)
-    WOQ_SHAPE(8, 1, 8, 1)
+    WOQ_SHAPE(2, 2, 8, 2, false)
+    WOQ_SHAPE(2, 1, 8, 2, false)
+    WOQ_SHAPE(4, 1, 8, 1, false)
+    WOQ_SHAPE(4, 2, 8, 1, false)
+    WOQ_SHAPE(8, 1, 4, 1, false)
+    WOQ_SHAPE(8, 1, 8, 1, false)
 #undef WOQ_SHAPE
-    return fail(WOQ_ERR_UNSUPPORTED, "stream shape mt=%d ns=%d waves=%d pf=%d is not instantiated", mt, sh.ns,
-        sh.waves, sh.pf);
+    return fail(WOQ_ERR_UNSUPPORTED, "stream shape mt=%d ns=%d waves=%d pf=%d lds=%d is not instantiated", mt, sh.ns,
+        sh.waves, sh.pf, sh.lds);
 }
 
 template <int DT, int BITS>

@@ -128,3 +128,35 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
     assert plug.enqueue(ins, [outg]) == 0
     torch.cuda.synchronize()
     assert oracle.max_rel_err(outg.float().cpu().numpy(), reference(oracle, pg)) < TOL
+
+
+STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,1", "4,4,4,1", "4,8,2,1",
+                 "1,8,4,0", "2,8,2,0", "4,4,2,0"]
+
+
+@pytest.mark.parametrize("shape", STREAM_SHAPES)
+@pytest.mark.parametrize("M", [1, 5])
+def test_stream_every_launch_shape(pkg, oracle, dev, monkeypatch, shape, M):
+    """Every instantiated (strips per wavefront, wavefronts, prefetch depth, LDS staging) variant
+    of the decode kernel, forced through WOQ_STREAM_SHAPE, against the oracle - including a strip
+    count that is not a multiple of the strips per wavefront."""
+    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    for bits, group, N in [(4, 128, 272), (8, 64, 64), (4, 0, 48)]:
+        p = random_problem(oracle, M, 1280, N, bits, group, "bf16", zero=group != 0, pqs=True, seed=M + N)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        assert err < TOL, (shape, bits, group, err)
+
+
+@pytest.mark.parametrize("N", [6144, 16384])
+def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
+    """Wide outputs take the multi-strip launch shapes of the heuristic."""
+    p = random_problem(oracle, 1, 512, N, 4, 128, "bf16", zero=True, seed=N)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+def test_stream_activations_too_large_for_lds(pkg, oracle, dev):
+    """M x K beyond the LDS staging area falls back to register-held activation fragments."""
+    p = random_problem(oracle, 16, 4096, 64, 4, 128, "bf16", zero=True, seed=77)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
