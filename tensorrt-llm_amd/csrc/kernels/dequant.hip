@@ -28,13 +28,13 @@ __global__ void __launch_bounds__(256) dequant_kernel(void* out, void const* wei
         size_t const gi = group_size ? (size_t) (k0 / group_size) * n + col : (size_t) col;
         float const s = Elem<SDT>::load(scales, gi);
         float const z = zeros ? Elem<SDT>::load(zeros, gi) : 0.f;
-        int q[8];
-        if constexpr (BITS == 4)
-            unpack_int4_signed(w[j], q);
-        else
-            unpack_int8_signed(w[2 * j], w[2 * j + 1], q);
         if constexpr (DT == WOQ_FP8_E4M3)
         {
+            int q[8];
+            if constexpr (BITS == 4)
+                unpack_int4_signed(w[j], q);
+            else
+                unpack_int8_signed(w[2 * j], w[2 * j + 1], q);
             u32x2 const r = dequant8_fp8(q, s, z);
             uint8_t* o = static_cast<uint8_t*>(out);
 #pragma unroll
@@ -43,7 +43,12 @@ __global__ void __launch_bounds__(256) dequant_kernel(void* out, void const* wei
         }
         else
         {
-            u32x4 const r = dequant8<DT>(q, s, z);
+            // the very functions the GEMM main loop calls
+            u32x4 r;
+            if constexpr (BITS == 4)
+                r = dequant_int4_dword<DT>(w[j], s, z);
+            else
+                r = dequant_int8_dwords<DT>(w[2 * j], w[2 * j + 1], s, z);
             uint16_t* o = static_cast<uint16_t*>(out);
 #pragma unroll
             for (int e = 0; e < 8; ++e)

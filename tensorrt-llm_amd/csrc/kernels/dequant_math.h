@@ -72,6 +72,24 @@ __device__ __forceinline__ u32x4 dequant8<WOQ_FP16>(int const (&q)[8], float s, 
     return r;
 }
 
+// one int4 dword (8 elements of one MFMA slab) -> the slab's B operand
+template <int DT>
+__device__ __forceinline__ u32x4 dequant_int4_dword(uint32_t w, float s, float z)
+{
+    int q[8];
+    unpack_int4_signed(w, q);
+    return dequant8<DT>(q, s, z);
+}
+
+// two int8 dwords (8 elements of one MFMA slab) -> the slab's B operand
+template <int DT>
+__device__ __forceinline__ u32x4 dequant_int8_dwords(uint32_t w0, uint32_t w1, float s, float z)
+{
+    int q[8];
+    unpack_int8_signed(w0, w1, q);
+    return dequant8<DT>(q, s, z);
+}
+
 // 8 dequantized values -> 8 e4m3 bytes (2 dwords), element order preserved
 __device__ __forceinline__ u32x2 dequant8_fp8(int const (&q)[8], float s, float z)
 {

@@ -1,0 +1,10 @@
+// Instantiates the prefill GEMM kernel for BF16 activations and int4 weights.
+#include "gemm_kernel.h"
+
+namespace woq
+{
+int launch_gemm_BF16_4(MatmulProblem const& p, void* stream)
+{
+    return launch_gemm_typed<WOQ_BF16, 4>(p, stream);
+}
+} // namespace woq

@@ -1,0 +1,10 @@
+// Instantiates the prefill GEMM kernel for FP16 activations and int8 weights.
+#include "gemm_kernel.h"
+
+namespace woq
+{
+int launch_gemm_FP16_8(MatmulProblem const& p, void* stream)
+{
+    return launch_gemm_typed<WOQ_FP16, 8>(p, stream);
+}
+} // namespace woq

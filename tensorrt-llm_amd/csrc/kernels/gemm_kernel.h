@@ -1,0 +1,290 @@
+// Prefill GEMM: fp16/bf16 activations x int4/int8 weights on the 16x16x32 matrix core.
+//
+// Counterpart of the reference's CUTLASS mixed-input GEMM
+// (cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:57-230 and the
+// dequantizing main loop in cutlass_extensions/.../gemm/threadblock/dq_mma_multistage_finegrained.h)
+// in semantics only: out = T(alpha * A x dequant(W) + bias), float32 accumulation, weights
+// dequantized to the activation type by the single definition in dequant_math.h.
+//
+// Design for CDNA4 (one workgroup of 4 wavefronts per CU, 256 x 256 output tile):
+//   * the 4 wavefronts sit side by side along N: each owns 256 rows x 64 columns (16 x 4 MFMA
+//     tiles, 256 float32 accumulator registers per lane).  Weight columns are therefore disjoint
+//     between wavefronts: every packed weight is loaded from memory once per workgroup, straight
+//     into the registers of the lane that feeds it to the matrix core (the tile layout of
+//     host_prep.cpp IS the B-operand register layout), and is dequantized exactly once.  Weights
+//     never touch LDS.
+//   * the activation tile (256 rows x one weight tile row of K) is shared by the 4 wavefronts: it
+//     is DMA-ed global -> LDS (buffer_load ... lds, no staging registers) in MFMA-fragment order,
+//     so every A-fragment read is one conflict-free ds_read_b128 of consecutive lanes.  Two LDS
+//     buffers alternate: the DMA for step k+1 runs under the MFMAs of step k.
+//   * rows >= M and the zero-filled tail of K come back as zeros from the buffer descriptor.
+#pragma once
+
+#include "dequant_math.h"
+
+namespace woq
+{
+
+struct GemmParams
+{
+    void const* act;
+    void const* weight;
+    void const* scales;
+    void const* zeros;
+    void const* bias;
+    void* out;
+    float alpha;
+    int m, n, k;
+    int k_tiles; // ceil(k / TILE_K)
+    int strips;  // n / 16
+    int tiles_m, tiles_n;
+};
+
+constexpr int kGemmBM = 256;
+constexpr int kGemmBN = 256;
+constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
+
+template <int DT, int BITS, int GROUP, bool ZERO>
+__global__ void __launch_bounds__(256) gemm_kernel(GemmParams p)
+{
+    using E = Elem<DT>;
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    constexpr int SLABS = TK / 32;
+    constexpr int RT = kGemmBM / 16;                             // 16 row tiles per wavefront
+    constexpr int NS = 4;                                        // strips (16 columns) per wavefront
+    constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
+    constexpr int SEGS = TK / SEG;
+    constexpr int SEG_SLABS = SEG / 32;
+    constexpr int A_BYTES = kGemmBM * TK * 2;
+
+    __shared__ u32x4 a_buf0[A_BYTES / 16];
+    __shared__ u32x4 a_buf1[A_BYTES / 16];
+
+    // ---- which output tile: XCD-contiguous chunks, m fastest inside groups of kGemmGroupM ------
+    int const total = p.tiles_m * p.tiles_n;
+    int const per_xcd = (total + 7) / 8;
+    int const t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int) (blockIdx.x >> 3) >= per_xcd || t >= total)
+        return;
+    int const in_group = kGemmGroupM * p.tiles_n;
+    int const first_m = (t / in_group) * kGemmGroupM;
+    int const gsz = p.tiles_m - first_m < kGemmGroupM ? p.tiles_m - first_m : kGemmGroupM;
+    int const tm = first_m + (t % in_group) % gsz;
+    int const tn = (t % in_group) / gsz;
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const c = lane & 15;
+    int const kg = lane >> 4;
+    int const K = p.k;
+    int const KT = p.k_tiles;
+    int const m0 = tm * kGemmBM;
+    int const strip0 = tn * (kGemmBN / 16) + wave * NS;
+
+    constexpr uint32_t kOob = 0x80000000u;
+    auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
+    uint32_t const sz_bytes
+        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
+    auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
+    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+
+    int strip_of[NS];
+    uint32_t wlane[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+    }
+
+    f32x4 acc[RT][NS];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            acc[rt][s] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // per-column scale of the per-channel mode (GROUP == 0) is loaded once
+    float pc_scale[NS];
+    if constexpr (GROUP == 0)
+    {
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            pc_scale[s] = E::load(p.scales, strip_of[s] * 16 + c);
+    }
+
+    // A tile -> LDS: fragment f = rt * SLABS + j is 1 KiB, lane l of it holds
+    // act[m0 + rt*16 + l%16][kt*TK + j*32 + (l/16)*8 .. +8]; wavefront w moves fragments w, w+4, ...
+    auto dma_a = [&](auto* buf, int kt)
+    {
+        constexpr int FRAGS = RT * SLABS;
+#pragma unroll
+        for (int i = 0; i < FRAGS / 4; ++i)
+        {
+            int const f = wave + i * 4;
+            int const rt = f / SLABS, j = f % SLABS;
+            uint32_t const row = (uint32_t) (m0 + rt * 16 + c);
+            int const kk = kt * TK + j * 32 + kg * 8;
+            uint32_t const off = (kk < K && kt < KT) ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
+                (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(buf) + f * 1024), 16, (int) off, 0,
+                0, 0);
+        }
+    };
+
+    struct BStage
+    {
+        u32x4 w[NS];
+        uint16_t s[NS][SEGS];
+        uint16_t z[NS][SEGS];
+    };
+
+    auto fetch_b = [&](BStage& st, int kt)
+    {
+        uint32_t const tile_off = kt < KT ? (uint32_t) kt * 1024u : kOob;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
+        if constexpr (GROUP != 0)
+        {
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    uint32_t const off = (grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u;
+                    st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
+                    if constexpr (ZERO)
+                        st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
+                }
+            }
+        }
+    };
+
+    auto compute = [&](auto const* buf, BStage const& st)
+    {
+        char const* a_base = reinterpret_cast<char const*>(buf) + lane * 16;
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+        {
+            int const seg = j / SEG_SLABS;
+            u32x4 b[NS];
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+            {
+                float sc, zr;
+                if constexpr (GROUP != 0)
+                {
+                    sc = E::from_bits(st.s[s][seg]);
+                    zr = ZERO ? E::from_bits(st.z[s][seg]) : 0.f;
+                }
+                else
+                {
+                    sc = pc_scale[s];
+                    zr = 0.f;
+                }
+                if constexpr (BITS == 4)
+                    b[s] = dequant_int4_dword<DT>(st.w[s][j], sc, zr);
+                else
+                    b[s] = dequant_int8_dwords<DT>(st.w[s][2 * j], st.w[s][2 * j + 1], sc, zr);
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+            {
+                u32x4 const a = *reinterpret_cast<u32x4 const*>(a_base + (rt * SLABS + j) * 1024);
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                    acc[rt][s] = E::mma(a, b[s], acc[rt][s]);
+            }
+        }
+    };
+
+    // ---- main loop: two tile rows per iteration so that each LDS buffer is a distinct object ---
+    BStage st0, st1;
+    dma_a(a_buf0, 0);
+    fetch_b(st0, 0);
+    for (int kt = 0; kt < KT; kt += 2)
+    {
+        __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
+        dma_a(a_buf1, kt + 1);
+        fetch_b(st1, kt + 1);
+        compute(a_buf0, st0);
+        __syncthreads();
+        dma_a(a_buf0, kt + 2);
+        fetch_b(st0, kt + 2);
+        if (kt + 1 < KT)
+            compute(a_buf1, st1);
+    }
+
+    // ---- epilogue: out = T(alpha * acc + bias) ------------------------------------------------
+    uint16_t* out16 = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        if (strip0 + s >= p.strips)
+            continue;
+        int const col = (strip0 + s) * 16 + c;
+        float const bias = p.bias ? E::load(p.bias, col) : 0.f;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                int const row = m0 + rt * 16 + kg * 4 + r;
+                if (row < p.m)
+                    out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias));
+            }
+        }
+    }
+}
+
+template <int DT, int BITS, int GROUP, bool ZERO>
+int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
+{
+    int const total = gp.tiles_m * gp.tiles_n;
+    dim3 grid(((total + 7) / 8) * 8), block(256);
+    hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO>), grid, block, 0, stream, gp);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        return fail(WOQ_ERR_RUNTIME, "gemm kernel launch failed: %s", hipGetErrorString(err));
+    return WOQ_OK;
+}
+
+template <int DT, int BITS>
+int launch_gemm_typed(MatmulProblem const& p, void* stream)
+{
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    GemmParams gp;
+    gp.act = p.act;
+    gp.weight = p.weight;
+    gp.scales = p.scales;
+    gp.zeros = p.zeros;
+    gp.bias = p.bias;
+    gp.out = p.out;
+    gp.alpha = p.alpha;
+    gp.m = p.m;
+    gp.n = p.n;
+    gp.k = p.k;
+    gp.k_tiles = (p.k + TK - 1) / TK;
+    gp.strips = p.n / kTileN;
+    gp.tiles_m = (p.m + kGemmBM - 1) / kGemmBM;
+    gp.tiles_n = (p.n + kGemmBN - 1) / kGemmBN;
+    auto s = static_cast<hipStream_t>(stream);
+    bool const zero = p.zeros != nullptr;
+    switch (p.group_size)
+    {
+    case 0: return launch_gemm_variant<DT, BITS, 0, false>(gp, s);
+    case 64:
+        return zero ? launch_gemm_variant<DT, BITS, 64, true>(gp, s) : launch_gemm_variant<DT, BITS, 64, false>(gp, s);
+    case 128:
+        return zero ? launch_gemm_variant<DT, BITS, 128, true>(gp, s)
+                    : launch_gemm_variant<DT, BITS, 128, false>(gp, s);
+    default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
+    }
+}
+
+} // namespace woq

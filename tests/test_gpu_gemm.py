@@ -1,0 +1,74 @@
+"""GPU parity of the prefill MFMA GEMM against the CPU oracle, through the C ABI.  Same bar as the
+streaming kernel: max|out - ref| / max|ref| <= 1e-2 against the float64-accumulated
+dequantize-then-matmul reference."""
+import numpy as np
+import pytest
+import torch
+
+from _util import random_problem, reference, run_product
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+GEMM = 2
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("bits,group", [(4, 128), (4, 64), (4, 0), (8, 0), (8, 64), (8, 128)])
+@pytest.mark.parametrize("zero", [False, True])
+def test_gemm_variants(pkg, oracle, dev, dtype, bits, group, zero):
+    if group == 0 and zero:
+        pytest.skip("per-channel has no zeros")
+    p = random_problem(oracle, 300, 512, 512, bits, group, dtype, zero=zero, seed=bits + group)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("M", [1, 16, 129, 256, 257, 512, 1000])
+def test_gemm_m_edges(pkg, oracle, dev, M):
+    """Row counts around the 256-row tile, including the decode sizes forced onto this kernel."""
+    p = random_problem(oracle, M, 256, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("K,N", [(64, 256), (192, 272), (320, 16), (1024, 784), (2048, 4096)])
+def test_gemm_ragged_shapes(pkg, oracle, dev, K, N):
+    """K with a padded last weight tile row, N that is not a multiple of the 256-column tile."""
+    for bits, group in [(4, 64), (8, 64), (4, 0)]:
+        p = random_problem(oracle, 260, K, N, bits, group, "bf16", zero=group != 0, seed=K + N)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+        assert err < TOL, (bits, group, err)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_gemm_prequant_scale_goes_through_workspace(pkg, oracle, dev, dtype):
+    """AWQ smoothing in the GEMM regime: the smoothing pass writes the workspace, the GEMM reads it."""
+    p = random_problem(oracle, 384, 512, 256, 4, 128, dtype, zero=True, bias=True, pqs=True, seed=5)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    assert err < TOL, err
+
+
+def test_gemm_identity_recovers_dequantized_weight_exactly(pkg, oracle, dev):
+    """Identity activation: every output is ONE product 1 * w, so the GEMM returns the dequantized
+    weight bit for bit - the in-kernel dequantize equals the oracle's definition."""
+    K, N = 256, 256
+    for dtype in ("bf16", "fp16"):
+        p = random_problem(oracle, K, K, N, 4, 64, dtype, zero=True, seed=9)
+        p["act"] = np.eye(K, dtype=np.float32)
+        out = run_product(pkg, oracle, dev, p, GEMM)
+        w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 64, dtype)
+        assert (out.view(np.uint32) == w.view(np.uint32)).all(), dtype
+
+
+def test_gemm_matches_stream_kernel(pkg, oracle, dev):
+    """The two regimes agree with each other at their crossover size."""
+    p = random_problem(oracle, 128, 1024, 512, 4, 128, "bf16", zero=True, seed=31)
+    a = run_product(pkg, oracle, dev, p, 1)
+    b = run_product(pkg, oracle, dev, p, GEMM)
+    assert oracle.max_rel_err(a, b) < 1e-2  # each is within 1e-2 of the oracle; they round differently
+
+
+def test_auto_regime_dispatches_large_m_to_gemm(pkg, oracle, dev):
+    p = random_problem(oracle, 640, 256, 256, 8, 0, "fp16", seed=41)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+    assert err < TOL, err
