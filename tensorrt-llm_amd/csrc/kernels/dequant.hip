@@ -43,12 +43,11 @@ __global__ void __launch_bounds__(256) dequant_kernel(void* out, void const* wei
         }
         else
         {
-            // the very functions the GEMM main loop calls
+            // the very function the GEMM main loop calls
             u32x4 r;
-            if constexpr (BITS == 4)
-                r = dequant_int4_dword<DT>(w[j], s, z);
-            else
-                r = dequant_int8_dwords<DT>(w[2 * j], w[2 * j + 1], s, z);
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr)
+                r[pr] = dequant_operand_reg<DT, BITS>(w, j, pr, s, z);
             uint16_t* o = static_cast<uint16_t*>(out);
 #pragma unroll
             for (int e = 0; e < 8; ++e)

@@ -72,22 +72,56 @@ __device__ __forceinline__ u32x4 dequant8<WOQ_FP16>(int const (&q)[8], float s, 
     return r;
 }
 
-// one int4 dword (8 elements of one MFMA slab) -> the slab's B operand
-template <int DT>
-__device__ __forceinline__ u32x4 dequant_int4_dword(uint32_t w, float s, float z)
+// ---- pair-granular form used by the GEMM main loop --------------------------------------------
+// An MFMA B operand is 4 registers, register p holding elements (2p, 2p+1) of the slab.  The GEMM
+// produces one such register at a time so the conversion work can be spread evenly between the
+// matrix instructions.
+
+// signed values of elements 2p and 2p+1 of an int4 dword; `t` is the dword XOR 0x88888888
+// (biased nibbles -> two's complement); element 2p sits at nibble p, element 2p+1 at nibble p+4
+__device__ __forceinline__ void int4_pair(uint32_t t, int p, int& q0, int& q1)
 {
-    int q[8];
-    unpack_int4_signed(w, q);
-    return dequant8<DT>(q, s, z);
+    q0 = (int) (t << (28 - 4 * p)) >> 28;
+    q1 = (int) (t << (12 - 4 * p)) >> 28;
 }
 
-// two int8 dwords (8 elements of one MFMA slab) -> the slab's B operand
-template <int DT>
-__device__ __forceinline__ u32x4 dequant_int8_dwords(uint32_t w0, uint32_t w1, float s, float z)
+// signed values of elements 2p and 2p+1 of an int8 slab held in two dwords (bytes, biased by 128)
+__device__ __forceinline__ void int8_pair(uint32_t w0, uint32_t w1, int p, int& q0, int& q1)
 {
-    int q[8];
-    unpack_int8_signed(w0, w1, q);
-    return dequant8<DT>(q, s, z);
+    uint32_t const w = p < 2 ? w0 : w1;
+    int const sh = (p & 1) * 16;
+    q0 = (int) ((w >> sh) & 0xFF) - 128;
+    q1 = (int) ((w >> (sh + 8)) & 0xFF) - 128;
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t dequant_pair(int q0, int q1, float s, float z);
+
+template <>
+__device__ __forceinline__ uint32_t dequant_pair<WOQ_BF16>(int q0, int q1, float s, float z)
+{
+    return Elem<WOQ_BF16>::pack(__builtin_fmaf((float) q0, s, z), __builtin_fmaf((float) q1, s, z));
+}
+
+template <>
+__device__ __forceinline__ uint32_t dequant_pair<WOQ_FP16>(int q0, int q1, float s, float z)
+{
+    f16x2 const q2 = {(_Float16) q0, (_Float16) q1};
+    f16x2 const s2 = {(_Float16) s, (_Float16) s};
+    f16x2 const z2 = {(_Float16) z, (_Float16) z};
+    return bit_cast<uint32_t>(__builtin_elementwise_fma(q2, s2, z2));
+}
+
+// register p (elements 2p, 2p+1) of the B operand of slab j of a lane's 16 packed bytes `w`
+template <int DT, int BITS>
+__device__ __forceinline__ uint32_t dequant_operand_reg(u32x4 const& w, int j, int p, float s, float z)
+{
+    int q0, q1;
+    if constexpr (BITS == 4)
+        int4_pair(w[j] ^ 0x88888888u, p, q0, q1);
+    else
+        int8_pair(w[2 * j], w[2 * j + 1], p, q0, q1);
+    return dequant_pair<DT>(q0, q1, s, z);
 }
 
 // 8 dequantized values -> 8 e4m3 bytes (2 dwords), element order preserved

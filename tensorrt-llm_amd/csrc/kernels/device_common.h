@@ -45,6 +45,17 @@ struct Elem<WOQ_BF16>
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(bit_cast<bf16x8>(a), bit_cast<bf16x8>(b), c, 0, 0, 0);
     }
 
+    // c += a x b with the accumulator tied to ONE AGPR quad.  The builtin leaves destination and
+    // addend independent; with 256 live accumulator registers the allocator then renames them
+    // along the K loop and pays for it with hundreds of AGPR<->VGPR copies per step.  (A and B
+    // operands written by ordinary VALU instructions need no software wait states before an
+    // MFMA; the result must not be read by VALU code until the MFMA has drained - see
+    // mma_drain().)
+    static __device__ __forceinline__ void mma_acc(u32x4 a, u32x4 b, f32x4& c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+
     static __device__ __forceinline__ float lo(uint32_t pair)
     {
         return bit_cast<float>(pair << 16);
@@ -98,6 +109,11 @@ struct Elem<WOQ_FP16>
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<f16x8>(a), bit_cast<f16x8>(b), c, 0, 0, 0);
     }
 
+    static __device__ __forceinline__ void mma_acc(u32x4 a, u32x4 b, f32x4& c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+
     static __device__ __forceinline__ float lo(uint32_t pair)
     {
         return (float) bit_cast<f16x2>(pair)[0];
@@ -136,6 +152,14 @@ struct Elem<WOQ_FP16>
         return bit_cast<uint32_t>(bit_cast<f16x2>(a) * bit_cast<f16x2>(b));
     }
 };
+
+// Wait until every MFMA issued through mma_acc() has written its result: the compiler cannot
+// see that those asm statements are matrix instructions, so the wait states it would insert
+// before the first VALU read of an accumulator are inserted here (16 passes at most).
+__device__ __forceinline__ void mma_drain()
+{
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+}
 
 // ---- packed weights -> MFMA B operand holding (BASE + u) exactly ---------------------------
 // int4: dword `w` holds elements e at nibble (e even ? e/2 : 4 + e/2); operand register i is

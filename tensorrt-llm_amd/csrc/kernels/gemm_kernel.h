@@ -44,8 +44,11 @@ constexpr int kGemmBM = 256;
 constexpr int kGemmBN = 256;
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
 
+// amdgpu_waves_per_eu(1, 1): one wavefront per SIMD is the design point (256 accumulator
+// registers per lane); without it the register allocator chases a higher occupancy it cannot
+// reach and parks live values in the accumulator file, shuffling them around every step.
 template <int DT, int BITS, int GROUP, bool ZERO>
-__global__ void __launch_bounds__(256) gemm_kernel(GemmParams p)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_kernel(GemmParams p)
 {
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
@@ -164,41 +167,64 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmParams p)
         }
     };
 
+    // One tile row of MFMAs.  Hand-pipelined, because left alone the compiler hoists all
+    // fragment reads and conversions of the step to its top and runs out of registers:
+    //   * iteration (j, rt) issues the A-fragment read of the NEXT iteration, converts ONE
+    //     operand register of the next slab's B operands (16 registers per slab = 16 row tiles),
+    //     and issues the 4 MFMAs of this row tile;
+    //   * a scheduling barrier after every iteration keeps that interleaving intact.
     auto compute = [&](auto const* buf, BStage const& st)
     {
         char const* a_base = reinterpret_cast<char const*>(buf) + lane * 16;
+        float sc[NS][SEGS], zr[NS][SEGS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                if constexpr (GROUP != 0)
+                {
+                    sc[s][seg] = E::from_bits(st.s[s][seg]);
+                    zr[s][seg] = ZERO ? E::from_bits(st.z[s][seg]) : 0.f;
+                }
+                else
+                {
+                    sc[s][seg] = pc_scale[s];
+                    zr[s][seg] = 0.f;
+                }
+            }
+        u32x4 b_cur[NS], b_nxt[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int pr = 0; pr < 4; ++pr)
+                b_cur[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], 0, pr, sc[s][0], zr[s][0]);
+        u32x4 a_cur = *reinterpret_cast<u32x4 const*>(a_base);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
         {
-            int const seg = j / SEG_SLABS;
-            u32x4 b[NS];
-#pragma unroll
-            for (int s = 0; s < NS; ++s)
-            {
-                float sc, zr;
-                if constexpr (GROUP != 0)
-                {
-                    sc = E::from_bits(st.s[s][seg]);
-                    zr = ZERO ? E::from_bits(st.z[s][seg]) : 0.f;
-                }
-                else
-                {
-                    sc = pc_scale[s];
-                    zr = 0.f;
-                }
-                if constexpr (BITS == 4)
-                    b[s] = dequant_int4_dword<DT>(st.w[s][j], sc, zr);
-                else
-                    b[s] = dequant_int8_dwords<DT>(st.w[s][2 * j], st.w[s][2 * j + 1], sc, zr);
-            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
             {
-                u32x4 const a = *reinterpret_cast<u32x4 const*>(a_base + (rt * SLABS + j) * 1024);
+                // next fragment in (j, rt) order; the last iteration re-reads a valid fragment
+                int const nf = (j * RT + rt + 1) < SLABS * RT ? (j * RT + rt + 1) : 0;
+                int const nj = nf / RT, nrt = nf % RT;
+                u32x4 const a_nxt = *reinterpret_cast<u32x4 const*>(a_base + (nrt * SLABS + nj) * 1024);
+                if (j + 1 < SLABS)
+                {
+                    int const s = rt / 4, pr = rt % 4, seg = (j + 1) / SEG_SLABS;
+                    b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], j + 1, pr, sc[s][seg], zr[s][seg]);
+                }
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
-                    acc[rt][s] = E::mma(a, b[s], acc[rt][s]);
+                    E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
+                a_cur = a_nxt;
+                __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                b_cur[s] = b_nxt[s];
         }
     };
 
@@ -215,11 +241,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmParams p)
         __syncthreads();
         dma_a(a_buf0, kt + 2);
         fetch_b(st0, kt + 2);
-        if (kt + 1 < KT)
-            compute(a_buf1, st1);
+        compute(a_buf1, st1); // past the end of K both operands read as zeros: no branch needed
     }
 
     // ---- epilogue: out = T(alpha * acc + bias) ------------------------------------------------
+    mma_drain();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int s = 0; s < NS; ++s)
