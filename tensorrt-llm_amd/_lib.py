@@ -5,7 +5,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libwoq.so")
+# WOQ_LIB_PATH selects another build of the library (e.g. one compiled with experimental flags)
+_LIB_PATH = os.environ.get("WOQ_LIB_PATH") or os.path.join(_HERE, "libwoq.so")
 
 # enums of include/woq.h
 FP16, BF16, FP8_E4M3, FP32 = 0, 1, 2, 3

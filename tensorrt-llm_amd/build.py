@@ -15,8 +15,8 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-OBJ = os.path.join(HERE, "build")
-LIB = os.path.join(HERE, "libwoq.so")
+OBJ = os.environ.get("WOQ_OBJ_DIR") or os.path.join(HERE, "build")
+LIB = os.environ.get("WOQ_LIB_OUT") or os.path.join(HERE, "libwoq.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -39,7 +39,8 @@ def sources():
 def _compile(src: str) -> str:
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ, rel + ".o")
-    cmd = [HIPCC, "-x", "hip"] + DEVICE_FLAGS + COMMON + ["-c", src, "-o", obj]
+    extra = os.environ.get("WOQ_EXTRA_FLAGS", "").split()
+    cmd = [HIPCC, "-x", "hip"] + DEVICE_FLAGS + COMMON + extra + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "unknown to the target"  # host pass does not know the device-only feature flag
     err = "\n".join(l for l in r.stderr.splitlines() if noise not in l and "'-packed-fp32-ops'" not in l)

@@ -117,24 +117,37 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             pc_scale[s] = E::load(p.scales, strip_of[s] * 16 + c);
     }
 
-    // A tile -> LDS: fragment f = rt * SLABS + j is 1 KiB, lane l of it holds
-    // act[m0 + rt*16 + l%16][kt*TK + j*32 + (l/16)*8 .. +8]; wavefront w moves fragments w, w+4, ...
+    // A tile -> LDS.  Fragment f = rt * SLABS + j is 1 KiB: the 16 rows x 32 k that one MFMA
+    // consumes.  The DMA writes lane l's 16 bytes at offset l*16 of the fragment, so the lane
+    // order of the load instruction IS the LDS layout.  Lane l = 4*r + q fetches row r's chunk
+    // (q ^ (r>>2)) of the slab (a chunk = 8 k = 16 bytes):
+    //   * the 4 lanes of a quad read one contiguous 64-byte piece of a row (the L1 handles a
+    //     wavefront quad by quad: per-lane scattered 16-byte reads run 4x slower);
+    //   * the XOR spreads the 16 rows that an MFMA lane group (fixed chunk) reads over all 64
+    //     banks, so the fragment read below is conflict-free.
+    // Wavefront w moves fragments w, w+4, ...
     auto dma_a = [&](auto* buf, int kt)
     {
+#ifdef EXP_NO_DMA
+        return;
+#endif
         constexpr int FRAGS = RT * SLABS;
+        int const r = lane >> 2, chunk = (lane & 3) ^ ((lane >> 4) & 3);
 #pragma unroll
         for (int i = 0; i < FRAGS / 4; ++i)
         {
             int const f = wave + i * 4;
             int const rt = f / SLABS, j = f % SLABS;
-            uint32_t const row = (uint32_t) (m0 + rt * 16 + c);
-            int const kk = kt * TK + j * 32 + kg * 8;
+            uint32_t const row = (uint32_t) (m0 + rt * 16 + r);
+            int const kk = kt * TK + j * 32 + chunk * 8;
             uint32_t const off = (kk < K && kt < KT) ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob;
             __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
                 (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(buf) + f * 1024), 16, (int) off, 0,
                 0, 0);
         }
     };
+    // where MFMA lane (kg, c) finds its operand (row c, chunk kg) inside a fragment
+    int const a_lane_off = (c * 4 + (kg ^ ((c >> 2) & 3))) * 16;
 
     struct BStage
     {
@@ -169,37 +182,39 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // One tile row of MFMAs.  Hand-pipelined, because left alone the compiler hoists all
     // fragment reads and conversions of the step to its top and runs out of registers:
-    //   * iteration (j, rt) issues the A-fragment read of the NEXT iteration, converts ONE
-    //     operand register of the next slab's B operands (16 registers per slab = 16 row tiles),
-    //     and issues the 4 MFMAs of this row tile;
+    //   * iteration (j, rt) issues the A-fragment read that is A_AHEAD iterations away (LDS
+    //     latency is a few MFMA groups long), converts ONE operand register of the next slab's B
+    //     operands (16 registers per slab = 16 row tiles) and issues the 4 MFMAs of this row tile;
+    //   * the B operands of the first slab of the NEXT tile row are converted during the last
+    //     slab of this one (its packed weights were fetched at the start of this step), so the
+    //     matrix core never waits for a conversion burst at a step boundary;
     //   * a scheduling barrier after every iteration keeps that interleaving intact.
-    auto compute = [&](auto const* buf, BStage const& st)
+    constexpr int A_AHEAD = 3;
+    u32x4 b_cur[NS], b_nxt[NS];
+
+    auto scale_of = [&](BStage const& st, int s, int seg, float& sc, float& zr)
     {
-        char const* a_base = reinterpret_cast<char const*>(buf) + lane * 16;
-        float sc[NS][SEGS], zr[NS][SEGS];
+        if constexpr (GROUP != 0)
+        {
+            sc = E::from_bits(st.s[s][seg]);
+            zr = ZERO ? E::from_bits(st.z[s][seg]) : 0.f;
+        }
+        else
+        {
+            sc = pc_scale[s];
+            zr = 0.f;
+        }
+    };
+
+    auto compute = [&](auto const* buf, BStage const& st, BStage const& st_next)
+    {
+        char const* a_base = reinterpret_cast<char const*>(buf) + a_lane_off;
+        constexpr int ITERS = SLABS * RT;
+        auto a_addr = [&](int it) { return a_base + ((it % RT) * SLABS + it / RT) * 1024; };
+        u32x4 a_ring[A_AHEAD + 1];
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
-#pragma unroll
-            for (int seg = 0; seg < SEGS; ++seg)
-            {
-                if constexpr (GROUP != 0)
-                {
-                    sc[s][seg] = E::from_bits(st.s[s][seg]);
-                    zr[s][seg] = ZERO ? E::from_bits(st.z[s][seg]) : 0.f;
-                }
-                else
-                {
-                    sc[s][seg] = pc_scale[s];
-                    zr[s][seg] = 0.f;
-                }
-            }
-        u32x4 b_cur[NS], b_nxt[NS];
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-#pragma unroll
-            for (int pr = 0; pr < 4; ++pr)
-                b_cur[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], 0, pr, sc[s][0], zr[s][0]);
-        u32x4 a_cur = *reinterpret_cast<u32x4 const*>(a_base);
+        for (int i = 0; i < A_AHEAD; ++i)
+            a_ring[i] = *reinterpret_cast<u32x4 const*>(a_addr(i));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
@@ -207,19 +222,34 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
             {
-                // next fragment in (j, rt) order; the last iteration re-reads a valid fragment
-                int const nf = (j * RT + rt + 1) < SLABS * RT ? (j * RT + rt + 1) : 0;
-                int const nj = nf / RT, nrt = nf % RT;
-                u32x4 const a_nxt = *reinterpret_cast<u32x4 const*>(a_base + (nrt * SLABS + nj) * 1024);
-                if (j + 1 < SLABS)
+                int const it = j * RT + rt;
+#ifndef EXP_NO_LDS
+                if (it + A_AHEAD < ITERS)
+                    a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
+                        = *reinterpret_cast<u32x4 const*>(a_addr(it + A_AHEAD));
+#endif
                 {
-                    int const s = rt / 4, pr = rt % 4, seg = (j + 1) / SEG_SLABS;
-                    b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], j + 1, pr, sc[s][seg], zr[s][seg]);
+                    int const s = rt / 4, pr = rt % 4;
+                    float sc, zr;
+#ifdef EXP_NO_DEQUANT
+                    if (j + 1 < SLABS) b_nxt[s][pr] = st.w[s][pr] + j; else b_nxt[s][pr] = st_next.w[s][pr];
+#else
+                    if (j + 1 < SLABS)
+                    {
+                        scale_of(st, s, (j + 1) / SEG_SLABS, sc, zr);
+                        b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], j + 1, pr, sc, zr);
+                    }
+                    else
+                    {
+                        scale_of(st_next, s, 0, sc, zr);
+                        b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st_next.w[s], 0, pr, sc, zr);
+                    }
+#endif
                 }
+                u32x4 const a_cur = a_ring[it % (A_AHEAD + 1)];
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                     E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
-                a_cur = a_nxt;
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
@@ -232,16 +262,25 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     BStage st0, st1;
     dma_a(a_buf0, 0);
     fetch_b(st0, 0);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr)
+        {
+            float sc, zr;
+            scale_of(st0, s, 0, sc, zr);
+            b_cur[s][pr] = dequant_operand_reg<DT, BITS>(st0.w[s], 0, pr, sc, zr);
+        }
     for (int kt = 0; kt < KT; kt += 2)
     {
         __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
         dma_a(a_buf1, kt + 1);
         fetch_b(st1, kt + 1);
-        compute(a_buf0, st0);
+        compute(a_buf0, st0, st1);
         __syncthreads();
         dma_a(a_buf0, kt + 2);
         fetch_b(st0, kt + 2);
-        compute(a_buf1, st1); // past the end of K both operands read as zeros: no branch needed
+        compute(a_buf1, st1, st0); // past the end of K both operands read as zeros: no branch needed
     }
 
     // ---- epilogue: out = T(alpha * acc + bias) ------------------------------------------------
