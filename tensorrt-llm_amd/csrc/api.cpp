@@ -22,11 +22,12 @@ int launch_gemm_BF16_4(MatmulProblem const& p, void* stream);
 int launch_gemm_BF16_8(MatmulProblem const& p, void* stream);
 int launch_gemm_FP16_4(MatmulProblem const& p, void* stream);
 int launch_gemm_FP16_8(MatmulProblem const& p, void* stream);
+int launch_gemm_w4a8(MatmulProblem const& p, void* stream);
 
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
-        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 GEMM is not built yet");
+        return launch_gemm_w4a8(p, stream);
     if (p.out_dtype == WOQ_BF16)
         return p.bits == 4 ? launch_gemm_BF16_4(p, stream) : launch_gemm_BF16_8(p, stream);
     return p.bits == 4 ? launch_gemm_FP16_4(p, stream) : launch_gemm_FP16_8(p, stream);

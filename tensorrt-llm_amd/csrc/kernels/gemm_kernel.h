@@ -128,9 +128,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // Wavefront w moves fragments w, w+4, ...
     auto dma_a = [&](auto* buf, int kt)
     {
-#ifdef EXP_NO_DMA
-        return;
-#endif
         constexpr int FRAGS = RT * SLABS;
         int const r = lane >> 2, chunk = (lane & 3) ^ ((lane >> 4) & 3);
 #pragma unroll
@@ -223,17 +220,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (int rt = 0; rt < RT; ++rt)
             {
                 int const it = j * RT + rt;
-#ifndef EXP_NO_LDS
                 if (it + A_AHEAD < ITERS)
                     a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
                         = *reinterpret_cast<u32x4 const*>(a_addr(it + A_AHEAD));
-#endif
                 {
                     int const s = rt / 4, pr = rt % 4;
                     float sc, zr;
-#ifdef EXP_NO_DEQUANT
-                    if (j + 1 < SLABS) b_nxt[s][pr] = st.w[s][pr] + j; else b_nxt[s][pr] = st_next.w[s][pr];
-#else
                     if (j + 1 < SLABS)
                     {
                         scale_of(st, s, (j + 1) / SEG_SLABS, sc, zr);
@@ -244,7 +236,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                         scale_of(st_next, s, 0, sc, zr);
                         b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st_next.w[s], 0, pr, sc, zr);
                     }
-#endif
                 }
                 u32x4 const a_cur = a_ring[it % (A_AHEAD + 1)];
 #pragma unroll

@@ -1,0 +1,72 @@
+"""GPU parity of the W4A8 path (fp8 e4m3 activations x int4 weights, fp8 MFMA) against the oracle:
+both operands rounded to e4m3, float accumulation, alpha in the epilogue.  Tolerance 1e-2 of
+max|ref| as for the other kernels (the oracle rounds exactly like the kernel, so observed errors
+are output-rounding only)."""
+import numpy as np
+import pytest
+import torch
+
+from _util import preprocess, to_dev, TORCH_DT
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, direct_fp8=False):
+    F = pkg.functional
+    w = preprocess(pkg, oracle, prob["q"], 4, torch.float8_e4m3fn).to(dev)
+    scales = to_dev(prob["scales"], "fp16", dev)
+    algo = F.FP8_ALPHA | (F.ZERO if zeros is not None else 0) | (F.BIAS if bias is not None else 0)
+    z = None if zeros is None else to_dev(zeros, "fp16", dev)
+    b = None if bias is None else to_dev(bias, out_dtype, dev)
+    if direct_fp8:
+        a8 = oracle.apply_per_channel_scale(prob["act"], prob["pre_quant_scale"], out_dtype, "fp8")
+        act = torch.from_numpy(a8).to(dev).to(torch.float8_e4m3fn)
+        out = F.woq_matmul_raw(act, None, w, scales, z, b, n=N, k=K, group_size=128, quant_algo=algo,
+                               alpha=prob["alpha"], out_dtype=TORCH_DT[out_dtype])
+        ref = oracle.woq_matmul_ref(a8, prob["q"], prob["scales"], zeros, bias, None, prob["alpha"], 128, out_dtype,
+                                    w4a8=True)
+    else:
+        algo |= F.PRE_QUANT_SCALE
+        out = F.woq_matmul_raw(to_dev(prob["act"], out_dtype, dev), to_dev(prob["pre_quant_scale"], out_dtype, dev), w,
+                               scales, z, b, n=N, k=K, group_size=128, quant_algo=algo, alpha=prob["alpha"],
+                               out_dtype=TORCH_DT[out_dtype])
+        ref = oracle.woq_matmul_ref(prob["act"], prob["q"], prob["scales"], zeros, bias, prob["pre_quant_scale"],
+                                    prob["alpha"], 128, out_dtype, w4a8=True)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy(), ref
+
+
+@pytest.mark.parametrize("out_dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("M", [1, 16, 256, 300])
+@pytest.mark.parametrize("direct", [False, True])
+def test_w4a8_awq_style(pkg, oracle, dev, out_dtype, M, direct):
+    """The benchmark's W4A8 configuration at test size: symmetric int4 g128, smoothing vector,
+    per-tensor scales folded into alpha; activations given as 16-bit + smoothing vector (the
+    reference plugin's input) or directly as fp8."""
+    K, N = 1024, 384
+    prob = oracle.make_w4a8_problem(M, K, N, seed=M, out_dtype=out_dtype)
+    out, ref = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, direct_fp8=direct)
+    assert oracle.max_rel_err(out, ref) < TOL
+
+
+def test_w4a8_zeros_and_bias(pkg, oracle, dev):
+    M, K, N = 130, 512, 272
+    prob = oracle.make_w4a8_problem(M, K, N, seed=3, out_dtype="bf16")
+    rng = np.random.default_rng(4)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+    out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=zeros, bias=bias)
+    assert oracle.max_rel_err(out, ref) < TOL
+
+
+def test_w4a8_identity_recovers_e4m3_weight(pkg, oracle, dev):
+    """Identity activation (exact in e4m3) returns the e4m3-rounded dequantized weight times alpha."""
+    K, N = 256, 128
+    rng = np.random.default_rng(6)
+    q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    s = oracle.round_f16(np.exp(rng.uniform(-2, 3, (K // 128, N))).astype(np.float32))
+    prob = dict(q=q, scales=s, act=np.eye(K, dtype=np.float32), pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+    out, _ = _run(pkg, oracle, dev, prob, K, K, N, "fp16", direct_fp8=True)
+    w8 = oracle.dequantize(q, s, None, 128, "fp8")
+    assert (out == oracle.round_f16(w8)).all()
