@@ -32,6 +32,10 @@ GROUP = 128
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# calibrated with a 256 MiB copy (profiles/stream_gemv_gate_up_m1_hbm_traffic.md); counters cannot
+# be read from inside this process, so the figure is the recorded one
+DOMINANT_TRAFFIC_BYTES = 62_613_000
 
 
 def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
@@ -182,6 +186,32 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
         return dict(error=str(e)[:200])
 
 
+def run_for_counters(pkg, dev, mode, reps=20):
+    """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
+    dominant kernel (gate_up GEMV, rotating weight copies); `copy` runs a plain device-to-device
+    copy of a known size (256 MiB read + 256 MiB written per launch), whose FETCH_SIZE /
+    WRITE_SIZE readings calibrate the counters."""
+    if mode == "copy":
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(reps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": "copy", "bytes_read_per_launch": 256 << 20, "bytes_written_per_launch": 256 << 20,
+                          "launches": reps}))
+        return
+    _, k, n = SHAPES_8B[2]
+    copies = max(2, -(-3 * CACHE_BYTES // (k * n // 2)))
+    layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
+    act = torch.randn((1, k), device=dev).to(torch.bfloat16)
+    out = torch.empty((1, n), dtype=torch.bfloat16, device=dev)
+    for r in range(reps):
+        launch(pkg, act, layers[r % copies], out)
+    torch.cuda.synchronize()
+    print(json.dumps({"mode": "dominant", "kernel": "stream_kernel on gate_up K=4096 N=28672 M=1",
+                      "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n), "launches": reps}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -189,6 +219,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy"], default="bench",
+                    help="dominant / copy: launch only that kernel, for rocprofv3 --pmc runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "
@@ -199,6 +231,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.mode != "bench":
+        run_for_counters(pkg, dev, args.mode)
+        return
     r = bench_decode(pkg, dev, args.steps, args.warmup)
     sec_per_step = r["host_s"] / args.steps
     value = r["per_step_bytes"] / sec_per_step / 1e9
@@ -211,7 +246,7 @@ def main():
                                "bf16 scales+zeros, decode GEMV M=1; %d rotating weight copies" % r["copies"],
                    "m": 1, "group_size": GROUP, "weight_bits": 4},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DOMINANT_TRAFFIC_BYTES,
                      "kernel": "stream_kernel<bf16,int4,g128,MT=1> on gate_up K=4096 N=28672",
                      "bytes_per_launch": r["dom_bytes"], "us_per_launch": round(r["dom_dur"] * 1e6, 3)},
         "per_shape": r["per_shape"],
