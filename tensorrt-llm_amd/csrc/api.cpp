@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <initializer_list>
 
 #include "woq_internal.h"
 
@@ -199,16 +200,56 @@ extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_
     return m <= kStreamMaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
 }
 
+namespace
+{
+inline size_t align256(size_t v)
+{
+    return (v + 255) & ~(size_t) 255;
+}
+
+// bytes of the smoothed-activation region at the front of the workspace
+size_t smooth_bytes(int m, int k, int quant_algo)
+{
+    return (quant_algo & WOQ_ALGO_PRE_QUANT_SCALE) ? align256((size_t) m * (size_t) k * 2) : 0;
+}
+} // namespace
+
+// what one GEMM-regime call with exactly m rows uses
+static size_t gemm_workspace_bytes(int m, int n, int k, int quant_algo)
+{
+    size_t bytes = smooth_bytes(m, k, quant_algo);
+    if (!(quant_algo & WOQ_ALGO_FP8_ALPHA))
+        bytes += plan_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
+    return bytes;
+}
+
 extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype)
 {
-    (void) n;
     (void) act_dtype;
-    if (m <= 0 || k <= 0)
+    if (m <= 0 || k <= 0 || n <= 0)
         return 0;
-    // the GEMM regime smooths activations into the workspace first (the streaming kernel fuses it)
-    if (quant_algo & WOQ_ALGO_PRE_QUANT_SCALE)
-        return (size_t) m * (size_t) k * 2;
-    return 0;
+    // Enough for every call with at most m rows (the reference sizes its workspace for the
+    // profile's largest M the same way), in either regime.  The smoothing region grows with m;
+    // the split-K region does not (large m does not split), so take its maximum over the row
+    // counts at which the plan changes.
+    size_t bytes = smooth_bytes(m, k, quant_algo);
+    if (!(quant_algo & WOQ_ALGO_FP8_ALPHA))
+    {
+        int const bits = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
+        int const tiles_n = (n + 255) / 256;
+        int const wide = 256 * (159 / tiles_n); // most rows of 256-row tiles that still split
+        size_t split = 0;
+        for (int cand : {64, 128, wide, m})
+        {
+            int const mm = cand < m ? cand : m;
+            if (mm <= 0)
+                continue;
+            size_t const b = plan_gemm(mm, n, k, bits).ws_bytes;
+            split = b > split ? b : split;
+        }
+        bytes += split;
+    }
+    return bytes;
 }
 
 extern "C" int woq_matmul_check(const woq_matmul_args* args)
@@ -222,10 +263,10 @@ extern "C" int woq_matmul_check(const woq_matmul_args* args)
             args->m);
     if (regime == WOQ_REGIME_STREAM && p.w4a8)
         return fail(WOQ_ERR_UNSUPPORTED, "W4A8 runs on the fp8 MFMA GEMM kernel only");
-    if (regime == WOQ_REGIME_GEMM && p.pre_quant_scale)
+    if (regime == WOQ_REGIME_GEMM && p.m > 0)
     {
-        size_t const need = woq_workspace_bytes(p.m, p.n, p.k, args->quant_algo, p.act_dtype);
-        if (p.m > 0 && (!p.workspace || p.workspace_bytes < need))
+        size_t const need = gemm_workspace_bytes(p.m, p.n, p.k, args->quant_algo);
+        if (need && (!p.workspace || p.workspace_bytes < need))
             return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
                 p.workspace ? p.workspace_bytes : (size_t) 0);
     }
@@ -252,6 +293,9 @@ extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
         p.act = p.workspace;
         p.act_dtype = smoothed_dtype;
         p.pre_quant_scale = nullptr;
+        size_t const used = smooth_bytes(p.m, p.k, args->quant_algo);
+        p.workspace = static_cast<char*>(p.workspace) + used;
+        p.workspace_bytes -= used;
     }
     return launch_gemm(p, stream);
 }

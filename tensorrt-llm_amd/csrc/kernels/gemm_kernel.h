@@ -38,22 +38,29 @@ struct GemmParams
     int k_tiles; // ceil(k / TILE_K)
     int strips;  // n / 16
     int tiles_m, tiles_n;
+    int k_splits;        // workgroups along K per output tile (blockIdx.y)
+    int tiles_per_split; // tile rows of K each of them covers
+    float* partial;      // [m, n] float32, zeroed, when k_splits > 1
 };
 
-constexpr int kGemmBM = 256;
 constexpr int kGemmBN = 256;
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
 
 // amdgpu_waves_per_eu(1, 1): one wavefront per SIMD is the design point (256 accumulator
 // registers per lane); without it the register allocator chases a higher occupancy it cannot
 // reach and parks live values in the accumulator file, shuffling them around every step.
-template <int DT, int BITS, int GROUP, bool ZERO>
+//
+// RT     row tiles (16 rows) per wavefront: the output tile is 16*RT rows x 256 columns.  16 for
+//        prefill; 8 / 4 for skinny M, where a 256-row tile would mostly multiply padding.
+// SPLITK several workgroups share one output tile, each covering a slice of K, and add their
+//        partial sums into a float32 buffer (skinny M x narrow N would otherwise leave most CUs idle).
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_kernel(GemmParams p)
 {
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
-    constexpr int RT = kGemmBM / 16;                             // 16 row tiles per wavefront
+    constexpr int kGemmBM = RT * 16;
     constexpr int NS = 4;                                        // strips (16 columns) per wavefront
     constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
     constexpr int SEGS = TK / SEG;
@@ -80,7 +87,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int const c = lane & 15;
     int const kg = lane >> 4;
     int const K = p.k;
-    int const KT = p.k_tiles;
+    // this workgroup's slice of K, in tile rows; loads outside it return zeros
+    int const kt_begin = SPLITK ? (int) blockIdx.y * p.tiles_per_split : 0;
+    int const KT = SPLITK ? (kt_begin + p.tiles_per_split < p.k_tiles ? kt_begin + p.tiles_per_split : p.k_tiles)
+                          : p.k_tiles;
     int const m0 = tm * kGemmBM;
     int const strip0 = tn * (kGemmBN / 16) + wave * NS;
 
@@ -90,7 +100,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
-    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
 
     int strip_of[NS];
     uint32_t wlane[NS];
@@ -98,7 +108,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int s = 0; s < NS; ++s)
     {
         strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
-        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
     }
 
     f32x4 acc[RT][NS];
@@ -168,7 +178,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                 {
-                    uint32_t const off = (grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u;
+                    uint32_t const off
+                        = kt < KT ? (grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u : kOob;
                     st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
                     if constexpr (ZERO)
                         st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
@@ -180,8 +191,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // One tile row of MFMAs.  Hand-pipelined, because left alone the compiler hoists all
     // fragment reads and conversions of the step to its top and runs out of registers:
     //   * iteration (j, rt) issues the A-fragment read that is A_AHEAD iterations away (LDS
-    //     latency is a few MFMA groups long), converts ONE operand register of the next slab's B
-    //     operands (16 registers per slab = 16 row tiles) and issues the 4 MFMAs of this row tile;
+    //     latency is a few MFMA groups long), converts 16/RT operand registers of the next slab's
+    //     B operands (16 registers per slab) and issues the 4 MFMAs of this row tile;
     //   * the B operands of the first slab of the NEXT tile row are converted during the last
     //     slab of this one (its packed weights were fetched at the start of this step), so the
     //     matrix core never waits for a conversion burst at a step boundary;
@@ -223,8 +234,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 if (it + A_AHEAD < ITERS)
                     a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
                         = *reinterpret_cast<u32x4 const*>(a_addr(it + A_AHEAD));
+#pragma unroll
+                for (int ci = rt * (16 / RT); ci < (rt + 1) * (16 / RT); ++ci)
                 {
-                    int const s = rt / 4, pr = rt % 4;
+                    int const s = ci / 4, pr = ci % 4;
                     float sc, zr;
                     if (j + 1 < SLABS)
                     {
@@ -251,8 +264,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // ---- main loop: two tile rows per iteration so that each LDS buffer is a distinct object ---
     BStage st0, st1;
-    dma_a(a_buf0, 0);
-    fetch_b(st0, 0);
+    dma_a(a_buf0, kt_begin);
+    fetch_b(st0, kt_begin);
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -262,7 +275,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             scale_of(st0, s, 0, sc, zr);
             b_cur[s][pr] = dequant_operand_reg<DT, BITS>(st0.w[s], 0, pr, sc, zr);
         }
-    for (int kt = 0; kt < KT; kt += 2)
+    for (int kt = kt_begin; kt < KT; kt += 2)
     {
         __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
         dma_a(a_buf1, kt + 1);
@@ -274,7 +287,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         compute(a_buf1, st1, st0); // past the end of K both operands read as zeros: no branch needed
     }
 
-    // ---- epilogue: out = T(alpha * acc + bias) ------------------------------------------------
+    // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
 #pragma unroll
@@ -283,7 +296,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         if (strip0 + s >= p.strips)
             continue;
         int const col = (strip0 + s) * 16 + c;
-        float const bias = p.bias ? E::load(p.bias, col) : 0.f;
+        float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
         {
@@ -292,28 +305,77 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             {
                 int const row = m0 + rt * 16 + kg * 4 + r;
                 if (row < p.m)
-                    out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias));
+                {
+                    if constexpr (SPLITK)
+                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, acc[rt][s][r]);
+                    else
+                        out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias));
+                }
             }
         }
     }
 }
 
-template <int DT, int BITS, int GROUP, bool ZERO>
+// split-K helpers: clear the float32 partial buffer, then out = T(alpha * partial + bias)
+template <int DT>
+__global__ void __launch_bounds__(256) gemm_zero_partial(float* partial, size_t count)
+{
+    size_t const i = ((size_t) blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i < count)
+        *reinterpret_cast<f32x4*>(partial + i) = f32x4{0.f, 0.f, 0.f, 0.f}; // count is a multiple of 16
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) gemm_finish_partial(
+    void* out, float const* partial, void const* bias, float alpha, int m, int n)
+{
+    using E = Elem<DT>;
+    size_t const i = (size_t) blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t) m * n)
+        return;
+    int const col = (int) (i % n);
+    float const b = bias ? E::load(bias, col) : 0.f;
+    static_cast<uint16_t*>(out)[i] = E::store(__builtin_fmaf(alpha, partial[i], b));
+}
+
+template <int DT, int BITS, int GROUP, bool ZERO, int RT>
 int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
 {
     int const total = gp.tiles_m * gp.tiles_n;
-    dim3 grid(((total + 7) / 8) * 8), block(256);
-    hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO>), grid, block, 0, stream, gp);
+    dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(256);
+    if (gp.k_splits > 1)
+    {
+        size_t const count = (size_t) gp.m * gp.n;
+        hipLaunchKernelGGL((gemm_zero_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream, gp.partial,
+            count);
+        hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, true>), grid, block, 0, stream, gp);
+        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count + 255) / 256)), block, 0, stream, gp.out,
+            gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
+    }
+    else
+        hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "gemm kernel launch failed: %s", hipGetErrorString(err));
     return WOQ_OK;
 }
 
+template <int DT, int BITS, int GROUP, bool ZERO>
+int launch_gemm_rt(GemmParams const& gp, int rt, hipStream_t s)
+{
+    switch (rt)
+    {
+    case 4: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 4>(gp, s);
+    case 8: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 8>(gp, s);
+    default: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 16>(gp, s);
+    }
+}
+
 template <int DT, int BITS>
 int launch_gemm_typed(MatmulProblem const& p, void* stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
+    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, BITS);
     GemmParams gp;
     gp.act = p.act;
     gp.weight = p.weight;
@@ -327,18 +389,25 @@ int launch_gemm_typed(MatmulProblem const& p, void* stream)
     gp.k = p.k;
     gp.k_tiles = (p.k + TK - 1) / TK;
     gp.strips = p.n / kTileN;
-    gp.tiles_m = (p.m + kGemmBM - 1) / kGemmBM;
+    gp.tiles_m = (p.m + plan.rt * 16 - 1) / (plan.rt * 16);
     gp.tiles_n = (p.n + kGemmBN - 1) / kGemmBN;
+    gp.k_splits = plan.k_splits;
+    gp.tiles_per_split = (gp.k_tiles + plan.k_splits - 1) / plan.k_splits;
+    gp.tiles_per_split += gp.tiles_per_split & 1; // the main loop walks tile rows in pairs
+    gp.partial = static_cast<float*>(p.workspace);
+    if (plan.k_splits > 1 && (!p.workspace || p.workspace_bytes < plan.ws_bytes))
+        return fail(WOQ_ERR_WORKSPACE, "split-K needs %zu workspace bytes", plan.ws_bytes);
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
     switch (p.group_size)
     {
-    case 0: return launch_gemm_variant<DT, BITS, 0, false>(gp, s);
+    case 0: return launch_gemm_rt<DT, BITS, 0, false>(gp, plan.rt, s);
     case 64:
-        return zero ? launch_gemm_variant<DT, BITS, 64, true>(gp, s) : launch_gemm_variant<DT, BITS, 64, false>(gp, s);
+        return zero ? launch_gemm_rt<DT, BITS, 64, true>(gp, plan.rt, s)
+                    : launch_gemm_rt<DT, BITS, 64, false>(gp, plan.rt, s);
     case 128:
-        return zero ? launch_gemm_variant<DT, BITS, 128, true>(gp, s)
-                    : launch_gemm_variant<DT, BITS, 128, false>(gp, s);
+        return zero ? launch_gemm_rt<DT, BITS, 128, true>(gp, plan.rt, s)
+                    : launch_gemm_rt<DT, BITS, 128, false>(gp, plan.rt, s);
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 }

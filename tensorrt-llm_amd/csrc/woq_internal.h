@@ -55,6 +55,35 @@ int launch_prequant(void* out, void const* act, void const* scale, int m, int k,
 int launch_dequant(void* out, void const* weight, void const* scales, void const* zeros, int k, int n, int group_size,
     int bits, int dtype, void* stream);
 
+// How the prefill GEMM is launched for a problem: rows per output tile (16 * rt) and the number
+// of workgroups that split K for one tile (with a float32 partial buffer of ws_bytes when > 1).
+struct GemmPlan
+{
+    int rt;
+    int k_splits;
+    size_t ws_bytes;
+};
+
+inline GemmPlan plan_gemm(int m, int n, int k, int bits)
+{
+    GemmPlan pl;
+    pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
+    int const tk = tile_k_of_bits(bits);
+    int const k_tiles = (k + tk - 1) / tk;
+    long const tiles = (long) ((m + pl.rt * 16 - 1) / (pl.rt * 16)) * ((n + 255) / 256);
+    pl.k_splits = 1;
+    if (tiles < 160 && k_tiles >= 8)
+    {
+        long splits = 320 / tiles;
+        if (splits > k_tiles / 4)
+            splits = k_tiles / 4;
+        if (splits > 1)
+            pl.k_splits = (int) splits;
+    }
+    pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+    return pl;
+}
+
 // largest M the streaming kernel is instantiated for
 constexpr int kStreamMaxM = 128;
 

@@ -71,8 +71,16 @@ def test_workspace_rule(pkg):
     L = pkg._lib
     lib = L.lib
     algo = L.ALGO_PRE_QUANT_SCALE
-    assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2
-    assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == 0
+    # the split-K partial buffer: none at m=4096 x n=4096 itself (256 tiles fill the chip), but the
+    # size covers every smaller m too, and up to 2304 rows (9 x 16 tiles) still split
+    split = 2304 * 4096 * 4
+    assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2 + split
+    assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == split
+    assert lib.woq_workspace_bytes(64, 4096, 8192, 0, L.BF16) == 64 * 4096 * 4
+    assert lib.woq_workspace_bytes(4096, 20480, 8192, 0, L.BF16) == 256 * 20480 * 4
+    # never shrinks as m grows
+    sizes = [lib.woq_workspace_bytes(m, 1024, 4096, algo, L.FP16) for m in range(1, 3000, 37)]
+    assert sizes == sorted(sizes)
     # GEMM regime with smoothing needs the workspace; the streaming regime fuses it
     rc, msg = status(pkg, m=512, pre_quant_scale=0x5000, quant_algo=algo)
     assert rc == -4 and "workspace" in msg

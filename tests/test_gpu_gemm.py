@@ -72,3 +72,33 @@ def test_auto_regime_dispatches_large_m_to_gemm(pkg, oracle, dev):
     p = random_problem(oracle, 640, 256, 256, 8, 0, "fp16", seed=41)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
     assert err < TOL, err
+
+
+@pytest.mark.parametrize("M", [17, 64, 65, 100, 128, 200, 512])
+@pytest.mark.parametrize("K,N", [(4096, 256), (2048, 1024), (1152, 528)])
+def test_gemm_skinny_m_splits_k(pkg, oracle, dev, M, K, N):
+    """Skinny M x narrow N: 64/128/256-row tiles and K split across workgroups through the float32
+    partial buffer (ragged K slices, a last slice shorter than the others, bias in the finish pass)."""
+    for bits, group, dtype in [(4, 128, "bf16"), (8, 64, "fp16"), (4, 0, "fp16")]:
+        p = random_problem(oracle, M, K, N, bits, group, dtype, zero=group != 0, bias=True, seed=M + K)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+        assert err < TOL, (bits, group, dtype, err)
+
+
+def test_gemm_split_k_reuses_a_dirty_workspace(pkg, oracle, dev):
+    """The partial buffer is cleared by the call itself: a workspace full of garbage, used twice."""
+    F = pkg.functional
+    p = random_problem(oracle, 48, 4096, 256, 4, 128, "bf16", zero=True, pqs=True, seed=77)
+    need = pkg._lib.lib.woq_workspace_bytes(48, 256, 4096, F.ZERO | F.PRE_QUANT_SCALE, pkg._lib.BF16)
+    assert need > 48 * 4096 * 2  # smoothing region plus partial sums
+    ws = torch.full((need,), 0x7F, dtype=torch.uint8, device=dev)
+    from _util import TORCH_DT, preprocess, to_dev
+    w = preprocess(pkg, oracle, p["q"], 4).to(dev)
+    ref = reference(oracle, p)
+    for _ in range(2):
+        out = F.woq_matmul_raw(to_dev(p["act"], "bf16", dev), to_dev(p["pqs"], "bf16", dev), w,
+                               to_dev(p["scales"], "bf16", dev), to_dev(p["zeros"], "bf16", dev), None, n=256,
+                               k=4096, group_size=128, quant_algo=F.ZERO | F.PRE_QUANT_SCALE, regime=GEMM,
+                               workspace=ws)
+        torch.cuda.synchronize()
+        assert oracle.max_rel_err(out.float().cpu().numpy(), ref) < TOL
