@@ -25,6 +25,9 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
           "-ffp-contract=off"]
+# Per-file additions.  The skinny-M kernel reads its MFMA results with VALU instructions every
+# group: keep those accumulators in the architectural VGPRs instead of copying them out of AGPRs.
+PER_FILE = {"skinny_": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources():
@@ -40,6 +43,9 @@ def _compile(src: str) -> str:
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ, rel + ".o")
     extra = os.environ.get("WOQ_EXTRA_FLAGS", "").split()
+    for prefix, flags in PER_FILE.items():
+        if os.path.basename(src).startswith(prefix):
+            extra = extra + flags
     cmd = [HIPCC, "-x", "hip"] + DEVICE_FLAGS + COMMON + extra + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "unknown to the target"  # host pass does not know the device-only feature flag

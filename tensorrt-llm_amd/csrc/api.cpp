@@ -19,19 +19,31 @@ int launch_stream_BF16_8(MatmulProblem const& p, void* stream);
 int launch_stream_FP16_4(MatmulProblem const& p, void* stream);
 int launch_stream_FP16_8(MatmulProblem const& p, void* stream);
 
-int launch_gemm_BF16_4(MatmulProblem const& p, void* stream);
-int launch_gemm_BF16_8(MatmulProblem const& p, void* stream);
-int launch_gemm_FP16_4(MatmulProblem const& p, void* stream);
-int launch_gemm_FP16_8(MatmulProblem const& p, void* stream);
+int launch_gemm_BF16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_gemm_BF16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_gemm_FP16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_gemm_FP16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_skinny_BF16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_skinny_BF16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_skinny_FP16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+int launch_skinny_FP16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream);
 int launch_gemm_w4a8(MatmulProblem const& p, void* stream);
 
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_gemm_w4a8(p, stream);
-    if (p.out_dtype == WOQ_BF16)
-        return p.bits == 4 ? launch_gemm_BF16_4(p, stream) : launch_gemm_BF16_8(p, stream);
-    return p.bits == 4 ? launch_gemm_FP16_4(p, stream) : launch_gemm_FP16_8(p, stream);
+    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, p.bits);
+    bool const bf16 = p.out_dtype == WOQ_BF16;
+    if (plan.skinny)
+    {
+        if (bf16)
+            return p.bits == 4 ? launch_skinny_BF16_4(p, plan, stream) : launch_skinny_BF16_8(p, plan, stream);
+        return p.bits == 4 ? launch_skinny_FP16_4(p, plan, stream) : launch_skinny_FP16_8(p, plan, stream);
+    }
+    if (bf16)
+        return p.bits == 4 ? launch_gemm_BF16_4(p, plan, stream) : launch_gemm_BF16_8(p, plan, stream);
+    return p.bits == 4 ? launch_gemm_FP16_4(p, plan, stream) : launch_gemm_FP16_8(p, plan, stream);
 }
 
 int launch_stream(MatmulProblem const& p, void* stream)
@@ -193,11 +205,16 @@ using namespace woq;
 
 extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo)
 {
-    (void) n;
-    (void) k;
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
         return WOQ_REGIME_GEMM;
-    return m <= kStreamMaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
+    // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed; with two row
+    // tiles the streaming kernel still wins on small matrices (it needs no split-K passes), and
+    // from 33 rows on the MFMA GEMM kernels (64-row deferred-scale tiles first) are faster.
+    if (m <= 16)
+        return WOQ_REGIME_STREAM;
+    if (m <= 32 && (int64_t) n * k < ((int64_t) 1 << 26))
+        return WOQ_REGIME_STREAM;
+    return WOQ_REGIME_GEMM;
 }
 
 namespace
@@ -231,19 +248,15 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     // Enough for every call with at most m rows (the reference sizes its workspace for the
     // profile's largest M the same way), in either regime.  The smoothing region grows with m;
     // the split-K region does not (large m does not split), so take its maximum over the row
-    // counts at which the plan changes.
+    // counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
     if (!(quant_algo & WOQ_ALGO_FP8_ALPHA))
     {
         int const bits = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
-        int const tiles_n = (n + 255) / 256;
-        int const wide = 256 * (159 / tiles_n); // most rows of 256-row tiles that still split
-        size_t split = 0;
-        for (int cand : {64, 128, wide, m})
+        // the plan changes at multiples of the 64-row tile; 160 or more tiles never split
+        size_t split = plan_gemm(m, n, k, bits).ws_bytes;
+        for (int mm = 64; mm < m && mm <= 64 * 160; mm += 64)
         {
-            int const mm = cand < m ? cand : m;
-            if (mm <= 0)
-                continue;
             size_t const b = plan_gemm(mm, n, k, bits).ws_bytes;
             split = b > split ? b : split;
         }

@@ -226,6 +226,17 @@ __device__ __forceinline__ u32x4 expand_int8<WOQ_FP16>(uint32_t w0, uint32_t w1)
     return r;
 }
 
+// one register of the above: `half` 0 -> bytes 0,1 of w, 1 -> bytes 2,3
+template <int DT>
+__device__ __forceinline__ uint32_t expand_int8_reg(uint32_t w, int half)
+{
+    if constexpr (DT == WOQ_BF16)
+        return half == 0 ? Elem<WOQ_BF16>::pack((float) (w & 0xFF), (float) ((w >> 8) & 0xFF))
+                         : Elem<WOQ_BF16>::pack((float) ((w >> 16) & 0xFF), (float) (w >> 24));
+    else
+        return __builtin_amdgcn_perm(0x64646464u, w, half == 0 ? 0x04010400u : 0x04030402u);
+}
+
 // additive constant carried by the expanded operand: expanded value = q + kOffset
 template <int DT, int BITS>
 struct Offset

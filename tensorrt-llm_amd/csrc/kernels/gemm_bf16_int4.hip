@@ -3,8 +3,8 @@
 
 namespace woq
 {
-int launch_gemm_BF16_4(MatmulProblem const& p, void* stream)
+int launch_gemm_BF16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream)
 {
-    return launch_gemm_typed<WOQ_BF16, 4>(p, stream);
+    return launch_gemm_typed<WOQ_BF16, 4>(p, plan, stream);
 }
 } // namespace woq

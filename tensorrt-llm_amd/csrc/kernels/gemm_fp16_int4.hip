@@ -3,8 +3,8 @@
 
 namespace woq
 {
-int launch_gemm_FP16_4(MatmulProblem const& p, void* stream)
+int launch_gemm_FP16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream)
 {
-    return launch_gemm_typed<WOQ_FP16, 4>(p, stream);
+    return launch_gemm_typed<WOQ_FP16, 4>(p, plan, stream);
 }
 } // namespace woq

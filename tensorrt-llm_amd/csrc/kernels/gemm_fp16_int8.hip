@@ -3,8 +3,8 @@
 
 namespace woq
 {
-int launch_gemm_FP16_8(MatmulProblem const& p, void* stream)
+int launch_gemm_FP16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream)
 {
-    return launch_gemm_typed<WOQ_FP16, 8>(p, stream);
+    return launch_gemm_typed<WOQ_FP16, 8>(p, plan, stream);
 }
 } // namespace woq

@@ -21,27 +21,10 @@
 #pragma once
 
 #include "dequant_math.h"
+#include "gemm_common.h"
 
 namespace woq
 {
-
-struct GemmParams
-{
-    void const* act;
-    void const* weight;
-    void const* scales;
-    void const* zeros;
-    void const* bias;
-    void* out;
-    float alpha;
-    int m, n, k;
-    int k_tiles; // ceil(k / TILE_K)
-    int strips;  // n / 16
-    int tiles_m, tiles_n;
-    int k_splits;        // workgroups along K per output tile (blockIdx.y)
-    int tiles_per_split; // tile rows of K each of them covers
-    float* partial;      // [m, n] float32, zeroed, when k_splits > 1
-};
 
 constexpr int kGemmBN = 256;
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
@@ -147,7 +130,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             int const rt = f / SLABS, j = f % SLABS;
             uint32_t const row = (uint32_t) (m0 + rt * 16 + r);
             int const kk = kt * TK + j * 32 + chunk * 8;
-            uint32_t const off = (kk < K && kt < KT) ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob;
+            // out of range (sign bit of K-1-kk or of KT-1-kt set) -> an offset the descriptor rejects
+            uint32_t const off
+                = ((row * (uint32_t) K + (uint32_t) kk) * 2u) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
                 (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(buf) + f * 1024), 16, (int) off, 0,
                 0, 0);
@@ -165,7 +150,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     auto fetch_b = [&](BStage& st, int kt)
     {
-        uint32_t const tile_off = kt < KT ? (uint32_t) kt * 1024u : kOob;
+        uint32_t const past = (uint32_t) (KT - 1 - kt) & kOob; // kt >= KT: every load of the step reads zeros
+        uint32_t const tile_off = (uint32_t) kt * 1024u | past;
 #pragma unroll
         for (int s = 0; s < NS; ++s)
             st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
@@ -178,8 +164,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                 {
-                    uint32_t const off
-                        = kt < KT ? (grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u : kOob;
+                    uint32_t const off = ((grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u) | past;
                     st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
                     if constexpr (ZERO)
                         st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
@@ -316,28 +301,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
 }
 
-// split-K helpers: clear the float32 partial buffer, then out = T(alpha * partial + bias)
-template <int DT>
-__global__ void __launch_bounds__(256) gemm_zero_partial(float* partial, size_t count)
-{
-    size_t const i = ((size_t) blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i < count)
-        *reinterpret_cast<f32x4*>(partial + i) = f32x4{0.f, 0.f, 0.f, 0.f}; // count is a multiple of 16
-}
-
-template <int DT>
-__global__ void __launch_bounds__(256) gemm_finish_partial(
-    void* out, float const* partial, void const* bias, float alpha, int m, int n)
-{
-    using E = Elem<DT>;
-    size_t const i = (size_t) blockIdx.x * 256 + threadIdx.x;
-    if (i >= (size_t) m * n)
-        return;
-    int const col = (int) (i % n);
-    float const b = bias ? E::load(bias, col) : 0.f;
-    static_cast<uint16_t*>(out)[i] = E::store(__builtin_fmaf(alpha, partial[i], b));
-}
-
 template <int DT, int BITS, int GROUP, bool ZERO, int RT>
 int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
 {
@@ -372,10 +335,9 @@ int launch_gemm_rt(GemmParams const& gp, int rt, hipStream_t s)
 }
 
 template <int DT, int BITS>
-int launch_gemm_typed(MatmulProblem const& p, void* stream)
+int launch_gemm_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, BITS);
     GemmParams gp;
     gp.act = p.act;
     gp.weight = p.weight;

@@ -1,0 +1,439 @@
+// Skinny-M GEMM: the rows-in-the-tens-to-hundreds regime between the streaming GEMV kernel and
+// the 256-row prefill GEMM (the reference covers it with CUTLASS tiles of 16..64 rows and split-K,
+// cpp/tensorrt_llm/kernels/cutlass_kernels/cutlass_heuristic.cpp:59-140).
+//
+// Here the work per weight byte is too small to pay for an exact dequantize of every weight (one
+// conversion per weight and only a few MFMAs to amortise it), so the kernel uses the streaming
+// kernel's arithmetic on a GEMM skeleton:
+//   * the packed integers are expanded to the activation type by one bit operation per pair
+//     (value q + OFFSET, exact) and multiplied as they are; per scale group the matrix core
+//     produces P = sum a * (q + OFFSET) and, against an all-ones operand, S = sum a;
+//   * the scale is applied to the float32 sums, once per group and output element:
+//     acc += s * P + (z - OFFSET * s) * S.
+// Output tile 64 rows x 256 columns; 4 wavefronts side by side along N, each 64 x 64, one
+// workgroup per CU.  Everything a step needs is requested DEPTH steps ahead (a skinny problem is
+// bound by memory latency unless tens of KiB per CU are in flight): the activation tile and the
+// group scales go global -> LDS by DMA, packed weights go straight to the registers of the lane
+// that feeds them to the matrix core.
+#pragma once
+
+#include "gemm_common.h"
+
+namespace woq
+{
+
+constexpr int kSkinnyBM = 64;
+constexpr int kSkinnyBN = 256;
+constexpr int kSkinnyWaves = 8; // two per SIMD: one wavefront's VALU and memory instructions run under the other's MFMAs
+
+template <int DT, int BITS, int GROUP, bool ZERO, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 4)>
+__global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) skinny_kernel(GemmParams p)
+{
+    using E = Elem<DT>;
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    constexpr int SLABS = TK / 32;
+    constexpr int RT = kSkinnyBM / 16;                           // row tiles per wavefront
+    constexpr int NS = kSkinnyBN / 16 / kSkinnyWaves;            // strips (16 columns) per wavefront
+    constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
+    constexpr int SEGS = TK / SEG;
+    constexpr int SEG_SLABS = SEG / 32;
+    constexpr int A_BYTES = kSkinnyBM * TK * 2;
+    constexpr float OFF = Offset<DT, BITS>::value;
+
+    constexpr int SC_SLOTS = GROUP != 0 ? SEGS * (ZERO ? 2 : 1) : 0; // 256-byte scale slots per wavefront and step
+
+    // One LDS object per step in flight.  They are separate variables on purpose: the compiler
+    // orders an LDS read after the DMA writes to the SAME variable only, so reading step kt's
+    // buffer does not wait for the DMA just issued into another one.
+    struct StageLds
+    {
+        u32x4 a[A_BYTES / 16];
+        u32x4 sc[kSkinnyWaves][(SC_SLOTS ? SC_SLOTS : 1) * 16];
+    };
+    static_assert(DEPTH + 1 <= 7, "seven stage buffers are declared");
+    __shared__ StageLds lds0, lds1, lds2, lds3, lds4, lds5, lds6;
+    StageLds* const stage_lds[7] = {&lds0, &lds1, &lds2, &lds3, &lds4, &lds5, &lds6};
+
+    int t;
+    if (!xcd_tile(p.tiles_m * p.tiles_n, t))
+        return;
+    int const tm = t % p.tiles_m, tn = t / p.tiles_m;
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const c = lane & 15;
+    int const kg = lane >> 4;
+    int const K = p.k;
+    // this workgroup's slice of K, in tile rows; loads outside it return zeros
+    int const kt_begin = SPLITK ? (int) blockIdx.y * p.tiles_per_split : 0;
+    int const KT = SPLITK ? (kt_begin + p.tiles_per_split < p.k_tiles ? kt_begin + p.tiles_per_split : p.k_tiles)
+                          : p.k_tiles;
+    int const m0 = tm * kSkinnyBM;
+    int const strip0 = tn * (kSkinnyBN / 16) + wave * NS;
+
+    constexpr uint32_t kOob = 0x80000000u;
+    auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
+    uint32_t const sz_bytes
+        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
+    auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
+    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
+
+    int strip_of[NS];
+    uint32_t wlane[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
+    }
+
+    f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
+    u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
+    [[maybe_unused]] NibbleConsts const nib = nibble_consts<DT>();
+
+    // acc: finished sums (GROUP != 0) or the running P (per-channel scales are applied at the end);
+    // acc_s: the running S of the per-channel mode
+    f32x4 acc[RT][NS];
+    f32x4 acc_s[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+    {
+        acc_s[rt] = zero4;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            acc[rt][s] = zero4;
+    }
+
+    // A tile -> LDS, same fragment layout as the prefill kernel: fragment f = rt * SLABS + j is the
+    // 16 rows x 32 k of one MFMA; lane l = 4*r + q fetches row r's 16-byte chunk (q ^ (r>>2)), so
+    // quads read contiguous 64 bytes from memory and the fragment read is bank-conflict free.
+    constexpr int FRAGS = RT * SLABS;
+    static_assert(FRAGS % kSkinnyWaves == 0, "fragments spread evenly over the wavefronts");
+    constexpr int DMA_OPS = FRAGS / kSkinnyWaves;
+    auto dma_a = [&](int buf, int kt)
+    {
+        int const r = lane >> 2, chunk = (lane & 3) ^ ((lane >> 4) & 3);
+#pragma unroll
+        for (int i = 0; i < DMA_OPS; ++i)
+        {
+            int const f = wave + i * kSkinnyWaves;
+            int const rt = f / SLABS, j = f % SLABS;
+            uint32_t const row = (uint32_t) (m0 + rt * 16 + r);
+            int const kk = kt * TK + j * 32 + chunk * 8;
+            // out of range (sign bit of K-1-kk or of KT-1-kt set) -> an offset the descriptor rejects
+            uint32_t const off
+                = ((row * (uint32_t) K + (uint32_t) kk) * 2u) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
+                (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(stage_lds[buf]->a) + f * 1024), 16,
+                (int) off, 0, 0, 0);
+        }
+    };
+    int const a_lane_off = (c * 4 + (kg ^ ((c >> 2) & 3))) * 16;
+
+    struct Stage
+    {
+        u32x4 w[NS];
+    };
+    // vector-memory instructions one fetch_b issues (the explicit wait below counts them)
+    constexpr int FETCH_OPS = NS + SC_SLOTS;
+
+    // Scales (and zeros) of the wavefront's 16*NS columns for one group, fetched by the first 8*NS
+    // lanes as dwords straight into LDS (the other lanes get zeros from an out-of-range offset).
+    int const col0 = strip0 * 16;
+    uint32_t const sc_lane_col = (uint32_t) (col0 + 2 * (lane & 31));
+    uint32_t const sc_lane_oob = (lane >= 8 * NS || (int) sc_lane_col >= p.n) ? kOob : 0u;
+
+    auto fetch_b = [&](Stage& st, int buf, int kt)
+    {
+        uint32_t const past = (uint32_t) (KT - 1 - kt) & kOob; // kt >= KT: every load of the step reads zeros
+        uint32_t const tile_off = (uint32_t) kt * 1024u | past;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
+        if constexpr (GROUP != 0)
+        {
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+                uint32_t const off = ((grow * (uint32_t) p.n + sc_lane_col) * 2u) | past | sc_lane_oob;
+                char* slot = reinterpret_cast<char*>(stage_lds[buf]->sc[wave]) + seg * (ZERO ? 512 : 256);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                    sc_rsrc, (__attribute__((address_space(3))) void*) slot, 4, (int) off, 0, 0, 0);
+                if constexpr (ZERO)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                        zr_rsrc, (__attribute__((address_space(3))) void*) (slot + 256), 4, (int) off, 0, 0, 0);
+            }
+        }
+    };
+
+    // One step = one tile row of K.  All A fragments of the step are read into registers once; the
+    // strips are then processed one after the other, so only one strip's group sums (P) are live
+    // at a time.  A single wavefront per SIMD has to overlap its own VALU work with the matrix
+    // core, so the step is written as mini-blocks of ONE MFMA plus a few VALU instructions (a
+    // scheduling barrier after each keeps them together):
+    //   * the B operand of the next 4 MFMAs is expanded one register per mini-block;
+    //   * the scale application of strip s-1 is spread over the 16 mini-blocks of strip s; that of
+    //     the last strip is carried into the next step, where it runs first and covers the
+    //     latency of the fragment reads.
+    f32x4 part[2][SEGS][RT];   // P of the strip in flight / of the strip being scaled
+    f32x4 part_s[SEGS][RT];    // S of the step's groups
+    float sc[NS][SEGS], cc[NS][SEGS]; // s and z - OFFSET * s of the step (strip NS-1: of the pending strip)
+#pragma unroll
+    for (int seg = 0; seg < SEGS; ++seg)
+    {
+        sc[NS - 1][seg] = cc[NS - 1][seg] = 0.f;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+            part[1][seg][rt] = part_s[seg][rt] = zero4;
+    }
+    static_assert(NS % 2 == 0, "the last strip uses part[1]");
+
+    // unit u of the scale application of strip s: one (group, row tile, register) of acc
+    auto apply_unit = [&](int s, int u)
+    {
+        if constexpr (GROUP != 0)
+        {
+            int const seg = u % SEGS, rt = (u / SEGS) / 4, r = (u / SEGS) % 4;
+            acc[rt][s][r] = __builtin_fmaf(
+                sc[s][seg], part[s & 1][seg][rt][r], __builtin_fmaf(cc[s][seg], part_s[seg][rt][r], acc[rt][s][r]));
+        }
+    };
+    constexpr int UNITS = SEGS * 16; // per strip
+
+    // register pr (elements 2pr, 2pr+1) of the B operand of slab j of a lane's 16 packed bytes
+    auto expand_reg = [&](u32x4 const& w, int j, int pr) -> uint32_t
+    {
+        if constexpr (BITS == 4)
+            return ((w[j] >> (4 * pr)) & nib.mask) | nib.magic;
+        else
+            return expand_int8_reg<DT>(w[2 * j + pr / 2], pr % 2);
+    };
+
+    auto compute = [&](int buf, Stage const& st)
+    {
+        char const* a_base = reinterpret_cast<char const*>(stage_lds[buf]->a) + a_lane_off;
+        [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_lds[buf]->sc[wave]) + c * 2;
+        u32x4 a[RT][SLABS];
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                a[rt][j] = *reinterpret_cast<u32x4 const*>(a_base + (rt * SLABS + j) * 1024);
+        uint16_t raw_s[NS][SEGS], raw_z[NS][SEGS];
+        if constexpr (GROUP != 0)
+        {
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int seg = 0; seg < SEGS; ++seg)
+                {
+                    char const* slot = sc_base + seg * (ZERO ? 512 : 256) + s * 32;
+                    raw_s[s][seg] = *reinterpret_cast<uint16_t const*>(slot);
+                    raw_z[s][seg] = ZERO ? *reinterpret_cast<uint16_t const*>(slot + 256) : (uint16_t) 0;
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // pending scale application of the previous step's last strip (uses the previous S)
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+            apply_unit(NS - 1, u);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (GROUP != 0)
+        {
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int seg = 0; seg < SEGS; ++seg)
+                {
+                    sc[s][seg] = E::from_bits(raw_s[s][seg]);
+                    cc[s][seg] = __builtin_fmaf(-OFF, sc[s][seg], ZERO ? E::from_bits(raw_z[s][seg]) : 0.f);
+                }
+        }
+
+        // S of every group of the step (per-channel mode: the running S); the first B operand is
+        // expanded underneath
+        u32x4 b_cur, b_nxt;
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+            {
+                if constexpr (GROUP != 0)
+                    part_s[j / SEG_SLABS][rt]
+                        = E::mma(a[rt][j], ones, j % SEG_SLABS == 0 ? zero4 : part_s[j / SEG_SLABS][rt]);
+                else
+                    acc_s[rt] = E::mma(a[rt][j], ones, acc_s[rt]);
+                if (j == SLABS - 1)
+                    b_cur[rt] = expand_reg(st.w[0], 0, rt);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+#pragma unroll
+            for (int j = 0; j < SLABS; ++j)
+            {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                {
+                    if constexpr (GROUP != 0)
+                        part[s & 1][j / SEG_SLABS][rt] = E::mma(
+                            a[rt][j], b_cur, j % SEG_SLABS == 0 ? zero4 : part[s & 1][j / SEG_SLABS][rt]);
+                    else
+                        acc[rt][s] = E::mma(a[rt][j], b_cur, acc[rt][s]);
+                    // one register of the next B operand (RT == 4 registers per operand)
+                    if (j + 1 < SLABS)
+                        b_nxt[rt] = expand_reg(st.w[s], j + 1, rt);
+                    else if (s + 1 < NS)
+                        b_nxt[rt] = expand_reg(st.w[s + 1], 0, rt);
+                    if (s > 0)
+                    {
+                        constexpr int BLOCKS = SLABS * RT; // mini-blocks per strip
+                        static_assert(UNITS % BLOCKS == 0, "scale units spread evenly");
+                        int const blk = j * RT + rt;
+#pragma unroll
+                        for (int u = blk * (UNITS / BLOCKS); u < (blk + 1) * (UNITS / BLOCKS); ++u)
+                            apply_unit(s - 1, u);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                b_cur = b_nxt;
+            }
+        }
+    };
+    static_assert(RT == 4, "one register of the next B operand per row-tile mini-block");
+
+    // ---- main loop --------------------------------------------------------------------------
+    // Step kt: wait until everything this wavefront requested for step kt has landed, barrier (now
+    // all of A(kt) is in LDS and nobody reads A(kt-1) any more), request step kt+DEPTH (its A tile
+    // goes into the buffer A(kt-1) used), compute step kt.
+    // Vector-memory operations retire in order, so "step kt has landed" is "at most the requests
+    // of the DEPTH-1 younger steps are outstanding".
+    constexpr int WAIT = (DEPTH - 1) * (FETCH_OPS + DMA_OPS);
+    static_assert(WAIT < 64, "vmcnt is a 6-bit counter");
+    Stage st[DEPTH + 1];
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i)
+    {
+        dma_a(i, kt_begin + i);
+        fetch_b(st[i], i, kt_begin + i);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int kt = kt_begin; kt < KT; kt += DEPTH + 1)
+    {
+#pragma unroll
+        for (int u = 0; u < DEPTH + 1; ++u)
+        {
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAIT) : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            dma_a((u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
+            fetch_b(st[(u + DEPTH) % (DEPTH + 1)], (u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt + u < KT) // uniform; the requests above go on (they read zeros past the end of K)
+                compute(u, st[u]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no DMA may still be writing LDS when the wavefront ends
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+        apply_unit(NS - 1, u); // the last step's last strip
+
+    // ---- epilogue ----------------------------------------------------------------------------
+    uint16_t* out16 = static_cast<uint16_t*>(p.out);
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        if (strip0 + s >= p.strips)
+            continue;
+        int const col = (strip0 + s) * 16 + c;
+        float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
+        [[maybe_unused]] float const pc = GROUP == 0 ? E::load(p.scales, col) : 0.f;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                int const row = m0 + rt * 16 + kg * 4 + r;
+                float v = acc[rt][s][r];
+                if constexpr (GROUP == 0)
+                    v = __builtin_fmaf(pc, v, (-OFF * pc) * acc_s[rt][r]);
+                if (row < p.m)
+                {
+                    if constexpr (SPLITK)
+                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, v);
+                    else
+                        out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, v, bias));
+                }
+            }
+        }
+    }
+}
+
+template <int DT, int BITS, int GROUP, bool ZERO>
+int launch_skinny_variant(GemmParams const& gp, hipStream_t stream)
+{
+    int const total = gp.tiles_m * gp.tiles_n;
+    dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(kSkinnyWaves * 64), block256(256);
+    if (gp.k_splits > 1)
+    {
+        size_t const count = (size_t) gp.m * gp.n;
+        hipLaunchKernelGGL((gemm_zero_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block256, 0, stream,
+            gp.partial, count);
+        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, true>), grid, block, 0, stream, gp);
+        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count + 255) / 256)), block256, 0, stream, gp.out,
+            gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
+    }
+    else
+        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, false>), grid, block, 0, stream, gp);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        return fail(WOQ_ERR_RUNTIME, "skinny gemm kernel launch failed: %s", hipGetErrorString(err));
+    return WOQ_OK;
+}
+
+template <int DT, int BITS>
+int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream)
+{
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    GemmParams gp;
+    gp.act = p.act;
+    gp.weight = p.weight;
+    gp.scales = p.scales;
+    gp.zeros = p.zeros;
+    gp.bias = p.bias;
+    gp.out = p.out;
+    gp.alpha = p.alpha;
+    gp.m = p.m;
+    gp.n = p.n;
+    gp.k = p.k;
+    gp.k_tiles = (p.k + TK - 1) / TK;
+    gp.strips = p.n / kTileN;
+    gp.tiles_m = (p.m + kSkinnyBM - 1) / kSkinnyBM;
+    gp.tiles_n = (p.n + kSkinnyBN - 1) / kSkinnyBN;
+    gp.k_splits = plan.k_splits;
+    gp.tiles_per_split = (gp.k_tiles + plan.k_splits - 1) / plan.k_splits;
+    gp.partial = static_cast<float*>(p.workspace);
+    if (plan.k_splits > 1 && (!p.workspace || p.workspace_bytes < plan.ws_bytes))
+        return fail(WOQ_ERR_WORKSPACE, "split-K needs %zu workspace bytes", plan.ws_bytes);
+    auto s = static_cast<hipStream_t>(stream);
+    bool const zero = p.zeros != nullptr;
+    switch (p.group_size)
+    {
+    case 0: return launch_skinny_variant<DT, BITS, 0, false>(gp, s);
+    case 64:
+        return zero ? launch_skinny_variant<DT, BITS, 64, true>(gp, s)
+                    : launch_skinny_variant<DT, BITS, 64, false>(gp, s);
+    case 128:
+        return zero ? launch_skinny_variant<DT, BITS, 128, true>(gp, s)
+                    : launch_skinny_variant<DT, BITS, 128, false>(gp, s);
+    default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
+    }
+}
+
+} // namespace woq

@@ -4,6 +4,8 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 #include "../../include/woq.h"
 
@@ -55,22 +57,34 @@ int launch_prequant(void* out, void const* act, void const* scale, int m, int k,
 int launch_dequant(void* out, void const* weight, void const* scales, void const* zeros, int k, int n, int group_size,
     int bits, int dtype, void* stream);
 
-// How the prefill GEMM is launched for a problem: rows per output tile (16 * rt) and the number
-// of workgroups that split K for one tile (with a float32 partial buffer of ws_bytes when > 1).
+// How the GEMM regime runs a problem: which kernel, rows per output tile and the number of
+// workgroups that split K for one tile (with a float32 partial buffer of ws_bytes when > 1).
 struct GemmPlan
 {
-    int rt;
+    bool skinny;  // deferred-scale 64-row kernel instead of the exact-dequantize prefill kernel
+    int rt;       // prefill kernel: row tiles per wavefront (tile rows = 16 * rt)
     int k_splits;
     size_t ws_bytes;
 };
 
+// The deferred-scale 64-row kernel is preferred up to 256 rows, and up to 512 rows when N is narrow
+// (few column panels: the 256-row tiles of the prefill kernel would leave most CUs idle).
+inline bool prefer_skinny(int m, int n)
+{
+    return m <= 256 || (m <= 512 && n <= 8192);
+}
+
+// Environment overrides for experiments: WOQ_GEMM_KERNEL=exact|skinny, WOQ_GEMM_SPLITS=<n>
 inline GemmPlan plan_gemm(int m, int n, int k, int bits)
 {
     GemmPlan pl;
+    char const* e = std::getenv("WOQ_GEMM_KERNEL");
+    pl.skinny = e ? !std::strcmp(e, "skinny") : prefer_skinny(m, n);
     pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
+    int const tile_rows = pl.skinny ? 64 : pl.rt * 16;
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
-    long const tiles = (long) ((m + pl.rt * 16 - 1) / (pl.rt * 16)) * ((n + 255) / 256);
+    long const tiles = (long) ((m + tile_rows - 1) / tile_rows) * ((n + 255) / 256);
     pl.k_splits = 1;
     if (tiles < 160 && k_tiles >= 8)
     {
@@ -79,6 +93,12 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits)
             splits = k_tiles / 4;
         if (splits > 1)
             pl.k_splits = (int) splits;
+    }
+    if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
+    {
+        int const v = std::atoi(f);
+        if (v >= 1 && v <= k_tiles)
+            pl.k_splits = v;
     }
     pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
     return pl;

@@ -77,7 +77,7 @@ def test_workspace_rule(pkg):
     assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2 + split
     assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == split
     assert lib.woq_workspace_bytes(64, 4096, 8192, 0, L.BF16) == 64 * 4096 * 4
-    assert lib.woq_workspace_bytes(4096, 20480, 8192, 0, L.BF16) == 256 * 20480 * 4
+    assert lib.woq_workspace_bytes(4096, 20480, 8192, 0, L.BF16) == 64 * 20480 * 4
     # never shrinks as m grows
     sizes = [lib.woq_workspace_bytes(m, 1024, 4096, algo, L.FP16) for m in range(1, 3000, 37)]
     assert sizes == sorted(sizes)
@@ -92,10 +92,13 @@ def test_workspace_rule(pkg):
 def test_regime_table(pkg):
     L = pkg._lib
     sel = L.lib.woq_select_regime
-    for m in (1, 2, 4, 15, 16, 64, 128):
+    for m in (1, 2, 4, 15, 16, 17, 32):
         assert sel(m, 4096, 4096, 0) == L.REGIME_STREAM
-    for m in (129, 256, 4096, 8192):
+    for m in (33, 64, 128, 129, 256, 4096, 8192):
         assert sel(m, 4096, 4096, 0) == L.REGIME_GEMM
+    # two row tiles: streaming on small matrices only
+    assert sel(32, 28672, 4096, 0) == L.REGIME_GEMM
+    assert sel(16, 28672, 4096, 0) == L.REGIME_STREAM
     assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
 
 

@@ -12,6 +12,14 @@ TOL = 1e-2
 GEMM = 2
 
 
+@pytest.fixture(params=["exact", "skinny"], autouse=True)
+def gemm_kernel(request, monkeypatch):
+    """The GEMM regime has two kernels (exact-dequantize 256-row tiles, deferred-scale 64-row tiles);
+    every test below runs on each, whatever the library would pick for the shape."""
+    monkeypatch.setenv("WOQ_GEMM_KERNEL", request.param)
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("bits,group", [(4, 128), (4, 64), (4, 0), (8, 0), (8, 64), (8, 128)])
 @pytest.mark.parametrize("zero", [False, True])
@@ -48,9 +56,11 @@ def test_gemm_prequant_scale_goes_through_workspace(pkg, oracle, dev, dtype):
     assert err < TOL, err
 
 
-def test_gemm_identity_recovers_dequantized_weight_exactly(pkg, oracle, dev):
+def test_gemm_identity_recovers_dequantized_weight_exactly(pkg, oracle, dev, gemm_kernel):
     """Identity activation: every output is ONE product 1 * w, so the GEMM returns the dequantized
     weight bit for bit - the in-kernel dequantize equals the oracle's definition."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel applies scales to float32 sums, not to single weights")
     K, N = 256, 256
     for dtype in ("bf16", "fp16"):
         p = random_problem(oracle, K, K, N, 4, 64, dtype, zero=True, seed=9)
@@ -68,7 +78,12 @@ def test_gemm_matches_stream_kernel(pkg, oracle, dev):
     assert oracle.max_rel_err(a, b) < 1e-2  # each is within 1e-2 of the oracle; they round differently
 
 
-def test_auto_regime_dispatches_large_m_to_gemm(pkg, oracle, dev):
+def test_auto_regime_and_kernel_choice(pkg, oracle, dev, monkeypatch):
+    monkeypatch.delenv("WOQ_GEMM_KERNEL")
+    for m in (200, 640):
+        p = random_problem(oracle, m, 512, 256, 4, 128, "bf16", zero=True, seed=40 + m)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+        assert err < TOL, (m, err)
     p = random_problem(oracle, 640, 256, 256, 8, 0, "fp16", seed=41)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
     assert err < TOL, err
