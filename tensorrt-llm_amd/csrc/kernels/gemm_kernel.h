@@ -119,24 +119,39 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     //   * the XOR spreads the 16 rows that an MFMA lane group (fixed chunk) reads over all 64
     //     banks, so the fragment read below is conflict-free.
     // Wavefront w moves fragments w, w+4, ...
+    // Wavefront w moves fragments w, w+4, ...: piece i is fragment f = w + 4i, i.e. slab w % SLABS
+    // of row tile i * (4 / SLABS) + w / SLABS - the same slab for every piece, rows a fixed stride
+    // apart, so one per-lane base (set once per step, out of range past the end of K) plus a
+    // compile-time multiple of the row stride addresses every piece.
+    constexpr int FRAGS = RT * SLABS;
+    constexpr int DMA_OPS = FRAGS / 4;
+    static_assert(4 % SLABS == 0 && FRAGS % 4 == 0, "fragment to wavefront mapping");
+    int const dma_j = wave % SLABS;
+    uint32_t const dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
+                                       + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
+        * 2u;
+    int const dma_lane_k = dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8); // k of this lane inside a tile row
+    uint32_t const dma_piece_stride = (uint32_t) (4 / SLABS) * 16u * (uint32_t) K * 2u;
+    auto dma_base = [&](int kt) -> uint32_t
+    {
+        // out of range (sign bit of K-1-k or of KT-1-kt set) -> an offset the descriptor rejects;
+        // rows past M fall outside the descriptor by themselves
+        int const kk = kt * TK + dma_lane_k;
+        return (dma_lane_base + (uint32_t) kt * (uint32_t) (TK * 2)) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
+    };
+    auto dma_piece = [&](auto* buf, uint32_t base, int i)
+    {
+        int const f = wave + i * 4;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
+            (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(buf) + f * 1024), 16,
+            (int) (base + (uint32_t) i * dma_piece_stride), 0, 0, 0);
+    };
     auto dma_a = [&](auto* buf, int kt)
     {
-        constexpr int FRAGS = RT * SLABS;
-        int const r = lane >> 2, chunk = (lane & 3) ^ ((lane >> 4) & 3);
+        uint32_t const base = dma_base(kt);
 #pragma unroll
-        for (int i = 0; i < FRAGS / 4; ++i)
-        {
-            int const f = wave + i * 4;
-            int const rt = f / SLABS, j = f % SLABS;
-            uint32_t const row = (uint32_t) (m0 + rt * 16 + r);
-            int const kk = kt * TK + j * 32 + chunk * 8;
-            // out of range (sign bit of K-1-kk or of KT-1-kt set) -> an offset the descriptor rejects
-            uint32_t const off
-                = ((row * (uint32_t) K + (uint32_t) kk) * 2u) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
-                (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(buf) + f * 1024), 16, (int) off, 0,
-                0, 0);
-        }
+        for (int i = 0; i < DMA_OPS; ++i)
+            dma_piece(buf, base, i);
     };
     // where MFMA lane (kg, c) finds its operand (row c, chunk kg) inside a fragment
     int const a_lane_off = (c * 4 + (kg ^ ((c >> 2) & 3))) * 16;
@@ -148,29 +163,34 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         uint16_t z[NS][SEGS];
     };
 
-    auto fetch_b = [&](BStage& st, int kt)
+    // piece i of the weight-side requests of step kt: the NS packed-weight loads, then the scales
+    // and zeros of the step's groups
+    constexpr int FETCH_OPS = NS + (GROUP != 0 ? NS * SEGS * (ZERO ? 2 : 1) : 0);
+    uint32_t sc_lane[NS]; // byte offset of this lane's column in a scale row
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        sc_lane[s] = (uint32_t) (strip_of[s] * 16 + c) * 2u;
+    auto fetch_piece = [&](BStage& st, int kt, int i)
     {
         uint32_t const past = (uint32_t) (KT - 1 - kt) & kOob; // kt >= KT: every load of the step reads zeros
-        uint32_t const tile_off = (uint32_t) kt * 1024u | past;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
-        if constexpr (GROUP != 0)
+        if (i < NS)
+            st.w[i] = buffer_load_x4(w_rsrc, wlane[i] + ((uint32_t) kt * 1024u | past));
+        else if constexpr (GROUP != 0)
         {
-#pragma unroll
-            for (int seg = 0; seg < SEGS; ++seg)
-            {
-                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
-#pragma unroll
-                for (int s = 0; s < NS; ++s)
-                {
-                    uint32_t const off = ((grow * (uint32_t) p.n + (uint32_t) (strip_of[s] * 16 + c)) * 2u) | past;
-                    st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
-                    if constexpr (ZERO)
-                        st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
-                }
-            }
+            int const q = i - NS, which = q / (NS * SEGS), seg = (q / NS) % SEGS, s = q % NS;
+            uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+            uint32_t const off = (grow * (uint32_t) p.n * 2u + sc_lane[s]) | past;
+            if (which == 0)
+                st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
+            else
+                st.z[s][seg] = buffer_load_u16(zr_rsrc, off);
         }
+    };
+    auto fetch_b = [&](BStage& st, int kt)
+    {
+#pragma unroll
+        for (int i = 0; i < FETCH_OPS; ++i)
+            fetch_piece(st, kt, i);
     };
 
     // One tile row of MFMAs.  Hand-pipelined, because left alone the compiler hoists all
@@ -181,6 +201,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     //   * the B operands of the first slab of the NEXT tile row are converted during the last
     //     slab of this one (its packed weights were fetched at the start of this step), so the
     //     matrix core never waits for a conversion burst at a step boundary;
+    //   * the memory requests of the next step (weight-side loads first: they are converted in this
+    //     step's last slab; then the A-tile DMAs) are spread over the iterations as well: a
+    //     wavefront that issues them in one burst sits in instruction issue while the matrix core
+    //     runs dry;
     //   * a scheduling barrier after every iteration keeps that interleaving intact.
     constexpr int A_AHEAD = 3;
     u32x4 b_cur[NS], b_nxt[NS];
@@ -199,10 +223,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
     };
 
-    auto compute = [&](auto const* buf, BStage const& st, BStage const& st_next)
+    auto compute = [&](auto const* buf, BStage const& st, BStage& st_next, auto* buf_next, int kt_next)
     {
         char const* a_base = reinterpret_cast<char const*>(buf) + a_lane_off;
         constexpr int ITERS = SLABS * RT;
+        uint32_t const next_base = dma_base(kt_next);
         auto a_addr = [&](int it) { return a_base + ((it % RT) * SLABS + it / RT) * 1024; };
         u32x4 a_ring[A_AHEAD + 1];
 #pragma unroll
@@ -216,6 +241,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             for (int rt = 0; rt < RT; ++rt)
             {
                 int const it = j * RT + rt;
+                // weight-side pieces all before the last slab (which converts them), DMAs throughout
+                constexpr int FETCH_WINDOW = (SLABS - 1) * RT;
+#pragma unroll
+                for (int q = 0; q < FETCH_OPS; ++q)
+                    if (q * FETCH_WINDOW / FETCH_OPS == it)
+                        fetch_piece(st_next, kt_next, q);
+#pragma unroll
+                for (int q = 0; q < DMA_OPS; ++q)
+                    if (q * ITERS / DMA_OPS == it)
+                        dma_piece(buf_next, next_base, q);
                 if (it + A_AHEAD < ITERS)
                     a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
                         = *reinterpret_cast<u32x4 const*>(a_addr(it + A_AHEAD));
@@ -263,13 +298,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int kt = kt_begin; kt < KT; kt += 2)
     {
         __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
-        dma_a(a_buf1, kt + 1);
-        fetch_b(st1, kt + 1);
-        compute(a_buf0, st0, st1);
+        compute(a_buf0, st0, st1, a_buf1, kt + 1);
         __syncthreads();
-        dma_a(a_buf0, kt + 2);
-        fetch_b(st0, kt + 2);
-        compute(a_buf1, st1, st0); // past the end of K both operands read as zeros: no branch needed
+        compute(a_buf1, st1, st0, a_buf0, kt + 2); // past the end of K both operands read as zeros: no branch needed
     }
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
