@@ -188,7 +188,8 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
 
 def run_for_counters(pkg, dev, mode, reps=20):
     """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
-    dominant kernel (gate_up GEMV, rotating weight copies); `copy` runs a plain device-to-device
+    dominant kernel (gate_up GEMV, rotating weight copies); `gemm<M>` launches the GEMM regime on
+    gate_up at M rows (prefill kernel at 4096, skinny kernel at 128); `copy` runs a plain device-to-device
     copy of a known size (256 MiB read + 256 MiB written per launch), whose FETCH_SIZE /
     WRITE_SIZE readings calibrate the counters."""
     if mode == "copy":
@@ -201,6 +202,17 @@ def run_for_counters(pkg, dev, mode, reps=20):
                           "launches": reps}))
         return
     _, k, n = SHAPES_8B[2]
+    if mode.startswith("gemm"):
+        m = int(mode[4:] or 4096)
+        layer = make_layer(pkg, dev, k, n, 2002)
+        act = torch.randn((m, k), device=dev).to(torch.bfloat16)
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        for r in range(reps):
+            launch(pkg, act, layer, out)
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": mode, "kernel": "GEMM regime on gate_up K=4096 N=28672 M=%d" % m,
+                          "flop_per_launch": 2.0 * m * n * k, "launches": reps}))
+        return
     copies = max(2, -(-3 * CACHE_BYTES // (k * n // 2)))
     layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
     act = torch.randn((1, k), device=dev).to(torch.bfloat16)
@@ -219,8 +231,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy"], default="bench",
-                    help="dominant / copy: launch only that kernel, for rocprofv3 --pmc runs")
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128"], default="bench",
+                    help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "

@@ -242,14 +242,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             {
                 int const it = j * RT + rt;
                 // weight-side pieces all before the last slab (which converts them), DMAs throughout
-                constexpr int FETCH_WINDOW = (SLABS - 1) * RT;
+                // (one per iteration from the start: they travel the farthest, from HBM)
+                constexpr int FETCH_WINDOW = (SLABS - 1) * RT < FETCH_OPS ? (SLABS - 1) * RT : FETCH_OPS;
 #pragma unroll
                 for (int q = 0; q < FETCH_OPS; ++q)
                     if (q * FETCH_WINDOW / FETCH_OPS == it)
                         fetch_piece(st_next, kt_next, q);
+                constexpr int DMA_WINDOW = ITERS * 5 / 8 > 0 ? ITERS * 5 / 8 : 1; // leave the tail of the step for them to land
 #pragma unroll
                 for (int q = 0; q < DMA_OPS; ++q)
-                    if (q * ITERS / DMA_OPS == it)
+                    if (q * DMA_WINDOW / DMA_OPS == it)
                         dma_piece(buf_next, next_base, q);
                 if (it + A_AHEAD < ITERS)
                     a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
