@@ -231,13 +231,18 @@ size_t smooth_bytes(int m, int k, int quant_algo)
 }
 } // namespace
 
+// float32 partial buffer of one GEMM-regime call with exactly m rows
+static size_t split_bytes(int m, int n, int k, int quant_algo)
+{
+    if (quant_algo & WOQ_ALGO_FP8_ALPHA)
+        return plan_gemm_w4a8(m, n, k).ws_bytes;
+    return plan_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
+}
+
 // what one GEMM-regime call with exactly m rows uses
 static size_t gemm_workspace_bytes(int m, int n, int k, int quant_algo)
 {
-    size_t bytes = smooth_bytes(m, k, quant_algo);
-    if (!(quant_algo & WOQ_ALGO_FP8_ALPHA))
-        bytes += plan_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
-    return bytes;
+    return smooth_bytes(m, k, quant_algo) + split_bytes(m, n, k, quant_algo);
 }
 
 extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype)
@@ -250,18 +255,14 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     // the split-K region does not (large m does not split), so take its maximum over the row
     // counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
-    if (!(quant_algo & WOQ_ALGO_FP8_ALPHA))
+    // the plan changes at multiples of the 64-row tile; 160 or more tiles never split
+    size_t split = split_bytes(m, n, k, quant_algo);
+    for (int mm = 64; mm < m && mm <= 64 * 160; mm += 64)
     {
-        int const bits = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
-        // the plan changes at multiples of the 64-row tile; 160 or more tiles never split
-        size_t split = plan_gemm(m, n, k, bits).ws_bytes;
-        for (int mm = 64; mm < m && mm <= 64 * 160; mm += 64)
-        {
-            size_t const b = plan_gemm(mm, n, k, bits).ws_bytes;
-            split = b > split ? b : split;
-        }
-        bytes += split;
+        size_t const b = split_bytes(mm, n, k, quant_algo);
+        split = b > split ? b : split;
     }
+    bytes += split;
     return bytes;
 }
 

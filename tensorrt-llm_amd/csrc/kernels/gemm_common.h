@@ -25,6 +25,8 @@ struct GemmParams
     float* partial;      // [m, n] float32, zeroed, when k_splits > 1
 };
 
+constexpr int kGemmBN = 256; // columns of an output tile (4 wavefronts x 64)
+
 // Output tiles are numbered m-fastest inside a column panel; the 8 XCDs each take one contiguous
 // chunk of that order (workgroup i runs on XCD i % 8), so the workgroups that share weight
 // columns or activation rows also share an L2.

@@ -26,7 +26,6 @@
 namespace woq
 {
 
-constexpr int kGemmBN = 256;
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
 
 // amdgpu_waves_per_eu(1, 1): one wavefront per SIMD is the design point (256 accumulator

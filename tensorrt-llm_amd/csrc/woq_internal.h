@@ -104,6 +104,33 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits)
     return pl;
 }
 
+// W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K)
+inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
+{
+    GemmPlan pl;
+    pl.skinny = false;
+    pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
+    int const k_tiles = (k + 127) / 128;
+    long const tiles = (long) ((m + pl.rt * 16 - 1) / (pl.rt * 16)) * ((n + 255) / 256);
+    pl.k_splits = 1;
+    if (tiles < 160 && k_tiles >= 8)
+    {
+        long splits = 320 / tiles;
+        if (splits > k_tiles / 4)
+            splits = k_tiles / 4;
+        if (splits > 1)
+            pl.k_splits = (int) splits;
+    }
+    if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
+    {
+        int const v = std::atoi(f);
+        if (v >= 1 && v <= k_tiles)
+            pl.k_splits = v;
+    }
+    pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+    return pl;
+}
+
 // largest M the streaming kernel is instantiated for
 constexpr int kStreamMaxM = 128;
 

@@ -60,6 +60,19 @@ def test_w4a8_zeros_and_bias(pkg, oracle, dev):
     assert oracle.max_rel_err(out, ref) < TOL
 
 
+@pytest.mark.parametrize("M,K,N", [(17, 4096, 256), (100, 2048, 272), (128, 1024, 512), (200, 2048, 1040), (520, 512, 256)])
+def test_w4a8_tile_heights_and_split_k(pkg, oracle, dev, M, K, N):
+    """64 / 128 / 256-row tiles, K split across workgroups (with a shorter last slice) and not,
+    N off the 256-column tile, zeros and bias (bias is added by the finish pass when K is split)."""
+    prob = oracle.make_w4a8_problem(M, K, N, seed=M + N, out_dtype="bf16")
+    rng = np.random.default_rng(M)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+    for z in (None, zeros):
+        out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=bias)
+        assert oracle.max_rel_err(out, ref) < TOL, (M, K, N, z is not None)
+
+
 def test_w4a8_identity_recovers_e4m3_weight(pkg, oracle, dev):
     """Identity activation (exact in e4m3) returns the e4m3-rounded dequantized weight times alpha."""
     K, N = 256, 128
