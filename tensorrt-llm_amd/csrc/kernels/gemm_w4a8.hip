@@ -8,10 +8,15 @@
 //
 // Same skeleton as the 16-bit prefill kernel (gemm_kernel.h): output tile 16*RT rows x 256
 // columns, 4 wavefronts side by side along N with 64 columns each; packed weights go global ->
-// registers (the tile layout is the B-operand layout of v_mfma_f32_16x16x32_fp8_fp8 as well: 8
-// consecutive k per lane) and are dequantized once per workgroup; the activation tile is DMA-ed
+// registers and are dequantized once per workgroup; the activation tile is DMA-ed
 // global -> LDS, double-buffered; the requests of the next step and the conversions are spread
 // between the MFMAs; skinny problems split K through the float32 partial buffer.
+// The matrix instruction is the CDNA4 v_mfma_f32_16x16x128_f8f6f4 (e4m3 x e4m3): one instruction
+// covers a whole 128-deep tile row, twice the rate of the 16x16x32 fp8 form and a quarter of its
+// issue slots.  A lane supplies 32 k-values of its row / column; which 32 is free as long as A
+// and B agree, so lane (kg, c) keeps the tile layout's own order - its 8 weights of slab 0, of
+// slab 1, ... (k = 32 j + 8 kg + e) - and reads the matching four 8-byte pieces of its activation
+// row from LDS.
 // An fp8 activation fragment is half the size of a 16-bit one, so LDS holds fragment PAIRS: 16
 // rows x 64 k = 1 KiB, written by one DMA instruction (lane 4r+q fetches row r's 16-byte chunk
 // q ^ (r>>2): quads read 64 contiguous bytes, the XOR spreads an MFMA lane group over the banks).
@@ -21,29 +26,55 @@
 namespace woq
 {
 
-// elements 4h .. 4h+3 of slab dword `w` -> 4 e4m3 bytes, element order preserved
-__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, float z)
+// elements 4h .. 4h+3 of slab dword `w` -> 4 e4m3 bytes, element order preserved.  `old` is the
+// register's previous content (both halves are overwritten; converting in place saves a move).
+// With zero-points the weight is fma(q, s, z) on the two's-complement nibble.  Without them
+// q * s = fma(u, s, -8 s) on the stored nibble u = q + 8: -8 s is exact, so this is the same
+// single rounding, and u comes out of a byte-to-float conversion with no sign extension.
+template <bool ZERO>
+__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t old, uint32_t w, int h, float s, float z)
 {
-    uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
     float v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
+    if constexpr (ZERO)
     {
-        int const e = 4 * h + i;
-        int const slot = (e & 1) ? 4 + (e >> 1) : (e >> 1);
-        int const q = (int) (t << (28 - 4 * slot)) >> 28;
-        v[i] = clamp_e4m3(__builtin_fmaf((float) q, s, z));
+        uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            int const e = 4 * h + i;
+            int const slot = (e & 1) ? 4 + (e >> 1) : (e >> 1);
+            int const q = (int) (t << (28 - 4 * slot)) >> 28;
+            v[i] = clamp_e4m3(__builtin_fmaf((float) q, s, z));
+        }
     }
-    uint32_t r = 0;
-    r = (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) r, false);
-    r = (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], (int) r, true);
-    return r;
+    else
+    {
+        // nibble slot n holds element 2n (n < 4) or 2(n-4)+1: byte b of the even-nibble word is
+        // slot 2b, of the odd-nibble word slot 2b+1
+        uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+        // opaque, so that the byte-to-float conversions below read the masked words (the compiler
+        // would otherwise fold each into a separate 4-bit field extract of w)
+        asm volatile("" : "+v"(even), "+v"(odd));
+        float const m8s = -8.f * s;
+        float const u0 = (float) ((even >> (8 * h)) & 0xFF);        // element 4h:   slot 2h
+        float const u1 = (float) ((even >> (8 * h + 16)) & 0xFF);   // element 4h+1: slot 4+2h
+        float const u2 = (float) ((odd >> (8 * h)) & 0xFF);         // element 4h+2: slot 2h+1
+        float const u3 = (float) ((odd >> (8 * h + 16)) & 0xFF);    // element 4h+3: slot 5+2h
+        v[0] = clamp_e4m3(__builtin_fmaf(u0, s, m8s));
+        v[1] = clamp_e4m3(__builtin_fmaf(u1, s, m8s));
+        v[2] = clamp_e4m3(__builtin_fmaf(u2, s, m8s));
+        v[3] = clamp_e4m3(__builtin_fmaf(u3, s, m8s));
+    }
+    old = (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) old, false);
+    return (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], (int) old, true);
 }
 
-// c += a x b (8 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)
-__device__ __forceinline__ void mma_fp8_acc(u32x2 a, u32x2 b, f32x4& c)
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+
+// c += a x b (32 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)
+__device__ __forceinline__ void mma_fp8_acc(u32x8 a, u32x8 b, f32x4& c)
 {
-    asm volatile("v_mfma_f32_16x16x32_fp8_fp8 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
 template <int ODT, bool ZERO, int RT, bool SPLITK>
@@ -145,77 +176,87 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
     };
 
-    // ---- one tile row of MFMAs, hand-pipelined like the 16-bit kernel: iteration (j, rt) issues
-    // the fragment read A_AHEAD iterations away, its share of the next step's requests and of the
-    // next slab's conversions (8 half-operands of 4 weights per slab), and the 4 MFMAs of row tile rt.
-    constexpr int A_AHEAD = 3;
-    u32x2 b_cur[NS], b_nxt[NS];
-    auto half_operand = [&](BStage const& st, int j, int ci) -> uint32_t
+    // ---- one step = one tile row of K = RT iterations of 4 MFMAs (one per strip).  Iteration rt
+    // issues the activation reads of the row tile A_AHEAD ahead, its share of the memory requests
+    // (packed weights of step kt+2, A tile of step kt+1) and of the conversions that build the B
+    // operands of step kt+1 (32 half-operands of 4 weights), then the 4 MFMAs of row tile rt.
+    constexpr int A_AHEAD = 2;
+    auto slab_at = [](int pos) { return ((pos & 1) << 1) | (pos >> 1); }; // its own inverse
+    auto half_operand = [&](uint32_t old, BStage const& st, int ci) -> uint32_t
     {
-        int const s = ci / 2, h = ci % 2;
+        // ci = (strip, slab, half) -> dword 2*slab + half of that strip's operand
+        int const s = ci / 8, j = (ci / 2) % 4, h = ci % 2;
         float const sc = EH::from_bits(st.s[s]);
         float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
-        return dequant4_fp8(st.w[s][j], h, sc, zr);
+        return dequant4_fp8<ZERO>(old, st.w[s][j], h, sc, zr);
     };
 
-    auto compute = [&](auto const* buf, BStage const& st, BStage& st_next, auto* buf_next, int kt_next)
+    auto compute = [&](auto const* buf, u32x8 const (&b_use)[NS], u32x8 (&b_make)[NS], BStage const& st_conv,
+                       BStage& st_req, auto* buf_next, int kt)
     {
         char const* a_base = reinterpret_cast<char const*>(buf);
-        constexpr int ITERS = SLABS * RT;
-        uint32_t const next_base = dma_base(kt_next);
-        auto a_read = [&](int it) -> u32x2
+        uint32_t const next_base = dma_base(kt + 1);
+        auto a_read = [&](int rt) -> u32x8
         {
-            int const rt = it % RT, j = it / RT;
-            return *reinterpret_cast<u32x2 const*>(a_base + (rt * 2 + j / 2) * 1024 + a_lane_off[j % 2]);
-        };
-        u32x2 a_ring[A_AHEAD + 1];
+            // operand position pos holds slab slab_at(pos) = 0, 2, 1, 3: the two pieces that sit
+            // 1 KiB apart in LDS (same half of the two fragment pairs) come from one two-address read
+            u32x8 a;
 #pragma unroll
-        for (int i = 0; i < A_AHEAD; ++i)
+            for (int pos = 0; pos < SLABS; ++pos)
+            {
+                int const j = slab_at(pos);
+                u32x2 const v = *reinterpret_cast<u32x2 const*>(a_base + (rt * 2 + j / 2) * 1024 + a_lane_off[j % 2]);
+                a[2 * pos] = v[0];
+                a[2 * pos + 1] = v[1];
+            }
+            return a;
+        };
+        u32x8 a_ring[A_AHEAD + 1];
+#pragma unroll
+        for (int i = 0; i < A_AHEAD && i < RT; ++i)
             a_ring[i] = a_read(i);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < SLABS; ++j)
+        for (int rt = 0; rt < RT; ++rt)
         {
+            // the A-tile DMAs first, the weight-side requests of step kt+2 after them: the barrier
+            // that ends the step then waits for the DMAs only (vector-memory operations retire in
+            // order) and leaves the weight loads, which travel from HBM, a whole further step
+            constexpr int DMA_WINDOW = RT / 2 > 0 ? RT / 2 : 1;
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
+            for (int q = 0; q < DMA_OPS; ++q)
+                if (q * DMA_WINDOW / DMA_OPS == rt)
+                    dma_piece(buf_next, next_base, q);
+            constexpr int FETCH_FIRST = RT / 2, FETCH_WINDOW = RT - RT / 2 - 1 > 0 ? RT - RT / 2 - 1 : 1;
+#pragma unroll
+            for (int q = 0; q < FETCH_OPS; ++q)
+                if (FETCH_FIRST + q * FETCH_WINDOW / FETCH_OPS == rt)
+                    fetch_piece(st_req, kt + 2, q);
+            if (rt + A_AHEAD < RT)
+                a_ring[(rt + A_AHEAD) % (A_AHEAD + 1)] = a_read(rt + A_AHEAD);
+#pragma unroll
+            for (int ci = rt * 32 / RT; ci < (rt + 1) * 32 / RT; ++ci)
             {
-                int const it = j * RT + rt;
-                constexpr int FETCH_WINDOW = (SLABS - 1) * RT < FETCH_OPS ? (SLABS - 1) * RT : FETCH_OPS;
-#pragma unroll
-                for (int q = 0; q < FETCH_OPS; ++q)
-                    if (q * FETCH_WINDOW / FETCH_OPS == it)
-                        fetch_piece(st_next, kt_next, q);
-                constexpr int DMA_WINDOW = ITERS * 5 / 8 > 0 ? ITERS * 5 / 8 : 1;
-#pragma unroll
-                for (int q = 0; q < DMA_OPS; ++q)
-                    if (q * DMA_WINDOW / DMA_OPS == it)
-                        dma_piece(buf_next, next_base, q);
-                if (it + A_AHEAD < ITERS)
-                    a_ring[(it + A_AHEAD) % (A_AHEAD + 1)] = a_read(it + A_AHEAD);
-                // 8 half-operands per slab over RT iterations
-#pragma unroll
-                for (int ci = 0; ci < 8; ++ci)
-                    if (ci * RT / 8 == rt)
-                    {
-                        if (j + 1 < SLABS)
-                            b_nxt[ci / 2][ci % 2] = half_operand(st, j + 1, ci);
-                        else
-                            b_nxt[ci / 2][ci % 2] = half_operand(st_next, 0, ci);
-                    }
-                u32x2 const a_cur = a_ring[it % (A_AHEAD + 1)];
-#pragma unroll
-                for (int s = 0; s < NS; ++s)
-                    mma_fp8_acc(a_cur, b_cur[s], acc[rt][s]);
-                __builtin_amdgcn_sched_barrier(0);
+                int const idx = slab_at((ci / 2) % 4) * 2 + ci % 2; // slab (ci/2)%4 sits at that operand position
+                b_make[ci / 8][idx] = half_operand(b_make[ci / 8][idx], st_conv, ci);
             }
+            u32x8 const a_cur = a_ring[rt % (A_AHEAD + 1)];
 #pragma unroll
             for (int s = 0; s < NS; ++s)
-                b_cur[s] = b_nxt[s];
+                mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // ---- main loop: two tile rows per iteration so that each LDS buffer is a distinct object ---
+    // ---- main loop: two steps per iteration so that LDS buffers, operand sets and weight stages
+    // are distinct objects.  Step kt multiplies with operand set kt%2 (converted during step kt-1
+    // from weight stage kt%2), converts set (kt+1)%2 from stage (kt+1)%2 and refills stage kt%2
+    // with the packed weights of step kt+2.
     BStage st0, st1;
+    u32x8 b0[NS], b1[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        b0[s] = b1[s] = u32x8{0, 0, 0, 0, 0, 0, 0, 0};
     {
         uint32_t const base = dma_base(kt_begin);
 #pragma unroll
@@ -226,14 +267,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int i = 0; i < FETCH_OPS; ++i)
         fetch_piece(st0, kt_begin, i);
 #pragma unroll
-    for (int ci = 0; ci < 8; ++ci)
-        b_cur[ci / 2][ci % 2] = half_operand(st0, 0, ci);
+    for (int i = 0; i < FETCH_OPS; ++i)
+        fetch_piece(st1, kt_begin + 1, i);
+#pragma unroll
+    for (int ci = 0; ci < 32; ++ci)
+    {
+        int const idx = slab_at((ci / 2) % 4) * 2 + ci % 2;
+        b0[ci / 8][idx] = half_operand(b0[ci / 8][idx], st0, ci);
+    }
     for (int kt = kt_begin; kt < KT; kt += 2)
     {
-        __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
-        compute(a_buf0, st0, st1, a_buf1, kt + 1);
-        __syncthreads();
-        compute(a_buf1, st1, st0, a_buf0, kt + 2); // past the end of K both operands read as zeros
+        // A(kt) has landed for every wavefront (at most the FETCH_OPS weight-side loads issued
+        // after its DMAs are still outstanding); everyone is done reading the other buffer
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FETCH_OPS) : "memory");
+        compute(a_buf0, b0, b1, st1, st0, a_buf1, kt);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FETCH_OPS) : "memory");
+        compute(a_buf1, b1, b0, st0, st1, a_buf0, kt + 1); // past the end of K both operands read as zeros
     }
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
