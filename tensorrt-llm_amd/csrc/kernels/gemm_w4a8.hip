@@ -26,47 +26,37 @@
 namespace woq
 {
 
-// elements 4h .. 4h+3 of slab dword `w` -> 4 e4m3 bytes, element order preserved.  `old` is the
-// register's previous content (both halves are overwritten; converting in place saves a move).
+// elements 4h+2p, 4h+2p+1 of slab dword `w` -> 2 e4m3 bytes in 16-bit word p of `old` (a dword of
+// the B operand holds elements 4h .. 4h+3 in order; the other word is kept).
 // With zero-points the weight is fma(q, s, z) on the two's-complement nibble.  Without them
 // q * s = fma(u, s, -8 s) on the stored nibble u = q + 8: -8 s is exact, so this is the same
 // single rounding, and u comes out of a byte-to-float conversion with no sign extension.
 template <bool ZERO>
-__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t old, uint32_t w, int h, float s, float z)
+__device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h, int p, float s, float z)
 {
-    float v[4];
+    float v0, v1;
+    int const e0 = 4 * h + 2 * p; // even element: nibble slot e0/2; the odd one after it: slot 4 + e0/2
     if constexpr (ZERO)
     {
         uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-        {
-            int const e = 4 * h + i;
-            int const slot = (e & 1) ? 4 + (e >> 1) : (e >> 1);
-            int const q = (int) (t << (28 - 4 * slot)) >> 28;
-            v[i] = clamp_e4m3(__builtin_fmaf((float) q, s, z));
-        }
+        int const q0 = (int) (t << (28 - 4 * (e0 / 2))) >> 28;
+        int const q1 = (int) (t << (12 - 4 * (e0 / 2))) >> 28;
+        v0 = clamp_e4m3(__builtin_fmaf((float) q0, s, z));
+        v1 = clamp_e4m3(__builtin_fmaf((float) q1, s, z));
     }
     else
     {
-        // nibble slot n holds element 2n (n < 4) or 2(n-4)+1: byte b of the even-nibble word is
-        // slot 2b, of the odd-nibble word slot 2b+1
-        uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
-        // opaque, so that the byte-to-float conversions below read the masked words (the compiler
-        // would otherwise fold each into a separate 4-bit field extract of w)
-        asm volatile("" : "+v"(even), "+v"(odd));
+        // slots e0/2 and 4 + e0/2 are bytes h and h+2 of the even-nibble word (p = 0) or of the
+        // odd-nibble word (p = 1).  The masked word is made opaque so that the byte-to-float
+        // conversions read it (the compiler would otherwise extract each 4-bit field from w).
+        uint32_t m = (p == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
+        asm volatile("" : "+v"(m));
         float const m8s = -8.f * s;
-        float const u0 = (float) ((even >> (8 * h)) & 0xFF);        // element 4h:   slot 2h
-        float const u1 = (float) ((even >> (8 * h + 16)) & 0xFF);   // element 4h+1: slot 4+2h
-        float const u2 = (float) ((odd >> (8 * h)) & 0xFF);         // element 4h+2: slot 2h+1
-        float const u3 = (float) ((odd >> (8 * h + 16)) & 0xFF);    // element 4h+3: slot 5+2h
-        v[0] = clamp_e4m3(__builtin_fmaf(u0, s, m8s));
-        v[1] = clamp_e4m3(__builtin_fmaf(u1, s, m8s));
-        v[2] = clamp_e4m3(__builtin_fmaf(u2, s, m8s));
-        v[3] = clamp_e4m3(__builtin_fmaf(u3, s, m8s));
+        v0 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h)) & 0xFF), s, m8s));
+        v1 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h + 16)) & 0xFF), s, m8s));
     }
-    old = (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) old, false);
-    return (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], (int) old, true);
+    return p == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, false)
+                  : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, true);
 }
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
@@ -182,14 +172,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // operands of step kt+1 (32 half-operands of 4 weights), then the 4 MFMAs of row tile rt.
     constexpr int A_AHEAD = 2;
     auto slab_at = [](int pos) { return ((pos & 1) << 1) | (pos >> 1); }; // its own inverse
-    auto half_operand = [&](uint32_t old, BStage const& st, int ci) -> uint32_t
+    // conversion unit cu = (strip, slab, half, pair): 2 weights -> 16 bits of the operand set
+    auto convert_unit = [&](u32x8 (&b)[NS], BStage const& st, int cu)
     {
-        // ci = (strip, slab, half) -> dword 2*slab + half of that strip's operand
-        int const s = ci / 8, j = (ci / 2) % 4, h = ci % 2;
+        int const s = cu / 16, j = (cu / 4) % 4, h = (cu / 2) % 2, pr = cu % 2;
+        int const idx = slab_at(j) * 2 + h; // slab j sits at operand position slab_at(j)
         float const sc = EH::from_bits(st.s[s]);
         float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
-        return dequant4_fp8<ZERO>(old, st.w[s][j], h, sc, zr);
+        b[s][idx] = dequant2_fp8<ZERO>(b[s][idx], st.w[s][j], h, pr, sc, zr);
     };
+    constexpr int UNITS = NS * SLABS * 4; // 64 per step
 
     auto compute = [&](auto const* buf, u32x8 const (&b_use)[NS], u32x8 (&b_make)[NS], BStage const& st_conv,
                        BStage& st_req, auto* buf_next, int kt)
@@ -234,17 +226,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     fetch_piece(st_req, kt + 2, q);
             if (rt + A_AHEAD < RT)
                 a_ring[(rt + A_AHEAD) % (A_AHEAD + 1)] = a_read(rt + A_AHEAD);
-#pragma unroll
-            for (int ci = rt * 32 / RT; ci < (rt + 1) * 32 / RT; ++ci)
-            {
-                int const idx = slab_at((ci / 2) % 4) * 2 + ci % 2; // slab (ci/2)%4 sits at that operand position
-                b_make[ci / 8][idx] = half_operand(b_make[ci / 8][idx], st_conv, ci);
-            }
             u32x8 const a_cur = a_ring[rt % (A_AHEAD + 1)];
+            // one MFMA, then its share of the conversions: a wavefront issues in order, so the
+            // VALU work has to sit between the matrix instructions to run under them
 #pragma unroll
             for (int s = 0; s < NS; ++s)
+            {
                 mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
-            __builtin_amdgcn_sched_barrier(0);
+                constexpr int PER = UNITS / (RT * NS);
+#pragma unroll
+                for (int cu = (rt * NS + s) * PER; cu < (rt * NS + s + 1) * PER; ++cu)
+                    convert_unit(b_make, st_conv, cu);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
 
@@ -270,11 +264,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int i = 0; i < FETCH_OPS; ++i)
         fetch_piece(st1, kt_begin + 1, i);
 #pragma unroll
-    for (int ci = 0; ci < 32; ++ci)
-    {
-        int const idx = slab_at((ci / 2) % 4) * 2 + ci % 2;
-        b0[ci / 8][idx] = half_operand(b0[ci / 8][idx], st0, ci);
-    }
+    for (int cu = 0; cu < UNITS; ++cu)
+        convert_unit(b0, st0, cu);
     for (int kt = kt_begin; kt < KT; kt += 2)
     {
         // A(kt) has landed for every wavefront (at most the FETCH_OPS weight-side loads issued
