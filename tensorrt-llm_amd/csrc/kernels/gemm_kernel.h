@@ -255,27 +255,65 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 if (it + A_AHEAD < ITERS)
                     a_ring[(it + A_AHEAD) % (A_AHEAD + 1)]
                         = *reinterpret_cast<u32x4 const*>(a_addr(it + A_AHEAD));
-#pragma unroll
-                for (int ci = rt * (16 / RT); ci < (rt + 1) * (16 / RT); ++ci)
+                // The conversion of this iteration's 16/RT operand registers runs in 4 stages, one
+                // after each of the 4 MFMAs: a wavefront issues in order, so VALU work only runs
+                // under the matrix core when it sits between the matrix instructions.
+                constexpr int CONV = 16 / RT;
+                int q0[CONV], q1[CONV];
+                float t0[CONV], t1[CONV], sc[CONV], zr[CONV];
+                auto conv_stage = [&](int stage)
                 {
-                    int const s = ci / 4, pr = ci % 4;
-                    float sc, zr;
-                    if (j + 1 < SLABS)
+#pragma unroll
+                    for (int x = 0; x < CONV; ++x)
                     {
-                        scale_of(st, s, (j + 1) / SEG_SLABS, sc, zr);
-                        b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st.w[s], j + 1, pr, sc, zr);
+                        int const ci = rt * CONV + x, s = ci / 4, pr = ci % 4;
+                        bool const same_step = j + 1 < SLABS;
+                        BStage const& src = same_step ? st : st_next;
+                        int const jn = same_step ? j + 1 : 0;
+                        if (stage == 0)
+                        {
+                            scale_of(src, s, jn / SEG_SLABS, sc[x], zr[x]);
+                            if constexpr (BITS == 4)
+                                int4_pair(src.w[s][jn] ^ 0x88888888u, pr, q0[x], q1[x]);
+                            else
+                                int8_pair(src.w[s][2 * jn], src.w[s][2 * jn + 1], pr, q0[x], q1[x]);
+                        }
+                        else if (stage == 1)
+                        {
+                            t0[x] = (float) q0[x];
+                            t1[x] = (float) q1[x];
+                        }
+                        else if (stage == 2)
+                        {
+                            if constexpr (DT == WOQ_BF16)
+                            {
+                                t0[x] = __builtin_fmaf(t0[x], sc[x], zr[x]);
+                                t1[x] = __builtin_fmaf(t1[x], sc[x], zr[x]);
+                            }
+                        }
+                        else
+                        {
+                            if constexpr (DT == WOQ_BF16)
+                                b_nxt[s][pr] = E::pack(t0[x], t1[x]);
+                            else
+                            {
+                                // half-precision FMA (single rounding), as dequant_pair<WOQ_FP16>
+                                f16x2 const q2 = {(_Float16) t0[x], (_Float16) t1[x]};
+                                f16x2 const s2 = {(_Float16) sc[x], (_Float16) sc[x]};
+                                f16x2 const z2 = {(_Float16) zr[x], (_Float16) zr[x]};
+                                b_nxt[s][pr] = bit_cast<uint32_t>(__builtin_elementwise_fma(q2, s2, z2));
+                            }
+                        }
                     }
-                    else
-                    {
-                        scale_of(st_next, s, 0, sc, zr);
-                        b_nxt[s][pr] = dequant_operand_reg<DT, BITS>(st_next.w[s], 0, pr, sc, zr);
-                    }
-                }
+                };
                 u32x4 const a_cur = a_ring[it % (A_AHEAD + 1)];
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
+                {
                     E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
-                __builtin_amdgcn_sched_barrier(0);
+                    conv_stage(s);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
 #pragma unroll
             for (int s = 0; s < NS; ++s)
