@@ -31,6 +31,7 @@ SHAPES_8B = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 2867
 GROUP = 128
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_FP8_PEAK_TFLOPS = 5000.0
 CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # calibrated with a 256 MiB copy (profiles/stream_gemv_gate_up_m1_hbm_traffic.md); counters cannot
@@ -186,6 +187,43 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
         return dict(error=str(e)[:200])
 
 
+def w4a8_setup(pkg, dev, m, k, n, seed=4000):
+    """W4A8 operands of the benchmark's kind: int4 symmetric g128 weights (same gfx950 layout),
+    fp16 group scales, activations already smoothed and cast to e4m3, alpha in the epilogue."""
+    F = pkg.functional
+    layer = make_layer(pkg, dev, k, n, seed)
+    scales = layer["scales"].to(torch.float16)
+    g = torch.Generator(device=dev).manual_seed(seed + 1)
+    act = (torch.randn((m, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+
+    def run():
+        F.woq_matmul_raw(act, None, layer["weight"], scales, None, None, n=n, k=k, group_size=GROUP,
+                         quant_algo=F.FP8_ALPHA, alpha=0.5, out_dtype=torch.bfloat16, out=out)
+    return run
+
+
+def bench_w4a8(pkg, dev, m=4096, reps=5):
+    """W4A8 (fp8 MFMA) on gate_up: TFLOP/s at M = 4096 against the 5 PFLOP/s dense fp8 peak."""
+    try:
+        name, k, n = SHAPES_8B[2]
+        run = w4a8_setup(pkg, dev, m, k, n)
+        run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / reps
+        tf = 2.0 * m * n * k / sec / 1e12
+        return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
+                    frac_of_fp8_peak=round(tf / MFMA_FP8_PEAK_TFLOPS, 4))
+    except Exception as e:
+        return dict(error=str(e)[:200])
+
+
 def run_for_counters(pkg, dev, mode, reps=20):
     """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
     dominant kernel (gate_up GEMV, rotating weight copies); `gemm<M>` launches the GEMM regime on
@@ -202,6 +240,14 @@ def run_for_counters(pkg, dev, mode, reps=20):
                           "launches": reps}))
         return
     _, k, n = SHAPES_8B[2]
+    if mode == "w4a8_4096":
+        run = w4a8_setup(pkg, dev, 4096, k, n)
+        for r in range(reps):
+            run()
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": mode, "kernel": "W4A8 GEMM on gate_up K=4096 N=28672 M=4096",
+                          "flop_per_launch": 2.0 * 4096 * n * k, "launches": reps}))
+        return
     if mode.startswith("gemm"):
         m = int(mode[4:] or 4096)
         layer = make_layer(pkg, dev, k, n, 2002)
@@ -231,7 +277,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128"], default="bench",
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096"], default="bench",
                     help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -266,6 +312,7 @@ def main():
     }
     if not args.no_gemm:
         line["gemm"] = bench_gemm(pkg, dev)
+        line["w4a8"] = bench_w4a8(pkg, dev)
     if not args.no_cpu:
         line["cpu_baseline"] = bench_cpu_baseline(r["layers"], r["acts"])
     print(json.dumps(line))
