@@ -10,11 +10,10 @@
 //     produces P = sum a * (q + OFFSET) and, against an all-ones operand, S = sum a;
 //   * the scale is applied to the float32 sums, once per group and output element:
 //     acc += s * P + (z - OFFSET * s) * S.
-// Output tile 64 rows x 256 columns; 4 wavefronts side by side along N, each 64 x 64, one
-// workgroup per CU.  Everything a step needs is requested DEPTH steps ahead (a skinny problem is
-// bound by memory latency unless tens of KiB per CU are in flight): the activation tile and the
-// group scales go global -> LDS by DMA, packed weights go straight to the registers of the lane
-// that feeds them to the matrix core.
+// Output tile 64 rows x 256 columns; 8 wavefronts side by side along N, each 64 rows x 32
+// columns, two per SIMD.  Everything a step needs is requested DEPTH steps ahead: the activation
+// tile and the group scales go global -> LDS by DMA, packed weights go straight to the registers
+// of the lane that feeds them to the matrix core.
 #pragma once
 
 #include "gemm_common.h"
@@ -24,7 +23,7 @@ namespace woq
 
 constexpr int kSkinnyBM = 64;
 constexpr int kSkinnyBN = 256;
-constexpr int kSkinnyWaves = 8; // two per SIMD: one wavefront's VALU and memory instructions run under the other's MFMAs
+constexpr int kSkinnyWaves = 8; // two per SIMD: while one waits at the barrier or for LDS the other issues
 
 template <int DT, int BITS, int GROUP, bool ZERO, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 4)>
 __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) skinny_kernel(GemmParams p)
