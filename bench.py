@@ -181,8 +181,20 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
         torch.cuda.synchronize()
         sec = e0.elapsed_time(e1) * 1e-3 / reps
         tf = 2.0 * m * n * k / sec / 1e12
+        # context, not a baseline: the vendor library's plain bf16 x bf16 GEMM (no dequantize) of the
+        # same shape on this box, through torch.matmul
+        dense = torch.randn((k, n), generator=g, device=dev).to(torch.bfloat16)
+        torch.matmul(act, dense, out=out)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            torch.matmul(act, dense, out=out)
+        e1.record()
+        torch.cuda.synchronize()
+        lib_tf = 2.0 * m * n * k / (e0.elapsed_time(e1) * 1e-3 / reps) / 1e12
         return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
-                    frac_of_bf16_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
+                    frac_of_bf16_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                    library_dense_bf16_gemm_tflops=round(lib_tf, 1))
     except Exception as e:  # the decode line is still valid without the prefill extra
         return dict(error=str(e)[:200])
 
