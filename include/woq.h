@@ -143,8 +143,8 @@ int woq_matmul_check(const woq_matmul_args* args);
  * plugin's own m*k*sizeof(half) smoothing buffer (weightOnlyGroupwiseQuantMatmulPlugin.cpp:377-379). */
 size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype);
 
-/* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k < 2^26), GEMM otherwise and always for
- * W4A8 - crossovers measured on MI355X.  Counterpart of the tactic choice
+/* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, < 2^26 for int8
+ * weights), GEMM otherwise and always for W4A8 - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 

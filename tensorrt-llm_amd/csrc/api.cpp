@@ -208,11 +208,14 @@ extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
         return WOQ_REGIME_GEMM;
     // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed; with two row
-    // tiles the streaming kernel still wins on small matrices (it needs no split-K passes), and
-    // from 33 rows on the MFMA GEMM kernels (64-row deferred-scale tiles first) are faster.
+    // tiles the streaming kernel still wins on small matrices (it needs no split-K passes): up to
+    // 2^24 int4 weights, where the MFMA kernel has 32-row tiles, and below 2^26 int8 weights,
+    // where its tiles have 64 rows.  From 33 rows on the MFMA GEMM kernels are faster.
     if (m <= 16)
         return WOQ_REGIME_STREAM;
-    if (m <= 32 && (int64_t) n * k < ((int64_t) 1 << 26))
+    int64_t const weights = (int64_t) n * k;
+    bool const small = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? weights < ((int64_t) 1 << 26) : weights <= ((int64_t) 1 << 24);
+    if (m <= 32 && small)
         return WOQ_REGIME_STREAM;
     return WOQ_REGIME_GEMM;
 }

@@ -10,8 +10,8 @@
 //     produces P = sum a * (q + OFFSET) and, against an all-ones operand, S = sum a;
 //   * the scale is applied to the float32 sums, once per group and output element:
 //     acc += s * P + (z - OFFSET * s) * S.
-// Output tile 64 rows x 256 columns; 8 wavefronts side by side along N, each 64 rows x 32
-// columns, two per SIMD.  Everything a step needs is requested DEPTH steps ahead: the activation
+// Output tile 64 (32 for M <= 32, int4) rows x 256 columns; 8 wavefronts side by side along N,
+// each 32 columns wide, two per SIMD.  Everything a step needs is requested DEPTH steps ahead: the activation
 // tile and the group scales go global -> LDS by DMA, packed weights go straight to the registers
 // of the lane that feeds them to the matrix core.
 #pragma once
@@ -21,17 +21,16 @@
 namespace woq
 {
 
-constexpr int kSkinnyBM = 64;
 constexpr int kSkinnyBN = 256;
 constexpr int kSkinnyWaves = 8; // two per SIMD: while one waits at the barrier or for LDS the other issues
 
-template <int DT, int BITS, int GROUP, bool ZERO, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 4)>
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 4)>
 __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) skinny_kernel(GemmParams p)
 {
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
-    constexpr int RT = kSkinnyBM / 16;                           // row tiles per wavefront
+    constexpr int kSkinnyBM = RT * 16;                           // RT row tiles per wavefront
     constexpr int NS = kSkinnyBN / 16 / kSkinnyWaves;            // strips (16 columns) per wavefront
     constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
     constexpr int SEGS = TK / SEG;
@@ -199,7 +198,9 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 sc[s][seg], part[s & 1][seg][rt][r], __builtin_fmaf(cc[s][seg], part_s[seg][rt][r], acc[rt][s][r]));
         }
     };
-    constexpr int UNITS = SEGS * 16; // per strip
+    constexpr int UNITS = SEGS * RT * 4; // per strip
+    constexpr int PER_B = 4 / RT;        // registers of the next B operand expanded per mini-block
+    static_assert(RT == 2 || RT == 4, "row tiles per wavefront");
 
     // register pr (elements 2pr, 2pr+1) of the B operand of slab j of a lane's 16 packed bytes
     auto expand_reg = [&](u32x4 const& w, int j, int pr) -> uint32_t
@@ -266,7 +267,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 else
                     acc_s[rt] = E::mma(a[rt][j], ones, acc_s[rt]);
                 if (j == SLABS - 1)
-                    b_cur[rt] = expand_reg(st.w[0], 0, rt);
+                {
+#pragma unroll
+                    for (int x = rt * PER_B; x < (rt + 1) * PER_B; ++x)
+                        b_cur[x] = expand_reg(st.w[0], 0, x);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
 
@@ -284,11 +289,15 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                             a[rt][j], b_cur, j % SEG_SLABS == 0 ? zero4 : part[s & 1][j / SEG_SLABS][rt]);
                     else
                         acc[rt][s] = E::mma(a[rt][j], b_cur, acc[rt][s]);
-                    // one register of the next B operand (RT == 4 registers per operand)
-                    if (j + 1 < SLABS)
-                        b_nxt[rt] = expand_reg(st.w[s], j + 1, rt);
-                    else if (s + 1 < NS)
-                        b_nxt[rt] = expand_reg(st.w[s + 1], 0, rt);
+                    // this mini-block's share of the next B operand (4 registers per operand)
+#pragma unroll
+                    for (int x = rt * PER_B; x < (rt + 1) * PER_B; ++x)
+                    {
+                        if (j + 1 < SLABS)
+                            b_nxt[x] = expand_reg(st.w[s], j + 1, x);
+                        else if (s + 1 < NS)
+                            b_nxt[x] = expand_reg(st.w[s + 1], 0, x);
+                    }
                     if (s > 0)
                     {
                         constexpr int BLOCKS = SLABS * RT; // mini-blocks per strip
@@ -304,7 +313,6 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             }
         }
     };
-    static_assert(RT == 4, "one register of the next B operand per row-tile mini-block");
 
     // ---- main loop --------------------------------------------------------------------------
     // Step kt: wait until everything this wavefront requested for step kt has landed, barrier (now
@@ -374,8 +382,8 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     }
 }
 
-template <int DT, int BITS, int GROUP, bool ZERO>
-int launch_skinny_variant(GemmParams const& gp, hipStream_t stream)
+template <int DT, int BITS, int GROUP, bool ZERO, int RT>
+int launch_skinny_rt(GemmParams const& gp, hipStream_t stream)
 {
     int const total = gp.tiles_m * gp.tiles_n;
     dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(kSkinnyWaves * 64), block256(256);
@@ -384,16 +392,27 @@ int launch_skinny_variant(GemmParams const& gp, hipStream_t stream)
         size_t const count = (size_t) gp.m * gp.n;
         hipLaunchKernelGGL((gemm_zero_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block256, 0, stream,
             gp.partial, count);
-        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, true>), grid, block, 0, stream, gp);
+        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, RT, true>), grid, block, 0, stream, gp);
         hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count + 255) / 256)), block256, 0, stream, gp.out,
             gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
     }
     else
-        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, false>), grid, block, 0, stream, gp);
+        hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "skinny gemm kernel launch failed: %s", hipGetErrorString(err));
     return WOQ_OK;
+}
+
+template <int DT, int BITS, int GROUP, bool ZERO>
+int launch_skinny_variant(GemmParams const& gp, int rt, hipStream_t stream)
+{
+    if constexpr (BITS == 4)
+    {
+        if (rt == 2)
+            return launch_skinny_rt<DT, BITS, GROUP, ZERO, 2>(gp, stream);
+    }
+    return launch_skinny_rt<DT, BITS, GROUP, ZERO, 4>(gp, stream);
 }
 
 template <int DT, int BITS>
@@ -413,7 +432,8 @@ int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stre
     gp.k = p.k;
     gp.k_tiles = (p.k + TK - 1) / TK;
     gp.strips = p.n / kTileN;
-    gp.tiles_m = (p.m + kSkinnyBM - 1) / kSkinnyBM;
+    int const rt = (BITS == 4 && plan.rt == 2) ? 2 : 4;
+    gp.tiles_m = (p.m + rt * 16 - 1) / (rt * 16);
     gp.tiles_n = (p.n + kSkinnyBN - 1) / kSkinnyBN;
     gp.k_splits = plan.k_splits;
     gp.tiles_per_split = (gp.k_tiles + plan.k_splits - 1) / plan.k_splits;
@@ -424,13 +444,13 @@ int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stre
     bool const zero = p.zeros != nullptr;
     switch (p.group_size)
     {
-    case 0: return launch_skinny_variant<DT, BITS, 0, false>(gp, s);
+    case 0: return launch_skinny_variant<DT, BITS, 0, false>(gp, rt, s);
     case 64:
-        return zero ? launch_skinny_variant<DT, BITS, 64, true>(gp, s)
-                    : launch_skinny_variant<DT, BITS, 64, false>(gp, s);
+        return zero ? launch_skinny_variant<DT, BITS, 64, true>(gp, rt, s)
+                    : launch_skinny_variant<DT, BITS, 64, false>(gp, rt, s);
     case 128:
-        return zero ? launch_skinny_variant<DT, BITS, 128, true>(gp, s)
-                    : launch_skinny_variant<DT, BITS, 128, false>(gp, s);
+        return zero ? launch_skinny_variant<DT, BITS, 128, true>(gp, rt, s)
+                    : launch_skinny_variant<DT, BITS, 128, false>(gp, rt, s);
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 }

@@ -62,7 +62,7 @@ int launch_dequant(void* out, void const* weight, void const* scales, void const
 struct GemmPlan
 {
     bool skinny;  // deferred-scale 64-row kernel instead of the exact-dequantize prefill kernel
-    int rt;       // prefill kernel: row tiles per wavefront (tile rows = 16 * rt)
+    int rt;       // row tiles per wavefront (tile rows = 16 * rt)
     int k_splits;
     size_t ws_bytes;
 };
@@ -80,8 +80,11 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits)
     GemmPlan pl;
     char const* e = std::getenv("WOQ_GEMM_KERNEL");
     pl.skinny = e ? !std::strcmp(e, "skinny") : prefer_skinny(m, n);
-    pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
-    int const tile_rows = pl.skinny ? 64 : pl.rt * 16;
+    if (pl.skinny)
+        pl.rt = (m <= 32 && bits == 4) ? 2 : 4; // 32- or 64-row tiles
+    else
+        pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
+    int const tile_rows = pl.rt * 16;
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
     long const tiles = (long) ((m + tile_rows - 1) / tile_rows) * ((n + 255) / 256);

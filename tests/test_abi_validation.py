@@ -99,6 +99,9 @@ def test_regime_table(pkg):
     # two row tiles: streaming on small matrices only
     assert sel(32, 28672, 4096, 0) == L.REGIME_GEMM
     assert sel(16, 28672, 4096, 0) == L.REGIME_STREAM
+    assert sel(32, 6144, 4096, 0) == L.REGIME_GEMM  # int4: 32-row MFMA tiles win above 2^24 weights
+    assert sel(32, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM
+    assert sel(32, 8192, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
     assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
 
 

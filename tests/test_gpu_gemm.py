@@ -31,6 +31,17 @@ def test_gemm_variants(pkg, oracle, dev, dtype, bits, group, zero):
     assert err < TOL, err
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("group,zero", [(128, False), (128, True), (64, False), (64, True), (0, False)])
+@pytest.mark.parametrize("M", [5, 17, 32])
+def test_gemm_at_most_32_rows(pkg, oracle, dev, dtype, group, zero, M):
+    """M <= 32 with int4 weights: the deferred-scale kernel switches to 32-row tiles; K long enough
+    that it also splits K, N ragged."""
+    p = random_problem(oracle, M, 2048, 784, 4, group, dtype, zero=zero, bias=True, seed=M + group)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    assert err < TOL, err
+
+
 @pytest.mark.parametrize("M", [1, 16, 129, 256, 257, 512, 1000])
 def test_gemm_m_edges(pkg, oracle, dev, M):
     """Row counts around the 256-row tile, including the decode sizes forced onto this kernel."""
