@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Benchmark of the weight-only quantized matmul hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py --mode sweep --sweep decode8b|prefill8b|llama70b|w4a8   (tables of the other
+                                                   benchmark configurations, one JSON line per case)
 
 Workload (the configuration the headline metric is quoted on): W4A16, group 128, bf16
 activations/scales/zeros, M = 1 — the four linear layers of one Llama-3-8B decoder layer
@@ -28,6 +30,7 @@ from __graft_entry__ import import_package
 
 METRIC = "W4A16 g128 GEMM: HBM GB/s at M=1, TFLOP/s at M=4096 (Llama-3-8B shapes)"
 SHAPES_8B = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+SHAPES_70B = [("qkv", 8192, 10240), ("o_proj", 8192, 8192), ("gate_up", 8192, 57344), ("down", 28672, 8192)]
 GROUP = 128
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
@@ -45,12 +48,12 @@ def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
     return k * n * bits // 8 + sz + m * k * act_bytes + m * n * 2
 
 
-def make_layer(pkg, dev, k, n, seed):
+def make_layer(pkg, dev, k, n, seed, group=GROUP):
     """Synthetic tensors of the benchmark configuration: W ~ N(0, 0.02) quantized to uint4 with
-    group 128 along K (asymmetric min/max), bf16 scales, bf16 zeros = (8 - zp) * scale."""
+    group 128 (or 64) along K (asymmetric min/max), bf16 scales, bf16 zeros = (8 - zp) * scale."""
     g = torch.Generator(device=dev).manual_seed(seed)
     w = torch.randn((k, n), generator=g, device=dev, dtype=torch.float32) * 0.02
-    wg = w.view(k // GROUP, GROUP, n)
+    wg = w.view(k // group, group, n)
     mx, mn = wg.amax(1), wg.amin(1)
     scale = ((mx - mn).clamp_min(1e-8) / 15.0).to(torch.bfloat16)
     sf = scale.float()
@@ -60,7 +63,23 @@ def make_layer(pkg, dev, k, n, seed):
     zeros = ((8.0 - zp) * sf).to(torch.bfloat16)
     packed = ((q[:, 0::2] & 0xF) | (q[:, 1::2] << 4)).to(torch.int8).cpu().contiguous()
     wq = pkg.ops.preprocess_weights_for_mixed_gemm(packed, torch.quint4x2, torch.bfloat16).to(dev)
-    return dict(k=k, n=n, q=q, weight=wq, scales=scale.contiguous(), zeros=zeros.contiguous())
+    return dict(k=k, n=n, q=q, weight=wq, scales=scale.contiguous(), zeros=zeros.contiguous(), group=group,
+                algo=pkg.functional.ZERO)
+
+
+def make_layer_int8(pkg, dev, k, n, seed):
+    """W8A16 per-channel: W ~ N(0, 0.02) quantized symmetrically to int8, one bf16 scale per column."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    w = torch.randn((k, n), generator=g, device=dev, dtype=torch.float32) * 0.02
+    scale = (w.abs().amax(0) / 127.0).to(torch.bfloat16)
+    q = torch.round(w / scale.float()).clamp(-128, 127).to(torch.int8)
+    wq = pkg.ops.preprocess_weights_for_mixed_gemm(q.cpu().contiguous(), torch.int8, torch.bfloat16).to(dev)
+    return dict(k=k, n=n, q=q, weight=wq, scales=scale.contiguous(), zeros=None, group=0,
+                algo=pkg.functional.INT8_WEIGHT)
+
+
+def copies_beyond_cache(weight_bytes, factor=2):
+    return max(2, -(-factor * CACHE_BYTES // weight_bytes))
 
 
 def rotated_copies(layer, copies):
@@ -72,7 +91,8 @@ def rotated_copies(layer, copies):
         c = dict(layer)
         c["weight"] = tiles.roll(977 * r + 1, 0).contiguous().view_as(layer["weight"])
         c["scales"] = layer["scales"].roll(r, 0).contiguous()
-        c["zeros"] = layer["zeros"].roll(r, 0).contiguous()
+        if layer["zeros"] is not None:
+            c["zeros"] = layer["zeros"].roll(r, 0).contiguous()
         out.append(c)
     return out
 
@@ -80,7 +100,8 @@ def rotated_copies(layer, copies):
 def launch(pkg, act, layer, out, regime=0):
     F = pkg.functional
     F.woq_matmul_raw(act, None, layer["weight"], layer["scales"], layer["zeros"], None, n=layer["n"], k=layer["k"],
-                     group_size=GROUP, quant_algo=F.ZERO, out_dtype=torch.bfloat16, out=out, regime=regime)
+                     group_size=layer["group"], quant_algo=layer["algo"], out_dtype=torch.bfloat16, out=out,
+                     regime=regime)
 
 
 def time_graph(fn_body, launches):
@@ -107,15 +128,17 @@ def time_graph(fn_body, launches):
 def bench_decode(pkg, dev, steps, warmup, m=1):
     per_step_bytes = sum(algorithmic_bytes(m, k, n) for _, k, n in SHAPES_8B)
     weight_bytes = sum(k * n // 2 for _, k, n in SHAPES_8B)
-    copies = max(2, -(-3 * CACHE_BYTES // weight_bytes))  # >= 3x the cache
-    layers = [rotated_copies(make_layer(pkg, dev, k, n, 2000 + i), copies) for i, (_, k, n) in enumerate(SHAPES_8B)]
+    copies = copies_beyond_cache(weight_bytes, 3)  # the step's own rotation: >= 3x the cache
+    # each shape is also timed alone, so each gets enough copies to exceed the cache by itself
+    layers = [rotated_copies(make_layer(pkg, dev, k, n, 2000 + i), max(copies, copies_beyond_cache(k * n // 2)))
+              for i, (_, k, n) in enumerate(SHAPES_8B)]
     g = torch.Generator(device=dev).manual_seed(2999)
     acts = {k: torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16) for k in (4096, 14336)}
     outs = [torch.empty((m, n), dtype=torch.bfloat16, device=dev) for _, _, n in SHAPES_8B]
 
     def step(s):
         for i, (_, k, _) in enumerate(SHAPES_8B):
-            launch(pkg, acts[k], layers[i][s % copies], outs[i])
+            launch(pkg, acts[k], layers[i][s % len(layers[i])], outs[i])
 
     for s in range(warmup):
         step(s)
@@ -127,13 +150,13 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
     _, gk, gn = SHAPES_8B[gi]
     reps = max(steps, 50)
     _, dom_s, dom_launches = time_graph(
-        lambda: [launch(pkg, acts[gk], layers[gi][r % copies], outs[gi]) for r in range(reps)], reps)
+        lambda: [launch(pkg, acts[gk], layers[gi][r % len(layers[gi])], outs[gi]) for r in range(reps)], reps)
     dom_bytes = algorithmic_bytes(m, gk, gn)
     dom_dur = dom_s / dom_launches
     per_shape = {}
     for i, (name, k, n) in enumerate(SHAPES_8B):
-        _, s_s, s_l = time_graph(lambda: [launch(pkg, acts[k], layers[i][r % copies], outs[i]) for r in range(reps)],
-                                 reps)
+        _, s_s, s_l = time_graph(
+            lambda: [launch(pkg, acts[k], layers[i][r % len(layers[i])], outs[i]) for r in range(reps)], reps)
         per_shape[name] = dict(us=round(s_s / s_l * 1e6, 3), gbs=round(algorithmic_bytes(m, k, n) / (s_s / s_l) / 1e9, 1))
     return dict(host_s=host_s, ev_s=ev_s, per_step_bytes=per_step_bytes, copies=copies, dom_dur=dom_dur,
                 dom_bytes=dom_bytes, per_shape=per_shape, layers=layers, acts=acts)
@@ -199,18 +222,20 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
         return dict(error=str(e)[:200])
 
 
-def w4a8_setup(pkg, dev, m, k, n, seed=4000):
+def w4a8_setup(pkg, dev, m, k, n, seed=4000, copies=1, layers=None):
     """W4A8 operands of the benchmark's kind: int4 symmetric g128 weights (same gfx950 layout),
-    fp16 group scales, activations already smoothed and cast to e4m3, alpha in the epilogue."""
+    fp16 group scales, activations already smoothed and cast to e4m3, alpha in the epilogue.
+    run(r) uses weight copy r % copies."""
     F = pkg.functional
-    layer = make_layer(pkg, dev, k, n, seed)
-    scales = layer["scales"].to(torch.float16)
+    layers = layers or rotated_copies(make_layer(pkg, dev, k, n, seed), copies)
+    scales = [l["scales"].to(torch.float16) for l in layers]
     g = torch.Generator(device=dev).manual_seed(seed + 1)
     act = (torch.randn((m, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
     out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
 
-    def run():
-        F.woq_matmul_raw(act, None, layer["weight"], scales, None, None, n=n, k=k, group_size=GROUP,
+    def run(r=0):
+        c = r % copies
+        F.woq_matmul_raw(act, None, layers[c]["weight"], scales[c], None, None, n=n, k=k, group_size=GROUP,
                          quant_algo=F.FP8_ALPHA, alpha=0.5, out_dtype=torch.bfloat16, out=out)
     return run
 
@@ -282,6 +307,54 @@ def run_for_counters(pkg, dev, mode, reps=20):
                       "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n), "launches": reps}))
 
 
+SWEEPS = {
+    # name: (shapes, kinds, row counts); kind = ("w4a16", group) | ("w8a16", 0) | ("w4a8", 128)
+    "decode8b": (SHAPES_8B, [("w4a16", 128)], [1, 4, 8, 16]),
+    "prefill8b": (SHAPES_8B, [("w4a16", 128), ("w8a16", 0)], [512, 2048, 4096, 8192]),
+    "llama70b": (SHAPES_70B, [("w4a16", 128), ("w4a16", 64)], [1, 2, 4, 8, 16, 32, 64, 128, 256]),
+    "w4a8": (SHAPES_70B, [("w4a8", 128)], [1, 16, 256, 4096]),
+}
+
+
+def run_sweep(pkg, dev, which):
+    """The benchmark's other configurations: one JSON line per (kind, shape, M) with the launch time,
+    algorithmic GB/s and TFLOP/s.  Launches rotate over weight copies exceeding the last-level cache
+    while M <= 256 (weight traffic matters there); all launches of a case replay from one HIP graph."""
+    shapes, kinds, ms = SWEEPS[which]
+    for kind, group in kinds:
+        for name, k, n in shapes:
+            bits = 8 if kind == "w8a16" else 4
+            copies = min(copies_beyond_cache(k * n * bits // 8), 64) if min(ms) <= 256 else 1
+            if kind == "w8a16":
+                layers = rotated_copies(make_layer_int8(pkg, dev, k, n, 5000), copies)
+            else:
+                layers = rotated_copies(make_layer(pkg, dev, k, n, 5000, group), copies)
+            for m in ms:
+                reps = 40 if m <= 256 else 5
+                if kind == "w4a8":
+                    runner = w4a8_setup(pkg, dev, m, k, n, 5000, copies, layers)
+                    body = lambda: [runner(r) for r in range(reps)]
+                    runner(0)
+                    act_bytes = 1
+                else:
+                    act = torch.randn((m, k), device=dev).to(torch.bfloat16)
+                    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+                    body = lambda: [launch(pkg, act, layers[r % copies], out) for r in range(reps)]
+                    launch(pkg, act, layers[0], out)
+                    act_bytes = 2
+                torch.cuda.synchronize()
+                _, sec, launches = time_graph(body, reps)
+                us = sec / launches * 1e6
+                n_sz = 1 if kind != "w4a16" else 2  # scales only, or scales + zeros
+                by = algorithmic_bytes(m, k, n, bits, group, n_sz, act_bytes)
+                print(json.dumps({"sweep": which, "kind": kind, "group": group, "shape": name, "k": k, "n": n, "m": m,
+                                  "us": round(us, 2), "gbs": round(by / us / 1e3, 1),
+                                  "tflops": round(2.0 * m * n * k / us / 1e6, 1), "weight_copies": copies}),
+                      flush=True)
+            layers = None
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -289,8 +362,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096"], default="bench",
-                    help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs")
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "sweep"],
+                    default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
+                                          "sweep: the table named by --sweep")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS), default="llama70b")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "
@@ -301,6 +376,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.mode == "sweep":
+        run_sweep(pkg, dev, args.sweep)
+        return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode)
         return

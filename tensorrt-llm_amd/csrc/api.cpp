@@ -79,7 +79,8 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
     {
         int const rows = m < 16 ? m : 16;
         size_t const act_lds = (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
-        if (act_lds <= 96 * 1024)
+        // beyond ~48 KiB the staging area costs more in resident workgroups than the L2 reads it saves
+        if (act_lds <= 48 * 1024)
         {
             if (strips >= 1024)
                 return {4, 8, 2, 1};
@@ -258,9 +259,10 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     // the split-K region does not (large m does not split), so take its maximum over the row
     // counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
-    // the plan changes at multiples of the 64-row tile; 160 or more tiles never split
+    // the plan changes at multiples of the 64-row tile; kEnoughTiles or more tiles never split,
+    // which even one column of the tallest (256-row) tiles reaches at 256 * kEnoughTiles rows
     size_t split = split_bytes(m, n, k, quant_algo);
-    for (int mm = 64; mm < m && mm <= 64 * 160; mm += 64)
+    for (int mm = 64; mm < m && mm <= 256 * (int) kEnoughTiles; mm += 64)
     {
         size_t const b = split_bytes(mm, n, k, quant_algo);
         split = b > split ? b : split;

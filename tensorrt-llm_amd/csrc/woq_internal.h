@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <initializer_list>
 
 #include "../../include/woq.h"
 
@@ -67,36 +68,79 @@ struct GemmPlan
     size_t ws_bytes;
 };
 
-// The deferred-scale 64-row kernel is preferred up to 256 rows, and up to 512 rows when N is narrow
-// (few column panels: the 256-row tiles of the prefill kernel would leave most CUs idle).
-inline bool prefer_skinny(int m, int n)
+// Output tiles (of 16*rt rows x 256 columns) a problem has.
+inline long gemm_tiles(int m, int n, int rt)
 {
-    return m <= 256 || (m <= 512 && n <= 8192);
+    return (long) ((m + rt * 16 - 1) / (rt * 16)) * ((n + 255) / 256);
 }
 
-// Environment overrides for experiments: WOQ_GEMM_KERNEL=exact|skinny, WOQ_GEMM_SPLITS=<n>
+// A launch fills the 256 CUs from about this many workgroups on; below it K is split.
+constexpr long kEnoughTiles = 160;
+
+// Tile height of the exact-dequantize kernels above 256 rows: the tallest tile amortises the
+// dequantize best (measured per-CU rates 1 : 0.87 : 0.58 for 256 : 128 : 64 rows), but only when
+// its tiles still fill the chip, and a partly filled last row tile is wasted matrix-core work.
+// Returns 0 when neither 256- nor 128-row tiles fill the chip.
+inline int tall_tile_rt(int m, int n)
+{
+    int best = 0;
+    double best_cost = 0;
+    for (int rt : {16, 8})
+    {
+        if (gemm_tiles(m, n, rt) < kEnoughTiles)
+            continue;
+        int const padded = (m + rt * 16 - 1) / (rt * 16) * (rt * 16);
+        double const cost = padded / (rt == 16 ? 1.0 : 0.87);
+        if (!best || cost < best_cost)
+            best = rt, best_cost = cost;
+    }
+    return best;
+}
+
+inline int auto_k_splits(long tiles, int k_tiles)
+{
+    if (tiles >= kEnoughTiles || k_tiles < 8)
+        return 1;
+    long splits = 2 * kEnoughTiles / tiles;
+    if (splits > k_tiles / 4)
+        splits = k_tiles / 4;
+    return splits > 1 ? (int) splits : 1;
+}
+
+// Kernel, tile height and K split of a 16-bit GEMM-regime problem, from measured crossovers:
+//   * up to 256 rows the deferred-scale kernel (32-row tiles for int4 up to 32 rows, else 64-row);
+//   * above, the exact-dequantize kernel with the tallest tile that fills the chip; when neither
+//     256- nor 128-row tiles do, 128-row tiles with K split if K is long (>= 8192: the float32
+//     partial sums are then small next to the weight work), else the deferred-scale kernel.
+// Environment overrides for experiments: WOQ_GEMM_KERNEL=exact|skinny, WOQ_GEMM_RT=4|8|16 (exact
+// kernel), WOQ_GEMM_SPLITS=<n>
 inline GemmPlan plan_gemm(int m, int n, int k, int bits)
 {
     GemmPlan pl;
-    char const* e = std::getenv("WOQ_GEMM_KERNEL");
-    pl.skinny = e ? !std::strcmp(e, "skinny") : prefer_skinny(m, n);
-    if (pl.skinny)
-        pl.rt = (m <= 32 && bits == 4) ? 2 : 4; // 32- or 64-row tiles
+    int exact_rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
+    if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
+        pl.skinny = !std::strcmp(e, "skinny");
+    else if (m <= 256)
+        pl.skinny = true;
+    else if (int const rt = tall_tile_rt(m, n))
+        pl.skinny = false, exact_rt = rt;
+    else if (k >= 8192 && gemm_tiles(m, n, 8) >= 96)
+        pl.skinny = false, exact_rt = 8;
     else
-        pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
-    int const tile_rows = pl.rt * 16;
+        pl.skinny = true;
+    if (pl.skinny)
+        pl.rt = (m <= 32 && bits == 4) ? 2 : 4;
+    else
+        pl.rt = exact_rt;
+    if (char const* r = std::getenv("WOQ_GEMM_RT"))
+    {
+        int const v = std::atoi(r);
+        if (!pl.skinny && (v == 4 || v == 8 || v == 16))
+            pl.rt = v;
+    }
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
-    long const tiles = (long) ((m + tile_rows - 1) / tile_rows) * ((n + 255) / 256);
-    pl.k_splits = 1;
-    if (tiles < 160 && k_tiles >= 8)
-    {
-        long splits = 320 / tiles;
-        if (splits > k_tiles / 4)
-            splits = k_tiles / 4;
-        if (splits > 1)
-            pl.k_splits = (int) splits;
-    }
+    pl.k_splits = auto_k_splits(gemm_tiles(m, n, pl.rt), k_tiles);
     if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
     {
         int const v = std::atoi(f);
@@ -107,23 +151,36 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits)
     return pl;
 }
 
-// W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K)
+// W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K).
+// Tile height above 128 rows, from measured crossovers (per-CU rates 1 : 0.65 : 0.37 for
+// 256 : 128 : 64 rows): 256 rows when those tiles fill the chip or K is very long (splitting K is
+// then cheap); else 128 rows when they fill it, or nearly do and K is long; else 64 rows.
+inline int w4a8_rt(int m, int n, int k)
+{
+    if (m <= 64)
+        return 4;
+    if (m <= 128)
+        return 8;
+    if (gemm_tiles(m, n, 16) >= kEnoughTiles || k >= 16384)
+        return 16;
+    if (gemm_tiles(m, n, 8) >= kEnoughTiles || (gemm_tiles(m, n, 8) >= 96 && k >= 8192))
+        return 8;
+    return 4;
+}
+
 inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
 {
     GemmPlan pl;
     pl.skinny = false;
-    pl.rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
-    int const k_tiles = (k + 127) / 128;
-    long const tiles = (long) ((m + pl.rt * 16 - 1) / (pl.rt * 16)) * ((n + 255) / 256);
-    pl.k_splits = 1;
-    if (tiles < 160 && k_tiles >= 8)
+    pl.rt = w4a8_rt(m, n, k);
+    if (char const* r = std::getenv("WOQ_GEMM_RT"))
     {
-        long splits = 320 / tiles;
-        if (splits > k_tiles / 4)
-            splits = k_tiles / 4;
-        if (splits > 1)
-            pl.k_splits = (int) splits;
+        int const v = std::atoi(r);
+        if (v == 4 || v == 8 || v == 16)
+            pl.rt = v;
     }
+    int const k_tiles = (k + 127) / 128;
+    pl.k_splits = auto_k_splits(gemm_tiles(m, n, pl.rt), k_tiles);
     if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
     {
         int const v = std::atoi(f);

@@ -72,8 +72,8 @@ def test_workspace_rule(pkg):
     lib = L.lib
     algo = L.ALGO_PRE_QUANT_SCALE
     # the split-K partial buffer: none at m=4096 x n=4096 itself (256 tiles fill the chip), but the
-    # size covers every smaller m too, and up to 2304 rows (9 x 16 tiles) still split
-    split = 2304 * 4096 * 4
+    # size covers every smaller m too, and up to 1152 rows (9 x 16 tiles of 128 rows) still split
+    split = 1152 * 4096 * 4
     assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2 + split
     assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == split
     assert lib.woq_workspace_bytes(64, 4096, 8192, 0, L.BF16) == 64 * 4096 * 4
@@ -81,6 +81,15 @@ def test_workspace_rule(pkg):
     # never shrinks as m grows
     sizes = [lib.woq_workspace_bytes(m, 1024, 4096, algo, L.FP16) for m in range(1, 3000, 37)]
     assert sizes == sorted(sizes)
+    # the size asked for m rows is enough for every call with fewer rows, whatever plan those get
+    for n, k, algo2, act in [(4096, 8192, 0, L.BF16), (256, 8192, 0, L.BF16), (1024, 4096, L.ALGO_INT8_WEIGHT, L.BF16),
+                             (6144, 4096, L.ALGO_FP8_ALPHA, L.FP8_E4M3)]:
+        group = 0 if algo2 & L.ALGO_INT8_WEIGHT else 128
+        bound = lib.woq_workspace_bytes(30000, n, k, algo2, act)
+        for m in list(range(1, 2600, 13)) + list(range(2600, 30000, 511)):
+            rc, msg = status(pkg, m=m, n=n, k=k, quant_algo=algo2, act_dtype=act, group_size=group, regime=2,
+                             workspace=0x9000, workspace_bytes=bound)
+            assert rc == 0, (m, n, k, msg)
     # GEMM regime with smoothing needs the workspace; the streaming regime fuses it
     rc, msg = status(pkg, m=512, pre_quant_scale=0x5000, quant_algo=algo)
     assert rc == -4 and "workspace" in msg
