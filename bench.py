@@ -196,25 +196,17 @@ def bench_gemm(pkg, dev, m=4096, reps=5):
         out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
         launch(pkg, act, layer, out)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            launch(pkg, act, layer, out)
-        e1.record()
-        torch.cuda.synchronize()
-        sec = e0.elapsed_time(e1) * 1e-3 / reps
+        # same timing as the decode part: the launches replay from a HIP graph, once untimed first
+        _, sec, launches = time_graph(lambda: [launch(pkg, act, layer, out) for _ in range(reps)], reps)
+        sec /= launches
         tf = 2.0 * m * n * k / sec / 1e12
         # context, not a baseline: the vendor library's plain bf16 x bf16 GEMM (no dequantize) of the
         # same shape on this box, through torch.matmul
         dense = torch.randn((k, n), generator=g, device=dev).to(torch.bfloat16)
         torch.matmul(act, dense, out=out)
         torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            torch.matmul(act, dense, out=out)
-        e1.record()
-        torch.cuda.synchronize()
-        lib_tf = 2.0 * m * n * k / (e0.elapsed_time(e1) * 1e-3 / reps) / 1e12
+        _, lib_sec, _ = time_graph(lambda: [torch.matmul(act, dense, out=out) for _ in range(reps)], reps)
+        lib_tf = 2.0 * m * n * k / (lib_sec / reps) / 1e12
         return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
                     frac_of_bf16_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                     library_dense_bf16_gemm_tflops=round(lib_tf, 1))
@@ -247,13 +239,8 @@ def bench_w4a8(pkg, dev, m=4096, reps=5):
         run = w4a8_setup(pkg, dev, m, k, n)
         run()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            run()
-        e1.record()
-        torch.cuda.synchronize()
-        sec = e0.elapsed_time(e1) * 1e-3 / reps
+        _, sec, launches = time_graph(lambda: [run() for _ in range(reps)], reps)
+        sec /= launches
         tf = 2.0 * m * n * k / sec / 1e12
         return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
                     frac_of_fp8_peak=round(tf / MFMA_FP8_PEAK_TFLOPS, 4))

@@ -73,7 +73,7 @@ typedef enum woq_quant_type
 typedef enum woq_regime
 {
     WOQ_REGIME_AUTO = 0,
-    WOQ_REGIME_STREAM = 1, /* weight-streaming kernel (decode GEMV, accepts m <= 128) */
+    WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 16) */
     WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMMs: 64-row deferred-scale tiles for skinny m, 256-row prefill
                               tiles, the fp8 kernel for W4A8; may split K through the workspace */
 } woq_regime;
@@ -144,7 +144,7 @@ int woq_matmul_check(const woq_matmul_args* args);
 size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype);
 
 /* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, < 2^26 for int8
- * weights), GEMM otherwise and always for W4A8 - crossovers measured on MI355X.  Counterpart of the tactic choice
+ * weights; m <= 16 for W4A8), GEMM otherwise - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 

@@ -28,6 +28,7 @@ int launch_skinny_BF16_8(MatmulProblem const& p, GemmPlan const& plan, void* str
 int launch_skinny_FP16_4(MatmulProblem const& p, GemmPlan const& plan, void* stream);
 int launch_skinny_FP16_8(MatmulProblem const& p, GemmPlan const& plan, void* stream);
 int launch_gemm_w4a8(MatmulProblem const& p, void* stream);
+int launch_stream_w4a8(MatmulProblem const& p, void* stream);
 
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
@@ -48,11 +49,11 @@ int launch_gemm(MatmulProblem const& p, void* stream)
 
 int launch_stream(MatmulProblem const& p, void* stream)
 {
+    if (p.w4a8)
+        return launch_stream_w4a8(p, stream);
     if (p.m > kStreamMaxM)
         return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
             p.m);
-    if (p.w4a8)
-        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 runs on the fp8 MFMA GEMM kernel only");
     if (p.out_dtype == WOQ_BF16)
         return p.bits == 4 ? launch_stream_BF16_4(p, stream) : launch_stream_BF16_8(p, stream);
     return p.bits == 4 ? launch_stream_FP16_4(p, stream) : launch_stream_FP16_8(p, stream);
@@ -206,8 +207,10 @@ using namespace woq;
 
 extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo)
 {
+    // W4A8: the streaming kernel converts every weight to e4m3 in registers and still runs at
+    // memory speed for one 16-row tile; beyond that the fp8 GEMM kernel
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
-        return WOQ_REGIME_GEMM;
+        return m <= kStreamW4a8MaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
     // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed; with two row
     // tiles the streaming kernel still wins on small matrices (it needs no split-K passes): up to
     // 2^24 int4 weights, where the MFMA kernel has 32-row tiles, and below 2^26 int8 weights,
@@ -277,14 +280,16 @@ extern "C" int woq_matmul_check(const woq_matmul_args* args)
     if (int rc = validate(args, p))
         return rc;
     int const regime = pick_regime(args);
-    if (regime == WOQ_REGIME_STREAM && args->m > kStreamMaxM)
-        return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
+    int const stream_max_m = p.w4a8 ? kStreamW4a8MaxM : kStreamMaxM;
+    if (regime == WOQ_REGIME_STREAM && args->m > stream_max_m)
+        return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", stream_max_m,
             args->m);
-    if (regime == WOQ_REGIME_STREAM && p.w4a8)
-        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 runs on the fp8 MFMA GEMM kernel only");
-    if (regime == WOQ_REGIME_GEMM && p.m > 0)
+    if (p.m > 0 && (regime == WOQ_REGIME_GEMM || p.w4a8))
     {
-        size_t const need = gemm_workspace_bytes(p.m, p.n, p.k, args->quant_algo);
+        // the W4A8 streaming kernel reads e4m3 activations: 16-bit ones go through the smoothing
+        // pass (and its workspace region) in either regime
+        size_t const need = regime == WOQ_REGIME_GEMM ? gemm_workspace_bytes(p.m, p.n, p.k, args->quant_algo)
+                                                      : smooth_bytes(p.m, p.k, args->quant_algo);
         if (need && (!p.workspace || p.workspace_bytes < need))
             return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
                 p.workspace ? p.workspace_bytes : (size_t) 0);
@@ -300,8 +305,9 @@ extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
     validate(args, p);
     if (p.m == 0)
         return WOQ_OK;
-    if (pick_regime(args) == WOQ_REGIME_STREAM)
-        return launch_stream(p, stream);
+    bool const streaming = pick_regime(args) == WOQ_REGIME_STREAM;
+    if (streaming && !p.w4a8)
+        return launch_stream(p, stream); // smoothing is fused into the 16-bit streaming kernel
     if (p.pre_quant_scale)
     {
         // smoothing pass into the workspace, then the GEMM reads the smoothed activations
@@ -316,7 +322,7 @@ extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
         p.workspace = static_cast<char*>(p.workspace) + used;
         p.workspace_bytes -= used;
     }
-    return launch_gemm(p, stream);
+    return streaming ? launch_stream(p, stream) : launch_gemm(p, stream);
 }
 
 extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,

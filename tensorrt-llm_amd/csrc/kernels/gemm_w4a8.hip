@@ -20,52 +20,11 @@
 // An fp8 activation fragment is half the size of a 16-bit one, so LDS holds fragment PAIRS: 16
 // rows x 64 k = 1 KiB, written by one DMA instruction (lane 4r+q fetches row r's 16-byte chunk
 // q ^ (r>>2): quads read 64 contiguous bytes, the XOR spreads an MFMA lane group over the banks).
-#include "dequant_math.h"
 #include "gemm_common.h"
+#include "w4a8_common.h"
 
 namespace woq
 {
-
-// elements 4h+2p, 4h+2p+1 of slab dword `w` -> 2 e4m3 bytes in 16-bit word p of `old` (a dword of
-// the B operand holds elements 4h .. 4h+3 in order; the other word is kept).
-// With zero-points the weight is fma(q, s, z) on the two's-complement nibble.  Without them
-// q * s = fma(u, s, -8 s) on the stored nibble u = q + 8: -8 s is exact, so this is the same
-// single rounding, and u comes out of a byte-to-float conversion with no sign extension.
-template <bool ZERO>
-__device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h, int p, float s, float z)
-{
-    float v0, v1;
-    int const e0 = 4 * h + 2 * p; // even element: nibble slot e0/2; the odd one after it: slot 4 + e0/2
-    if constexpr (ZERO)
-    {
-        uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
-        int const q0 = (int) (t << (28 - 4 * (e0 / 2))) >> 28;
-        int const q1 = (int) (t << (12 - 4 * (e0 / 2))) >> 28;
-        v0 = clamp_e4m3(__builtin_fmaf((float) q0, s, z));
-        v1 = clamp_e4m3(__builtin_fmaf((float) q1, s, z));
-    }
-    else
-    {
-        // slots e0/2 and 4 + e0/2 are bytes h and h+2 of the even-nibble word (p = 0) or of the
-        // odd-nibble word (p = 1).  The masked word is made opaque so that the byte-to-float
-        // conversions read it (the compiler would otherwise extract each 4-bit field from w).
-        uint32_t m = (p == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
-        asm volatile("" : "+v"(m));
-        float const m8s = -8.f * s;
-        v0 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h)) & 0xFF), s, m8s));
-        v1 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h + 16)) & 0xFF), s, m8s));
-    }
-    return p == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, false)
-                  : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, true);
-}
-
-typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
-
-// c += a x b (32 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)
-__device__ __forceinline__ void mma_fp8_acc(u32x8 a, u32x8 b, f32x4& c)
-{
-    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
 
 template <int ODT, bool ZERO, int RT, bool SPLITK>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_w4a8_kernel(GemmParams p)

@@ -1,0 +1,281 @@
+// W4A8 decode: weight-streaming kernel for fp8 (e4m3) activations and int4 weights, M <= 16.
+//
+// Same semantics as the W4A8 GEMM (gemm_w4a8.hip; the reference's fpA_intB runner instantiated
+// for __nv_fp8_e4m3 x uint4, selected by weightOnlyGroupwiseQuantMatmulPlugin.cpp:203-276): every
+// weight is dequantized with its fp16 group scale (and zero) and rounded to e4m3, the matrix core
+// accumulates fp8 x fp8 products in float32, the epilogue applies alpha and the bias.  Because the
+// rounding to e4m3 is part of the result, the scale cannot be deferred to the group sums as in the
+// 16-bit streaming kernel: each weight is converted exactly, in registers, by the lane that loaded
+// it (about 3 VALU instructions per weight - still under what HBM delivers).
+//
+// Same skeleton as the 16-bit streaming kernel (stream_kernel.h): a workgroup owns NS strips of 16
+// columns, its wavefronts split K (tile row kt goes to wave kt % WAVES, PF tile rows in flight
+// each) and are reduced through LDS in a fixed order.  One v_mfma_f32_16x16x128_f8f6f4 covers a
+// whole 128-deep tile row: lane (kg, c) supplies, for output column c (B) and activation row c (A),
+// the 32 k-values 32 j + 8 kg + e (j = 0..3 slabs, e = 0..7) in that order - the tile layout's own
+// order for the weights, four 8-byte loads of its activation row for A (rows >= M fall outside the
+// buffer descriptor and read as zeros).
+#include "stream_kernel.h"
+#include "w4a8_common.h"
+
+namespace woq
+{
+
+__device__ __forceinline__ u32x2 buffer_load_x2(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int) byte_offset, 0, 0);
+}
+
+template <int ODT, bool ZERO, int NS, int WAVES, int PF>
+__global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
+{
+    using EO = Elem<ODT>;
+    using EH = Elem<WOQ_FP16>;
+    constexpr int TK = 128, SLABS = 4;
+
+    int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
+    if (group >= p.groups)
+        return; // whole workgroup leaves together
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const c = lane & 15, kg = lane >> 4;
+    int const K = p.k;
+    int const KT = p.k_tiles;
+    int const strip0 = group * NS;
+
+    f32x4 acc[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    constexpr uint32_t kPast = 0x80000000u;
+    auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K);
+    uint32_t const sz_bytes = (uint32_t) (K / TK) * (uint32_t) p.n * 2u;
+    auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
+    auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
+    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+
+    // strips past the end of N (last group only) are clamped for loads and skipped at the store
+    uint32_t wlane[NS], sc_lane[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        int const strip = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        wlane[s] = ((uint32_t) strip * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+        sc_lane[s] = (uint32_t) (strip * 16 + c) * 2u;
+    }
+    // activation row c (rows >= m start past the end of the buffer), this lane's 8 bytes of slab 0
+    uint32_t const a_lane = (uint32_t) c * (uint32_t) K + (uint32_t) kg * 8u;
+
+    struct Stage
+    {
+        u32x4 w[NS];
+        u32x2 a[SLABS];
+        uint16_t s[NS];
+        uint16_t z[NS];
+    };
+
+    auto fetch = [&](Stage& st, int kt)
+    {
+        uint32_t const past = kt < KT ? 0u : kPast; // scalar select: a tile row past K reads zeros everywhere
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            st.w[s] = buffer_load_x4(w_rsrc, (wlane[s] + (uint32_t) kt * 1024u) | past);
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+            st.a[j] = buffer_load_x2(act_rsrc, (a_lane + (uint32_t) (kt * TK + j * 32)) | past);
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + sc_lane[s]) | past;
+            st.s[s] = buffer_load_u16(sc_rsrc, off);
+            if constexpr (ZERO)
+                st.z[s] = buffer_load_u16(zr_rsrc, off);
+        }
+    };
+
+    // Saturation to +-448 is part of the conversion, but a weight cannot reach it while
+    // 8|s| + |z| stays below: one wavefront-wide test per tile row takes the clamp (a quarter of
+    // the conversion's instructions) out of the common case.
+    auto convert_and_multiply = [&](Stage const& st, i32x8 a, auto clamp_tag)
+    {
+        constexpr bool CLAMP = decltype(clamp_tag)::value;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            float const sc = EH::from_bits(st.s[s]);
+            float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
+            i32x8 b;
+#pragma unroll
+            for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    b[2 * j + h] = (int) dequant4_fp8<ZERO, CLAMP>(st.w[s][j], h, sc, zr);
+            acc[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[s], 0, 0, 0, 0, 0, 0);
+        }
+    };
+    auto compute = [&](Stage const& st)
+    {
+        i32x8 a;
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+        {
+            a[2 * j] = (int) st.a[j][0];
+            a[2 * j + 1] = (int) st.a[j][1];
+        }
+        bool may_saturate = false;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            float const bound = __builtin_fmaf(8.f, __builtin_fabsf(EH::from_bits(st.s[s])),
+                ZERO ? __builtin_fabsf(EH::from_bits(st.z[s])) : 0.f);
+            may_saturate |= !(bound <= 440.f); // also true for NaN scales
+        }
+        if (__builtin_amdgcn_ballot_w64(may_saturate) != 0)
+            convert_and_multiply(st, a, std::true_type{});
+        else
+            convert_and_multiply(st, a, std::false_type{});
+    };
+
+    // tile rows of this wavefront: kt = wave + it * WAVES.  Every load tolerates kt >= KT, so
+    // prologue and loop are unconditional and the compiler's wait counts stay exact.
+    int const n_my = (KT - wave + WAVES - 1) / WAVES;
+    Stage st[PF];
+#pragma unroll
+    for (int i = 0; i < PF; ++i)
+        fetch(st[i], wave + i * WAVES);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int it = 0; it < n_my; it += PF)
+    {
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+        {
+            if (it + i < n_my)
+                compute(st[i]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(st[i], wave + (it + i + PF) * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- cross-wavefront reduction (fixed order) and epilogue: out = T(alpha * sum + bias) ----
+    constexpr int SLOTS = NS * 4;
+    __shared__ float red[WAVES][SLOTS][64];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (kg * 4 + r < p.m)
+                red[wave][s * 4 + r][lane] = acc[s][r];
+    __syncthreads();
+
+    uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    for (int e = threadIdx.x; e < SLOTS * 64; e += WAVES * 64)
+    {
+        int const slot = e >> 6, ln = e & 63;
+        int const s = slot >> 2, r = slot & 3;
+        int const row = (ln >> 4) * 4 + r;
+        if (row >= p.m || strip0 + s >= p.strips)
+            continue;
+        float sum = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2)
+            sum += red[w2][slot][ln];
+        int const ocol = (strip0 + s) * 16 + (ln & 15);
+        float const bias = p.bias ? EO::load(p.bias, ocol) : 0.f;
+        out16[(size_t) row * p.n + ocol] = EO::store(__builtin_fmaf(p.alpha, sum, bias));
+    }
+}
+
+namespace
+{
+
+struct W4a8Shape
+{
+    int ns, waves, pf;
+};
+
+// WOQ_STREAM_SHAPE="ns,waves,pf" overrides the heuristic (for tuning sweeps)
+W4a8Shape pick_shape(int m, int strips, int k_tiles)
+{
+    if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
+    {
+        W4a8Shape sh{0, 0, 0};
+        if (std::sscanf(e, "%d,%d,%d", &sh.ns, &sh.waves, &sh.pf) == 3)
+            return sh;
+    }
+    // measured on MI355X: two strips per wavefront share the activation loads once there are
+    // enough column groups to fill the chip; narrow matrices keep one strip and 8-way split K
+    if (strips >= 2048)
+        return {2, 4, 4};
+    if (strips >= 512)
+        return k_tiles >= 128 ? W4a8Shape{2, 8, 3} : W4a8Shape{2, 8, 2};
+    if (strips >= 384 && m > 4)
+        return {2, 8, 2};
+    return {1, 8, 2};
+}
+
+template <int ODT, bool ZERO, int NS, int WAVES, int PF>
+int launch_variant(StreamParams sp, hipStream_t stream)
+{
+    sp.groups = (sp.strips + NS - 1) / NS;
+    sp.groups_per_xcd = (sp.groups + 7) / 8;
+    dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    hipLaunchKernelGGL((stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF>), grid, block, 0, stream, sp);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        return fail(WOQ_ERR_RUNTIME, "W4A8 stream kernel launch failed: %s", hipGetErrorString(err));
+    return WOQ_OK;
+}
+
+template <int ODT, bool ZERO>
+int launch_shaped(StreamParams const& sp, hipStream_t s)
+{
+    W4a8Shape const sh = pick_shape(sp.m, sp.strips, sp.k_tiles);
+#define WOQ_SHAPE(NS_, WAVES_, PF_)                                                                                    \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_)                                                            \
+        return launch_variant<ODT, ZERO, NS_, WAVES_, PF_>(sp, s);
+    WOQ_SHAPE(1, 8, 2)
+    WOQ_SHAPE(1, 16, 2)
+    WOQ_SHAPE(2, 8, 2)
+    WOQ_SHAPE(2, 8, 3)
+    WOQ_SHAPE(2, 4, 4)
+    WOQ_SHAPE(4, 8, 2)
+#undef WOQ_SHAPE
+    return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d is not instantiated", sh.ns, sh.waves,
+        sh.pf);
+}
+
+} // namespace
+
+int launch_stream_w4a8(MatmulProblem const& p, void* stream)
+{
+    if (p.m > kStreamW4a8MaxM)
+        return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the W4A8 streaming kernel covers m <= %d (got %d)",
+            kStreamW4a8MaxM, p.m);
+    if (p.act_dtype != WOQ_FP8_E4M3 || p.group_size != 128 || p.k % 128)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "W4A8 streaming kernel: e4m3 activations, group 128, k %% 128 == 0");
+    StreamParams sp;
+    sp.act = p.act;
+    sp.pqs = nullptr;
+    sp.weight = p.weight;
+    sp.scales = p.scales;
+    sp.zeros = p.zeros;
+    sp.bias = p.bias;
+    sp.out = p.out;
+    sp.alpha = p.alpha;
+    sp.m = p.m;
+    sp.n = p.n;
+    sp.k = p.k;
+    sp.k_tiles = p.k / 128;
+    sp.strips = p.n / kTileN;
+    sp.groups = sp.groups_per_xcd = 0;
+    auto s = static_cast<hipStream_t>(stream);
+    bool const zero = p.zeros != nullptr;
+    if (p.out_dtype == WOQ_BF16)
+        return zero ? launch_shaped<WOQ_BF16, true>(sp, s) : launch_shaped<WOQ_BF16, false>(sp, s);
+    return zero ? launch_shaped<WOQ_FP16, true>(sp, s) : launch_shaped<WOQ_FP16, false>(sp, s);
+}
+
+} // namespace woq

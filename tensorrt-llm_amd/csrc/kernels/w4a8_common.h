@@ -1,0 +1,91 @@
+// Pieces shared by the W4A8 kernels: the exact int4 -> e4m3 dequantize and the fp8 matrix instruction.
+#pragma once
+
+#include "dequant_math.h"
+#include "device_common.h"
+
+namespace woq
+{
+
+// elements 4h+2p, 4h+2p+1 of slab dword `w` -> 2 e4m3 bytes in 16-bit word p of `old` (a dword of
+// the B operand holds elements 4h .. 4h+3 in order; the other word is kept).
+// With zero-points the weight is fma(q, s, z) on the two's-complement nibble.  Without them
+// q * s = fma(u, s, -8 s) on the stored nibble u = q + 8: -8 s is exact, so this is the same
+// single rounding, and u comes out of a byte-to-float conversion with no sign extension.
+template <bool ZERO>
+__device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h, int p, float s, float z)
+{
+    float v0, v1;
+    int const e0 = 4 * h + 2 * p; // even element: nibble slot e0/2; the odd one after it: slot 4 + e0/2
+    if constexpr (ZERO)
+    {
+        uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
+        int const q0 = (int) (t << (28 - 4 * (e0 / 2))) >> 28;
+        int const q1 = (int) (t << (12 - 4 * (e0 / 2))) >> 28;
+        v0 = clamp_e4m3(__builtin_fmaf((float) q0, s, z));
+        v1 = clamp_e4m3(__builtin_fmaf((float) q1, s, z));
+    }
+    else
+    {
+        // slots e0/2 and 4 + e0/2 are bytes h and h+2 of the even-nibble word (p = 0) or of the
+        // odd-nibble word (p = 1).  The masked word is made opaque so that the byte-to-float
+        // conversions read it (the compiler would otherwise extract each 4-bit field from w).
+        uint32_t m = (p == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
+        asm volatile("" : "+v"(m));
+        float const m8s = -8.f * s;
+        v0 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h)) & 0xFF), s, m8s));
+        v1 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h + 16)) & 0xFF), s, m8s));
+    }
+    return p == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, false)
+                  : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, true);
+}
+
+// One dword of the B operand (elements 4h .. 4h+3 of slab dword `w`), same arithmetic.  CLAMP =
+// false leaves the saturation to +-448 out: for callers that know 8|s| + |z| stays below it.
+template <bool ZERO, bool CLAMP>
+__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, float z)
+{
+    float v[4]; // elements 4h, 4h+1, 4h+2, 4h+3: nibble slots 2h, 4+2h, 2h+1, 5+2h
+    if constexpr (ZERO)
+    {
+        uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
+        int const slot[4] = {2 * h, 4 + 2 * h, 2 * h + 1, 5 + 2 * h};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = __builtin_fmaf((float) ((int) (t << (28 - 4 * slot[i])) >> 28), s, z);
+    }
+    else
+    {
+        // even slots are the low nibbles of bytes, odd slots the high nibbles: bytes h and h+2 of
+        // the two masked words (made opaque so that the byte-to-float conversions read them)
+        uint32_t me = w & 0x0F0F0F0Fu, mo = (w >> 4) & 0x0F0F0F0Fu;
+        asm volatile("" : "+v"(me), "+v"(mo));
+        float const m8s = -8.f * s;
+        v[0] = __builtin_fmaf((float) ((me >> (8 * h)) & 0xFF), s, m8s);
+        v[1] = __builtin_fmaf((float) ((me >> (8 * h + 16)) & 0xFF), s, m8s);
+        v[2] = __builtin_fmaf((float) ((mo >> (8 * h)) & 0xFF), s, m8s);
+        v[3] = __builtin_fmaf((float) ((mo >> (8 * h + 16)) & 0xFF), s, m8s);
+    }
+    if constexpr (CLAMP)
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            v[i] = clamp_e4m3(v[i]);
+    }
+    // the first conversion overwrites a register that is dead anyway (v[0]'s), the second fills
+    // the other half of it
+    int r = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], bit_cast<int>(v[0]), false);
+    r = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], r, true);
+    return (uint32_t) r;
+}
+
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// c += a x b (32 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)
+__device__ __forceinline__ void mma_fp8_acc(u32x8 a, u32x8 b, f32x4& c)
+{
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+} // namespace woq

@@ -191,7 +191,8 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
     return pl;
 }
 
-// largest M the streaming kernel is instantiated for
+// largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;
+constexpr int kStreamW4a8MaxM = 16;
 
 } // namespace woq

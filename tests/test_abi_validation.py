@@ -111,7 +111,15 @@ def test_regime_table(pkg):
     assert sel(32, 6144, 4096, 0) == L.REGIME_GEMM  # int4: 32-row MFMA tiles win above 2^24 weights
     assert sel(32, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM
     assert sel(32, 8192, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
-    assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
+    # W4A8: streaming kernel for one 16-row tile, the fp8 GEMM above
+    assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
+    assert sel(16, 57344, 8192, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
+    assert sel(17, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
+    rc, msg = status(pkg, m=17, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, regime=1)
+    assert rc == -3 and "unsupported m" in msg
+    # 16-bit activations reach the W4A8 streaming kernel through the smoothing pass: workspace needed
+    rc, msg = status(pkg, m=4, quant_algo=L.ALGO_FP8_ALPHA | L.ALGO_PRE_QUANT_SCALE, pre_quant_scale=0x5000)
+    assert rc == -4 and "workspace" in msg
 
 
 def test_python_wrappers_refuse_cpu_tensors(pkg):

@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, direct_fp8=False):
+def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, direct_fp8=False, regime=0):
     F = pkg.functional
     w = preprocess(pkg, oracle, prob["q"], 4, torch.float8_e4m3fn).to(dev)
     scales = to_dev(prob["scales"], "fp16", dev)
@@ -23,14 +23,14 @@ def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, dire
         a8 = oracle.apply_per_channel_scale(prob["act"], prob["pre_quant_scale"], out_dtype, "fp8")
         act = torch.from_numpy(a8).to(dev).to(torch.float8_e4m3fn)
         out = F.woq_matmul_raw(act, None, w, scales, z, b, n=N, k=K, group_size=128, quant_algo=algo,
-                               alpha=prob["alpha"], out_dtype=TORCH_DT[out_dtype])
+                               alpha=prob["alpha"], out_dtype=TORCH_DT[out_dtype], regime=regime)
         ref = oracle.woq_matmul_ref(a8, prob["q"], prob["scales"], zeros, bias, None, prob["alpha"], 128, out_dtype,
                                     w4a8=True)
     else:
         algo |= F.PRE_QUANT_SCALE
         out = F.woq_matmul_raw(to_dev(prob["act"], out_dtype, dev), to_dev(prob["pre_quant_scale"], out_dtype, dev), w,
                                scales, z, b, n=N, k=K, group_size=128, quant_algo=algo, alpha=prob["alpha"],
-                               out_dtype=TORCH_DT[out_dtype])
+                               out_dtype=TORCH_DT[out_dtype], regime=regime)
         ref = oracle.woq_matmul_ref(prob["act"], prob["q"], prob["scales"], zeros, bias, prob["pre_quant_scale"],
                                     prob["alpha"], 128, out_dtype, w4a8=True)
     torch.cuda.synchronize()
@@ -83,3 +83,90 @@ def test_w4a8_identity_recovers_e4m3_weight(pkg, oracle, dev):
     out, _ = _run(pkg, oracle, dev, prob, K, K, N, "fp16", direct_fp8=True)
     w8 = oracle.dequantize(q, s, None, 128, "fp8")
     assert (out == oracle.round_f16(w8)).all()
+
+
+STREAM, GEMM = 1, 2
+
+
+@pytest.mark.parametrize("out_dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("M", [1, 3, 16])
+@pytest.mark.parametrize("direct", [False, True])
+def test_w4a8_streaming_kernel(pkg, oracle, dev, out_dtype, M, direct):
+    """Decode sizes on the weight-streaming W4A8 kernel (forced, and what AUTO picks for M <= 16):
+    same oracle, same bar; the GEMM kernel on the same inputs agrees to float32 summation order."""
+    K, N = 1024, 384
+    prob = oracle.make_w4a8_problem(M, K, N, seed=40 + M, out_dtype=out_dtype)
+    out, ref = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, direct_fp8=direct, regime=STREAM)
+    assert oracle.max_rel_err(out, ref) < TOL
+    auto, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, direct_fp8=direct)
+    assert (auto == out).all()
+    gemm, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, direct_fp8=direct, regime=GEMM)
+    assert oracle.max_rel_err(gemm, out) < 2e-3
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 128, 16), (5, 640, 272), (16, 2176, 1040), (2, 8192, 48), (9, 4096, 4112)])
+def test_w4a8_streaming_shapes(pkg, oracle, dev, M, K, N):
+    """Fewer tile rows than wavefronts, a last column group that is only partly there, long K,
+    both launch shapes; with and without zeros, bias."""
+    prob = oracle.make_w4a8_problem(M, K, N, seed=M + N, out_dtype="bf16")
+    rng = np.random.default_rng(M)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+    for z in (None, zeros):
+        out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=bias, regime=STREAM)
+        assert oracle.max_rel_err(out, ref) < TOL, (M, K, N, z is not None)
+
+
+@pytest.mark.parametrize("shape", ["1,8,2", "1,16,2", "2,8,2", "2,8,3", "2,4,4", "4,8,2"])
+def test_w4a8_streaming_launch_shapes(pkg, oracle, dev, monkeypatch, shape):
+    """Every instantiated launch shape (strips per wavefront, wavefronts, tile rows in flight), whatever
+    the table would pick: K with a tile-row count that no shape divides, N that ends inside a group."""
+    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    M, K, N = 7, 2176, 272
+    prob = oracle.make_w4a8_problem(M, K, N, seed=17, out_dtype="fp16")
+    rng = np.random.default_rng(18)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    for z in (None, zeros):
+        out, ref = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=STREAM)
+        assert oracle.max_rel_err(out, ref) < TOL, (shape, z is not None)
+
+
+def test_w4a8_streaming_saturating_scales(pkg, oracle, dev):
+    """Group scales large enough that dequantized weights pass +-448: the conversion saturates
+    (the kernel's clamped path), as the oracle's e4m3 rounding does."""
+    M, K, N = 4, 512, 64
+    rng = np.random.default_rng(21)
+    q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    s = oracle.round_f16(rng.uniform(40, 120, (K // 128, N)).astype(np.float32))
+    s[0, :8] = 0.01  # some columns stay on the unclamped path within the same call
+    act = np.zeros((M, K), np.float32)
+    act[np.arange(M), [3, 130, 300, 511]] = 1.0
+    prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+    out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", direct_fp8=True, regime=STREAM)
+    w8 = oracle.dequantize(q, s, None, 128, "fp8")
+    assert np.abs(w8).max() == 448.0
+    assert (out == oracle.round_f16(w8[[3, 130, 300, 511]])).all()
+
+
+def test_w4a8_streaming_one_hot_rows_recover_e4m3_weight(pkg, oracle, dev):
+    """One-hot activation rows (exact in e4m3): row r of the output is row k_r of the e4m3-rounded
+    dequantized weight, bit for bit - with and without zero-points."""
+    M, K, N = 16, 1024, 256
+    rng = np.random.default_rng(8)
+    q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    s = oracle.round_f16(np.exp(rng.uniform(-2, 3, (K // 128, N))).astype(np.float32))
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    rows = rng.choice(K, size=M, replace=False)
+    act = np.zeros((M, K), np.float32)
+    act[np.arange(M), rows] = 1.0
+    prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+    for z in (None, zeros):
+        out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=STREAM)
+        w8 = oracle.dequantize(q, s, z, 128, "fp8")
+        assert (out == oracle.round_f16(w8[rows])).all()
+
+
+def test_w4a8_streaming_kernel_refuses_more_than_16_rows(pkg, oracle, dev):
+    prob = oracle.make_w4a8_problem(17, 256, 64, seed=1, out_dtype="bf16")
+    with pytest.raises(RuntimeError, match="unsupported m"):
+        _run(pkg, oracle, dev, prob, 17, 256, 64, "bf16", direct_fp8=True, regime=STREAM)
