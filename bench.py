@@ -104,25 +104,32 @@ def launch(pkg, act, layer, out, regime=0):
                      regime=regime)
 
 
-def time_graph(fn_body, launches):
+def time_graph(fn_body, launches, repeats=1):
     """Captures fn_body() (which issues `launches` kernels) in a HIP graph, replays it once
-    untimed, then times one replay with HIP events on the replay stream and with the host clock."""
+    untimed, then times one replay with HIP events on the replay stream and with the host clock
+    (`repeats` > 1: the fastest of that many timed replays, for short cases that would otherwise
+    be measured while the clocks still ramp up)."""
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
+    best = None
     with torch.cuda.stream(stream):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
             fn_body()
         graph.replay()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record(stream)
-        graph.replay()
-        e1.record(stream)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    return (t1 - t0), e0.elapsed_time(e1) * 1e-3, launches
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record(stream)
+            graph.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            cur = ((t1 - t0), e0.elapsed_time(e1) * 1e-3, launches)
+            if best is None or cur[1] < best[1]:
+                best = cur
+    return best
 
 
 def bench_decode(pkg, dev, steps, warmup, m=1):
@@ -330,7 +337,7 @@ def run_sweep(pkg, dev, which):
                     launch(pkg, act, layers[0], out)
                     act_bytes = 2
                 torch.cuda.synchronize()
-                _, sec, launches = time_graph(body, reps)
+                _, sec, launches = time_graph(body, reps, repeats=3)
                 us = sec / launches * 1e6
                 n_sz = 1 if kind != "w4a16" else 2  # scales only, or scales + zeros
                 by = algorithmic_bytes(m, k, n, bits, group, n_sz, act_bytes)

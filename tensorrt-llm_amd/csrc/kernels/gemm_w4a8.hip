@@ -138,7 +138,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         int const idx = slab_at(j) * 2 + h; // slab j sits at operand position slab_at(j)
         float const sc = EH::from_bits(st.s[s]);
         float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
-        b[s][idx] = dequant2_fp8<ZERO>(b[s][idx], st.w[s][j], h, pr, sc, zr);
+        b[s][idx] = dequant2_fp8<ZERO, false>(b[s][idx], st.w[s][j], h, pr, sc, zr);
     };
     constexpr int UNITS = NS * SLABS * 4; // 64 per step
 
@@ -207,6 +207,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // with the packed weights of step kt+2.
     BStage st0, st1;
     u32x8 b0[NS], b1[NS];
+    fp8_saturation_on(); // the conversions rely on it; off again before the epilogue
 #pragma unroll
     for (int s = 0; s < NS; ++s)
         b0[s] = b1[s] = u32x8{0, 0, 0, 0, 0, 0, 0, 0};
@@ -237,6 +238,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
+    fp8_saturation_off();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
 #pragma unroll
     for (int s = 0; s < NS; ++s)
@@ -256,7 +258,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     if constexpr (SPLITK)
                         unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, acc[rt][s][r]);
                     else
-                        out16[(size_t) row * p.n + col] = EO::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias));
+                        out16[(size_t) row * p.n + col]
+                            = EO::store(after_mode_change(__builtin_fmaf(p.alpha, acc[rt][s][r], bias)));
                 }
             }
     }

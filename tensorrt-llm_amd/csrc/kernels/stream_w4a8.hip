@@ -6,7 +6,8 @@
 // accumulates fp8 x fp8 products in float32, the epilogue applies alpha and the bias.  Because the
 // rounding to e4m3 is part of the result, the scale cannot be deferred to the group sums as in the
 // 16-bit streaming kernel: each weight is converted exactly, in registers, by the lane that loaded
-// it (about 3 VALU instructions per weight - still under what HBM delivers).
+// it (about 3 VALU instructions per weight - still under what HBM delivers; the saturation to
+// +-448 is done by the conversion instruction itself, see fp8_saturation_on()).
 //
 // Same skeleton as the 16-bit streaming kernel (stream_kernel.h): a workgroup owns NS strips of 16
 // columns, its wavefronts split K (tile row kt goes to wave kt % WAVES, PF tile rows in flight
@@ -26,12 +27,15 @@ __device__ __forceinline__ u32x2 buffer_load_x2(__amdgpu_buffer_rsrc_t rsrc, uin
     return __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int) byte_offset, 0, 0);
 }
 
-template <int ODT, bool ZERO, int NS, int WAVES, int PF>
+// ALDS: the workgroup stages the activation rows in LDS once (small M x K) and the lanes read
+// their A pieces from there; a pipeline stage then holds packed weights and scales only.
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
 __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 {
     using EO = Elem<ODT>;
     using EH = Elem<WOQ_FP16>;
     constexpr int TK = 128, SLABS = 4;
+    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (K + 16) bytes
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
     if (group >= p.groups)
@@ -68,10 +72,16 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     // activation row c (rows >= m start past the end of the buffer), this lane's 8 bytes of slab 0
     uint32_t const a_lane = (uint32_t) c * (uint32_t) K + (uint32_t) kg * 8u;
 
+    // LDS copy: row r at byte r * lds_row (+16: the rows of a half-wavefront's 8-byte reads fall
+    // into different banks); lanes of rows >= m read row m-1, their outputs are never stored
+    uint32_t const lds_row = (uint32_t) K + 16u;
+    int const a_row = c < p.m ? c : p.m - 1;
+    char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 8u;
+
     struct Stage
     {
         u32x4 w[NS];
-        u32x2 a[SLABS];
+        u32x2 a[ALDS ? 1 : SLABS];
         uint16_t s[NS];
         uint16_t z[NS];
     };
@@ -82,9 +92,12 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 #pragma unroll
         for (int s = 0; s < NS; ++s)
             st.w[s] = buffer_load_x4(w_rsrc, (wlane[s] + (uint32_t) kt * 1024u) | past);
+        if constexpr (!ALDS)
+        {
 #pragma unroll
-        for (int j = 0; j < SLABS; ++j)
-            st.a[j] = buffer_load_x2(act_rsrc, (a_lane + (uint32_t) (kt * TK + j * 32)) | past);
+            for (int j = 0; j < SLABS; ++j)
+                st.a[j] = buffer_load_x2(act_rsrc, (a_lane + (uint32_t) (kt * TK + j * 32)) | past);
+        }
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
@@ -115,14 +128,15 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             acc[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[s], 0, 0, 0, 0, 0, 0);
         }
     };
-    auto compute = [&](Stage const& st)
+    auto compute = [&](Stage const& st, int kt)
     {
         i32x8 a;
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
         {
-            a[2 * j] = (int) st.a[j][0];
-            a[2 * j + 1] = (int) st.a[j][1];
+            u32x2 const v = ALDS ? *reinterpret_cast<u32x2 const*>(a_lds + (uint32_t) (kt * TK + j * 32)) : st.a[ALDS ? 0 : j];
+            a[2 * j] = (int) v[0];
+            a[2 * j + 1] = (int) v[1];
         }
         bool may_saturate = false;
 #pragma unroll
@@ -142,17 +156,32 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     // prologue and loop are unconditional and the compiler's wait counts stay exact.
     int const n_my = (KT - wave + WAVES - 1) / WAVES;
     Stage st[PF];
+    fp8_saturation_on(); // the conversions below rely on it; off again before the epilogue
 #pragma unroll
     for (int i = 0; i < PF; ++i)
         fetch(st[i], wave + i * WAVES);
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (ALDS)
+    {
+        // behind the first weight prefetches: the activations come from L2 and land first
+        int const rows = p.m < 16 ? p.m : 16;
+        int const chunks_per_row = K / 16;
+        for (int idx = threadIdx.x; idx < rows * chunks_per_row; idx += WAVES * 64)
+        {
+            int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
+            u32x4 const v = buffer_load_x4(act_rsrc, (uint32_t) row * (uint32_t) K + (uint32_t) ch * 16u);
+            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + (uint32_t) row * lds_row + (uint32_t) ch * 16u) = v;
+        }
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    }
     for (int it = 0; it < n_my; it += PF)
     {
 #pragma unroll
         for (int i = 0; i < PF; ++i)
         {
             if (it + i < n_my)
-                compute(st[i]);
+                compute(st[i], wave + (it + i) * WAVES);
             __builtin_amdgcn_sched_barrier(0);
             fetch(st[i], wave + (it + i + PF) * WAVES);
             __builtin_amdgcn_sched_barrier(0);
@@ -160,6 +189,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     }
 
     // ---- cross-wavefront reduction (fixed order) and epilogue: out = T(alpha * sum + bias) ----
+    fp8_saturation_off();
     constexpr int SLOTS = NS * 4;
     __shared__ float red[WAVES][SLOTS][64];
 #pragma unroll
@@ -184,7 +214,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             sum += red[w2][slot][ln];
         int const ocol = (strip0 + s) * 16 + (ln & 15);
         float const bias = p.bias ? EO::load(p.bias, ocol) : 0.f;
-        out16[(size_t) row * p.n + ocol] = EO::store(__builtin_fmaf(p.alpha, sum, bias));
+        out16[(size_t) row * p.n + ocol] = EO::store(after_mode_change(__builtin_fmaf(p.alpha, sum, bias)));
     }
 }
 
@@ -193,36 +223,68 @@ namespace
 
 struct W4a8Shape
 {
-    int ns, waves, pf;
+    int ns, waves, pf, lds;
 };
 
-// WOQ_STREAM_SHAPE="ns,waves,pf" overrides the heuristic (for tuning sweeps)
-W4a8Shape pick_shape(int m, int strips, int k_tiles)
+constexpr size_t kMaxActLds = 48 * 1024;
+
+size_t act_lds_bytes(int m, int k)
+{
+    return (size_t) (m < 16 ? m : 16) * ((size_t) k + 16);
+}
+
+// WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
+W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
 {
     if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
     {
-        W4a8Shape sh{0, 0, 0};
-        if (std::sscanf(e, "%d,%d,%d", &sh.ns, &sh.waves, &sh.pf) == 3)
+        W4a8Shape sh{0, 0, 0, 0};
+        if (std::sscanf(e, "%d,%d,%d,%d", &sh.ns, &sh.waves, &sh.pf, &sh.lds) == 4)
             return sh;
     }
-    // measured on MI355X: two strips per wavefront share the activation loads once there are
-    // enough column groups to fill the chip; narrow matrices keep one strip and 8-way split K
+    // measured on MI355X.  Activations that fit the LDS staging area: one strip per wavefront
+    // and 8-way split K (two strips on very wide matrices, deeper prefetch on long K).
+    if (act_lds_bytes(m, k) <= kMaxActLds)
+    {
+        if (strips >= 2048)
+            return {2, 8, 2, 1};
+        return k_tiles >= 112 ? W4a8Shape{1, 8, 4, 1} : W4a8Shape{1, 8, 2, 1};
+    }
+    // otherwise two strips per wavefront share the activation loads once there are enough
+    // column groups to fill the chip; narrow matrices keep one strip
     if (strips >= 2048)
-        return {2, 4, 4};
+        return {2, 4, 4, 0};
     if (strips >= 512)
-        return k_tiles >= 128 ? W4a8Shape{2, 8, 3} : W4a8Shape{2, 8, 2};
+        return k_tiles >= 128 ? W4a8Shape{2, 8, 3, 0} : W4a8Shape{2, 8, 2, 0};
     if (strips >= 384 && m > 4)
-        return {2, 8, 2};
-    return {1, 8, 2};
+        return {2, 8, 2, 0};
+    return {1, 8, 2, 0};
 }
 
-template <int ODT, bool ZERO, int NS, int WAVES, int PF>
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
 int launch_variant(StreamParams sp, hipStream_t stream)
 {
+    auto kernel = stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF, ALDS>;
+    size_t lds = 0;
+    if constexpr (ALDS)
+    {
+        lds = act_lds_bytes(sp.m, sp.k);
+        if (lds > kMaxActLds)
+            return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
+        static bool raised = false; // benign race: the attribute call is idempotent
+        if (lds > 32 * 1024 && !raised)
+        {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxActLds);
+            if (e != hipSuccess)
+                return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
-    hipLaunchKernelGGL((stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF>), grid, block, 0, stream, sp);
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "W4A8 stream kernel launch failed: %s", hipGetErrorString(err));
@@ -232,19 +294,24 @@ int launch_variant(StreamParams sp, hipStream_t stream)
 template <int ODT, bool ZERO>
 int launch_shaped(StreamParams const& sp, hipStream_t s)
 {
-    W4a8Shape const sh = pick_shape(sp.m, sp.strips, sp.k_tiles);
-#define WOQ_SHAPE(NS_, WAVES_, PF_)                                                                                    \
-    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_)                                                            \
-        return launch_variant<ODT, ZERO, NS_, WAVES_, PF_>(sp, s);
-    WOQ_SHAPE(1, 8, 2)
-    WOQ_SHAPE(1, 16, 2)
-    WOQ_SHAPE(2, 8, 2)
-    WOQ_SHAPE(2, 8, 3)
-    WOQ_SHAPE(2, 4, 4)
-    WOQ_SHAPE(4, 8, 2)
+    W4a8Shape const sh = pick_shape(sp.m, sp.k, sp.strips, sp.k_tiles);
+#define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                                   \
+        return launch_variant<ODT, ZERO, NS_, WAVES_, PF_, LDS_>(sp, s);
+    WOQ_SHAPE(1, 8, 2, false)
+    WOQ_SHAPE(1, 16, 2, false)
+    WOQ_SHAPE(2, 8, 2, false)
+    WOQ_SHAPE(2, 8, 3, false)
+    WOQ_SHAPE(2, 4, 4, false)
+    WOQ_SHAPE(4, 8, 2, false)
+    WOQ_SHAPE(1, 8, 2, true)
+    WOQ_SHAPE(1, 8, 4, true)
+    WOQ_SHAPE(2, 8, 2, true)
+    WOQ_SHAPE(2, 4, 4, true)
+    WOQ_SHAPE(4, 8, 2, true)
 #undef WOQ_SHAPE
-    return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d is not instantiated", sh.ns, sh.waves,
-        sh.pf);
+    return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated", sh.ns,
+        sh.waves, sh.pf, sh.lds);
 }
 
 } // namespace

@@ -9,10 +9,12 @@ namespace woq
 
 // elements 4h+2p, 4h+2p+1 of slab dword `w` -> 2 e4m3 bytes in 16-bit word p of `old` (a dword of
 // the B operand holds elements 4h .. 4h+3 in order; the other word is kept).
+// CLAMP = false is for kernels that run with fp8_saturation_on(): the conversion instruction then
+// saturates by itself and the clamp (a quarter of the instructions) is not needed.
 // With zero-points the weight is fma(q, s, z) on the two's-complement nibble.  Without them
 // q * s = fma(u, s, -8 s) on the stored nibble u = q + 8: -8 s is exact, so this is the same
 // single rounding, and u comes out of a byte-to-float conversion with no sign extension.
-template <bool ZERO>
+template <bool ZERO, bool CLAMP = true>
 __device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h, int p, float s, float z)
 {
     float v0, v1;
@@ -22,8 +24,8 @@ __device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h
         uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
         int const q0 = (int) (t << (28 - 4 * (e0 / 2))) >> 28;
         int const q1 = (int) (t << (12 - 4 * (e0 / 2))) >> 28;
-        v0 = clamp_e4m3(__builtin_fmaf((float) q0, s, z));
-        v1 = clamp_e4m3(__builtin_fmaf((float) q1, s, z));
+        v0 = __builtin_fmaf((float) q0, s, z);
+        v1 = __builtin_fmaf((float) q1, s, z);
     }
     else
     {
@@ -33,8 +35,13 @@ __device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h
         uint32_t m = (p == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
         asm volatile("" : "+v"(m));
         float const m8s = -8.f * s;
-        v0 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h)) & 0xFF), s, m8s));
-        v1 = clamp_e4m3(__builtin_fmaf((float) ((m >> (8 * h + 16)) & 0xFF), s, m8s));
+        v0 = __builtin_fmaf((float) ((m >> (8 * h)) & 0xFF), s, m8s);
+        v1 = __builtin_fmaf((float) ((m >> (8 * h + 16)) & 0xFF), s, m8s);
+    }
+    if constexpr (CLAMP) // saturation to +-448 in software; off when the conversion itself saturates
+    {
+        v0 = clamp_e4m3(v0);
+        v1 = clamp_e4m3(v1);
     }
     return p == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, false)
                   : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, true);
@@ -79,7 +86,32 @@ __device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, flo
     return (uint32_t) r;
 }
 
+// MODE.FP16_OVFL (bit 23 of the wavefront's MODE register) makes v_cvt_pk_fp8_f32 saturate finite
+// overflow to +-448 instead of producing NaN - the rounding the W4A8 dequantize is defined with.
+// The bit also makes fp16 results clamp instead of overflowing to infinity, so it is switched off
+// again before an epilogue converts outputs: pass every value that a later conversion reads
+// through after_mode_change() so that the conversion cannot be scheduled before the switch
+// (volatile asm statements keep their order).  MODE is per wavefront and set from the kernel
+// descriptor at launch: nothing leaks into other kernels.
+__device__ __forceinline__ void fp8_saturation_on()
+{
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1\n\ts_nop 3" ::: "memory");
+}
+
+__device__ __forceinline__ void fp8_saturation_off()
+{
+    asm volatile("s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 0\n\ts_nop 3" ::: "memory");
+}
+
+template <typename T>
+__device__ __forceinline__ T after_mode_change(T v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // c += a x b (32 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)

@@ -117,7 +117,8 @@ def test_w4a8_streaming_shapes(pkg, oracle, dev, M, K, N):
         assert oracle.max_rel_err(out, ref) < TOL, (M, K, N, z is not None)
 
 
-@pytest.mark.parametrize("shape", ["1,8,2", "1,16,2", "2,8,2", "2,8,3", "2,4,4", "4,8,2"])
+@pytest.mark.parametrize("shape", ["1,8,2,0", "1,16,2,0", "2,8,2,0", "2,8,3,0", "2,4,4,0", "4,8,2,0", "1,8,2,1", "1,8,4,1",
+                                   "2,8,2,1", "2,4,4,1", "4,8,2,1"])
 def test_w4a8_streaming_launch_shapes(pkg, oracle, dev, monkeypatch, shape):
     """Every instantiated launch shape (strips per wavefront, wavefronts, tile rows in flight), whatever
     the table would pick: K with a tile-row count that no shape divides, N that ends inside a group."""
@@ -131,21 +132,31 @@ def test_w4a8_streaming_launch_shapes(pkg, oracle, dev, monkeypatch, shape):
         assert oracle.max_rel_err(out, ref) < TOL, (shape, z is not None)
 
 
-def test_w4a8_streaming_saturating_scales(pkg, oracle, dev):
-    """Group scales large enough that dequantized weights pass +-448: the conversion saturates
-    (the kernel's clamped path), as the oracle's e4m3 rounding does."""
+@pytest.mark.parametrize("regime", [STREAM, GEMM])
+def test_w4a8_saturating_scales(pkg, oracle, dev, regime):
+    """Group scales (and zeros) large enough that dequantized weights pass +-448: the conversion
+    saturates as the oracle's e4m3 rounding does, in both kernels, bit for bit.  A second call with
+    a large alpha overflows fp16: those outputs are infinite, not clamped."""
     M, K, N = 4, 512, 64
     rng = np.random.default_rng(21)
     q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
     s = oracle.round_f16(rng.uniform(40, 120, (K // 128, N)).astype(np.float32))
-    s[0, :8] = 0.01  # some columns stay on the unclamped path within the same call
+    s[0, :8] = 0.01  # some columns stay far from saturation within the same call
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 300).astype(np.float32))
+    rows = [3, 130, 300, 511]
     act = np.zeros((M, K), np.float32)
-    act[np.arange(M), [3, 130, 300, 511]] = 1.0
-    prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
-    out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", direct_fp8=True, regime=STREAM)
-    w8 = oracle.dequantize(q, s, None, 128, "fp8")
-    assert np.abs(w8).max() == 448.0
-    assert (out == oracle.round_f16(w8[[3, 130, 300, 511]])).all()
+    act[np.arange(M), rows] = 1.0
+    for z in (None, zeros):
+        w8 = oracle.dequantize(q, s, z, 128, "fp8")
+        assert np.abs(w8).max() == 448.0
+        prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+        out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=regime)
+        assert (out == oracle.round_f16(w8[rows])).all()
+        prob["alpha"] = 1024.0
+        out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=regime)
+        expect = oracle.round_f16(1024.0 * w8[rows])
+        assert np.isinf(expect).any()
+        assert (out == expect).all()
 
 
 def test_w4a8_streaming_one_hot_rows_recover_e4m3_weight(pkg, oracle, dev):
