@@ -2,7 +2,7 @@
 """Benchmark of the weight-only quantized matmul hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-    python bench.py --mode sweep --sweep decode8b|prefill8b|llama70b|w4a8   (tables of the other
+    python bench.py --mode sweep --sweep decode8b|prefill8b|llama70b|w4a8|moe   (tables of the other
                                                    benchmark configurations, one JSON line per case)
 
 Workload (the configuration the headline metric is quoted on): W4A16, group 128, bf16
@@ -349,6 +349,47 @@ def run_sweep(pkg, dev, which):
             torch.cuda.empty_cache()
 
 
+def run_moe_sweep(pkg, dev):
+    """Grouped (mixture-of-experts) matmul on Mixtral-8x7B expert shapes: 8 experts, W4A16 g128 with
+    bf16 scales + zeros, top-2 routing of T tokens drawn uniformly (seeded), rows sorted by expert.
+    One JSON line per (shape, T): launch time, algorithmic GB/s (weights of the experts that own
+    rows + scales + activations + outputs) and TFLOP/s."""
+    F = pkg.functional
+    experts, top_k = 8, 2
+    for name, k, n in [("fc1 gate_up", 4096, 28672), ("fc2 down", 14336, 4096)]:
+        layers = [make_layer(pkg, dev, k, n, 6000 + e) for e in range(experts)]
+        copies = copies_beyond_cache(experts * k * n // 2)
+        weight = [torch.stack([l["weight"] for l in layers]).roll(r, 0).contiguous() for r in range(copies)]
+        scales = torch.stack([l["scales"] for l in layers]).contiguous()
+        zeros = torch.stack([l["zeros"] for l in layers]).contiguous()
+        layers = None
+        for tokens in [1, 4, 16, 64, 256, 1024, 4096]:
+            g = torch.Generator().manual_seed(tokens)
+            picks = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(tokens)]).flatten()
+            rows = torch.bincount(picks, minlength=experts)
+            total = torch.cumsum(rows, 0).to(torch.int64).to(dev)
+            m = int(rows.sum())
+            act = torch.randn((m, k), device=dev).to(torch.bfloat16)
+            out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            reps = 20 if m <= 512 else 4
+
+            def run(r):
+                F.woq_grouped_matmul_raw(act, weight[r % copies], scales, zeros, None, total, n=n, k=k,
+                                         group_size=GROUP, quant_algo=F.ZERO, out=out)
+            run(0)
+            torch.cuda.synchronize()
+            _, sec, launches = time_graph(lambda: [run(r) for r in range(reps)], reps, repeats=3)
+            us = sec / launches * 1e6
+            active = int((rows > 0).sum())
+            by = active * (k * n // 2 + (k // GROUP) * n * 4) + m * k * 2 + m * n * 2
+            print(json.dumps({"sweep": "moe", "shape": name, "k": k, "n": n, "experts": experts, "tokens": tokens,
+                              "rows": m, "rows_per_expert": rows.tolist(), "us": round(us, 2),
+                              "gbs": round(by / us / 1e3, 1), "tflops": round(2.0 * m * n * k / us / 1e6, 1)}),
+                  flush=True)
+        weight = scales = zeros = None
+        torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -359,7 +400,7 @@ def main():
     ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "sweep"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
-    ap.add_argument("--sweep", choices=sorted(SWEEPS), default="llama70b")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "
@@ -371,7 +412,10 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.mode == "sweep":
-        run_sweep(pkg, dev, args.sweep)
+        if args.sweep == "moe":
+            run_moe_sweep(pkg, dev)
+        else:
+            run_sweep(pkg, dev, args.sweep)
         return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode)

@@ -143,6 +143,37 @@ int woq_matmul_check(const woq_matmul_args* args);
  * plugin's own m*k*sizeof(half) smoothing buffer (weightOnlyGroupwiseQuantMatmulPlugin.cpp:377-379). */
 size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype);
 
+/*
+ * Grouped (mixture-of-experts) matmul: expert e multiplies its own rows of `act` with its own
+ * weight matrix, out[rows_e] = act[rows_e] x dequant(W_e) (+ bias_e).  Replaces
+ * MoeGemmRunner<T, uint8_t | cutlass::uint4b_t>::moeGemm / moeGemmBiasAct without an activation
+ * (kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:235-244) with the weight-only
+ * scales of QuantParams::Int (moe_kernels.h:144-198); groupwise scales / zeros are accepted too.
+ *   base.act     [total_rows, k], rows sorted by expert;  base.out  [total_rows, n]
+ *   base.m       total_rows
+ *   base.weight  num_experts preprocessed matrices back to back (what woq_preprocess_weights
+ *                writes for experts = num_experts), woq_preprocessed_bytes(k, n, type) apart
+ *   base.scales / base.zeros   [num_experts, n] (group_size 0) or [num_experts, k/group_size, n]
+ *   base.bias    [num_experts, n] or NULL
+ *   total_rows_before_expert   device memory, int64 [num_experts]: rows of experts 0..e
+ *                (inclusive prefix sums, non-decreasing, last = total_rows; the reference's
+ *                total_tokens_including_expert); experts may own no rows
+ * pre_quant_scale, FP8_ALPHA and the workspace are not used (must be NULL / unset).
+ * AUTO regime: the streaming kernel while the average expert has at most 16 rows (an expert with
+ * more streams its weights once per 16 rows), tiled MFMA kernels above.
+ */
+typedef struct woq_grouped_matmul_args
+{
+    woq_matmul_args base;
+    const int64_t* total_rows_before_expert;
+    int32_t num_experts;
+} woq_grouped_matmul_args;
+
+int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);
+
+/* Validation only (no launch): what woq_grouped_matmul would return for these arguments. */
+int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);
+
 /* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, < 2^26 for int8
  * weights; m <= 16 for W4A8), GEMM otherwise - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */

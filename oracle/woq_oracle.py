@@ -467,6 +467,26 @@ def woq_matmul_ref(act, q, scales, zeros=None, bias=None, pre_quant_scale=None, 
     return out
 
 
+def grouped_matmul_ref(act, q, scales, zeros, bias, total_rows_before_expert, group_size: int = 0,
+                       act_dtype: str = "bf16") -> np.ndarray:
+    """The MoE expert GEMM (MoeGemmRunner::moeGemm / moeGemmBiasAct without activation,
+    kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:235-244; the CUTLASS problem visitor
+    gives expert e the rows [total[e-1], total[e]), cutlass_extensions/gemm/kernel/moe_problem_visitor.h):
+    rows of expert e times ITS dequantized weight, plus its bias row.  q [E, K, N], scales / zeros
+    [E, N] or [E, K/g, N], bias [E, N]; float64 accumulation, not rounded."""
+    act = np.asarray(act, np.float32)
+    total = np.asarray(total_rows_before_expert, np.int64)
+    out = np.zeros((act.shape[0], np.asarray(q).shape[2]), np.float64)
+    begin = 0
+    for e, end in enumerate(total):
+        end = int(end)
+        if end > begin:
+            out[begin:end] = woq_matmul_ref(act[begin:end], q[e], scales[e], None if zeros is None else zeros[e],
+                                            None if bias is None else bias[e], None, 1.0, group_size, act_dtype)
+        begin = end
+    return out
+
+
 def max_rel_err(out, ref) -> float:
     """The parity norm used by every output test: max|out - ref| / max|ref|."""
     ref = np.asarray(ref, np.float64)

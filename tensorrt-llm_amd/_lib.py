@@ -40,6 +40,10 @@ class MatmulArgs(ctypes.Structure):
     ]
 
 
+class GroupedMatmulArgs(ctypes.Structure):
+    _fields_ = [("base", MatmulArgs), ("total_rows_before_expert", ctypes.c_void_p), ("num_experts", ctypes.c_int32)]
+
+
 def lib_path() -> str:
     return _LIB_PATH
 
@@ -54,6 +58,8 @@ def _load():
     sig = {
         "woq_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), vp]),
         "woq_matmul_check": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
+        "woq_grouped_matmul": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs), vp]),
+        "woq_grouped_matmul_check": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs)]),
         "woq_workspace_bytes": (sz, [i32, i32, i32, i32, i32]),
         "woq_select_regime": (ctypes.c_int, [i32, i32, i32, i32]),
         "woq_preprocessed_bytes": (sz, [i64, i64, i32]),

@@ -30,11 +30,17 @@ int launch_skinny_FP16_8(MatmulProblem const& p, GemmPlan const& plan, void* str
 int launch_gemm_w4a8(MatmulProblem const& p, void* stream);
 int launch_stream_w4a8(MatmulProblem const& p, void* stream);
 
+int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream);
+
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_gemm_w4a8(p, stream);
-    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, p.bits);
+    return launch_gemm_planned(p, plan_gemm(p.m, p.n, p.k, p.bits), stream);
+}
+
+int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream)
+{
     bool const bf16 = p.out_dtype == WOQ_BF16;
     if (plan.skinny)
     {
@@ -51,7 +57,7 @@ int launch_stream(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_stream_w4a8(p, stream);
-    if (p.m > kStreamMaxM)
+    if (!p.expert_rows && p.m > kStreamMaxM) // a grouped problem runs 16-row passes per expert
         return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
             p.m);
     if (p.out_dtype == WOQ_BF16)
@@ -323,6 +329,75 @@ extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
         p.workspace_bytes -= used;
     }
     return streaming ? launch_stream(p, stream) : launch_gemm(p, stream);
+}
+
+namespace
+{
+// Kernel family and tile height of a grouped problem.  Only the total row count is known on the
+// host, so the choice goes by the average expert: streaming passes of 16 rows while that is at
+// most 16 rows; 64-row deferred-scale tiles up to 256; exact-dequantize 256-row tiles above (128
+// when those would not fill the chip).  K is never split.
+int grouped_regime(woq_grouped_matmul_args const* a)
+{
+    int r = a->base.regime != WOQ_REGIME_AUTO ? a->base.regime : env_regime();
+    if (r == WOQ_REGIME_AUTO)
+        r = (int64_t) a->base.m <= (int64_t) 16 * a->num_experts ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
+    return r;
+}
+
+GemmPlan plan_grouped(int total_rows, int num_experts, int n)
+{
+    GemmPlan pl;
+    int const avg = (total_rows + num_experts - 1) / num_experts;
+    pl.skinny = avg <= 256;
+    if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
+        pl.skinny = !std::strcmp(e, "skinny");
+    if (pl.skinny)
+        pl.rt = 4;
+    else
+        pl.rt = (long) num_experts * gemm_tiles(avg, n, 16) >= kEnoughTiles ? 16 : 8;
+    pl.k_splits = 1;
+    pl.ws_bytes = 0;
+    return pl;
+}
+} // namespace
+
+extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
+{
+    if (!args)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "args is NULL");
+    MatmulProblem p;
+    if (int rc = validate(&args->base, p))
+        return rc;
+    if (p.w4a8 || p.pre_quant_scale)
+        return fail(WOQ_ERR_UNSUPPORTED, "grouped matmul: FP8_ALPHA and PRE_QUANT_SCALE are not supported");
+    if (args->num_experts <= 0)
+        return fail(WOQ_ERR_BAD_SHAPE, "num_experts must be positive (got %d)", args->num_experts);
+    if (p.m > 0 && !args->total_rows_before_expert)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "total_rows_before_expert must not be NULL");
+    int const r = args->base.regime;
+    if (r != WOQ_REGIME_AUTO && r != WOQ_REGIME_STREAM && r != WOQ_REGIME_GEMM)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", r);
+    return WOQ_OK;
+}
+
+extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream)
+{
+    if (int rc = woq_grouped_matmul_check(args))
+        return rc;
+    MatmulProblem p;
+    validate(&args->base, p);
+    if (p.m == 0)
+        return WOQ_OK;
+    p.expert_rows = args->total_rows_before_expert;
+    p.num_experts = args->num_experts;
+    p.weight_stride = woq_preprocessed_bytes(p.k, p.n, p.bits == 8 ? WOQ_W8_A16 : WOQ_W4_A16);
+    p.scale_stride = (size_t) (p.group_size ? p.k / p.group_size : 1) * (size_t) p.n * 2;
+    p.workspace = nullptr;
+    p.workspace_bytes = 0;
+    if (grouped_regime(args) == WOQ_REGIME_STREAM)
+        return launch_stream(p, stream);
+    return launch_gemm_planned(p, plan_grouped(p.m, p.num_experts, p.n), stream);
 }
 
 extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,

@@ -261,6 +261,17 @@ __device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc,
     return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int) byte_offset, 0, 0);
 }
 
+// A pointer (or count) that is the same in every lane but was computed from loaded values: moved
+// into scalar registers, so that buffer descriptors built from it stay scalar too.
+template <typename T>
+__device__ __forceinline__ T* uniform_ptr(T* ptr)
+{
+    uint64_t const v = reinterpret_cast<uint64_t>(ptr);
+    uint32_t const lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) v);
+    uint32_t const hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (v >> 32));
+    return reinterpret_cast<T*>(((uint64_t) hi << 32) | lo);
+}
+
 // Workgroups are handed to the 8 XCDs round-robin.  Mapping block b to
 // strip (b % 8) * strips_per_xcd + b / 8 keeps neighbouring 16-column strips (which share
 // 128-byte lines of the scale / zero rows) on one XCD, hence in one L2.

@@ -23,7 +23,55 @@ struct GemmParams
     int k_splits;        // workgroups along K per output tile (blockIdx.y)
     int tiles_per_split; // tile rows of K each of them covers
     float* partial;      // [m, n] float32, zeroed, when k_splits > 1
+    // grouped problems (see MatmulProblem): m is the total row count, tiles_m an upper bound of
+    // the row tiles of all experts together
+    int64_t const* expert_rows = nullptr;
+    int num_experts = 0;
+    size_t weight_stride = 0, scale_stride = 0;
 };
+
+inline void set_group_fields(GemmParams& gp, MatmulProblem const& p, int tile_rows)
+{
+    gp.expert_rows = p.expert_rows;
+    gp.num_experts = p.num_experts;
+    gp.weight_stride = p.weight_stride;
+    gp.scale_stride = p.scale_stride;
+    if (p.expert_rows) // every expert may end with a partly filled tile
+        gp.tiles_m = p.m / tile_rows + p.num_experts;
+}
+
+// Grouped problems: row tile `tm` counts through the row tiles of expert 0, 1, ... in turn.
+// Finds the expert it belongs to, narrows the parameter block to that expert's operands and rows
+// (so that the kernel proceeds as for an ordinary problem) and makes tm the tile index inside
+// the expert.  False when tm is past the last tile.  All values are wavefront-uniform.
+__device__ __forceinline__ bool select_expert(GemmParams& p, int& tm, int tile_rows)
+{
+    int64_t begin = 0;
+    int first_tile = 0;
+    for (int e = 0; e < p.num_experts; ++e)
+    {
+        int64_t const end = p.expert_rows[e];
+        int const rows = (int) (end - begin);
+        int const tiles = (rows + tile_rows - 1) / tile_rows;
+        if (tm < first_tile + tiles)
+        {
+            p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
+            p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) p.n * 2);
+            p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
+            p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
+            if (p.zeros)
+                p.zeros = uniform_ptr(static_cast<char const*>(p.zeros) + (size_t) e * p.scale_stride);
+            if (p.bias)
+                p.bias = uniform_ptr(static_cast<char const*>(p.bias) + (size_t) e * (size_t) p.n * 2);
+            p.m = __builtin_amdgcn_readfirstlane(rows);
+            tm = __builtin_amdgcn_readfirstlane(tm - first_tile);
+            return true;
+        }
+        first_tile += tiles;
+        begin = end;
+    }
+    return false;
+}
 
 constexpr int kGemmBN = 256; // columns of an output tile (4 wavefronts x 64)
 

@@ -61,8 +61,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int const in_group = kGemmGroupM * p.tiles_n;
     int const first_m = (t / in_group) * kGemmGroupM;
     int const gsz = p.tiles_m - first_m < kGemmGroupM ? p.tiles_m - first_m : kGemmGroupM;
-    int const tm = first_m + (t % in_group) % gsz;
+    int tm = first_m + (t % in_group) % gsz;
     int const tn = (t % in_group) / gsz;
+    if (p.expert_rows && !select_expert(p, tm, kGemmBM))
+        return;
 
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -429,6 +431,7 @@ int launch_gemm_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream
     gp.partial = static_cast<float*>(p.workspace);
     if (plan.k_splits > 1 && (!p.workspace || p.workspace_bytes < plan.ws_bytes))
         return fail(WOQ_ERR_WORKSPACE, "split-K needs %zu workspace bytes", plan.ws_bytes);
+    set_group_fields(gp, p, plan.rt * 16);
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
     switch (p.group_size)

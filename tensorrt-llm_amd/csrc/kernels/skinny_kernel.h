@@ -55,7 +55,10 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     int t;
     if (!xcd_tile(p.tiles_m * p.tiles_n, t))
         return;
-    int const tm = t % p.tiles_m, tn = t / p.tiles_m;
+    int tm = t % p.tiles_m;
+    int const tn = t / p.tiles_m;
+    if (p.expert_rows && !select_expert(p, tm, kSkinnyBM))
+        return;
 
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -440,6 +443,7 @@ int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stre
     gp.partial = static_cast<float*>(p.workspace);
     if (plan.k_splits > 1 && (!p.workspace || p.workspace_bytes < plan.ws_bytes))
         return fail(WOQ_ERR_WORKSPACE, "split-K needs %zu workspace bytes", plan.ws_bytes);
+    set_group_fields(gp, p, rt * 16);
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
     switch (p.group_size)

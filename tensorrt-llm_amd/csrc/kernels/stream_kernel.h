@@ -42,6 +42,11 @@ struct StreamParams
     int strips;         // n / 16
     int groups;         // ceil(strips / NS): column groups, one workgroup each
     int groups_per_xcd; // ceil(groups / 8)
+    // grouped problems (rows sorted by expert, expert_rows[e] = rows of experts 0..e, device
+    // memory): blockIdx.y is the expert, strides are bytes per expert, m is unused
+    int64_t const* expert_rows = nullptr;
+    int num_experts = 0;
+    size_t weight_stride = 0, scale_stride = 0;
 };
 
 // Everything one wavefront needs for one tile row (NS tiles side by side), fetched together so
@@ -62,7 +67,7 @@ struct StreamStage
 // PF    tile rows in flight per wavefront
 // ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
-__global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
+__device__ __forceinline__ void stream_body(StreamParams const& p)
 {
     static_assert(!ALDS || MT == 1, "LDS-staged activations are for M <= 16");
     using E = Elem<DT>;
@@ -347,6 +352,39 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
     }
 }
 
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
+__global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
+{
+    stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>(p);
+}
+
+// Grouped problems: workgroup (x, e) is workgroup x of expert e's own matmul.  The parameters are
+// narrowed to that expert's operands and rows; an expert with more than 16 rows streams its
+// weights once per 16 rows (this kernel is chosen when that is rare).
+template <int DT, int BITS, int GROUP, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
+__global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams p)
+{
+    int const e = (int) blockIdx.y;
+    int64_t const begin = e ? p.expert_rows[e - 1] : 0;
+    int rows_left = __builtin_amdgcn_readfirstlane((int) (p.expert_rows[e] - begin));
+    p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
+    p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) p.n * 2);
+    p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
+    p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
+    if (ZERO)
+        p.zeros = uniform_ptr(static_cast<char const*>(p.zeros) + (size_t) e * p.scale_stride);
+    if (p.bias)
+        p.bias = uniform_ptr(static_cast<char const*>(p.bias) + (size_t) e * (size_t) p.n * 2);
+    for (; rows_left > 0; rows_left -= 16)
+    {
+        p.m = rows_left;
+        stream_body<DT, BITS, GROUP, false, ZERO, 1, NS, WAVES, PF, ALDS>(p);
+        __syncthreads(); // this pass is done with the LDS areas
+        p.act = static_cast<char const*>(p.act) + (size_t) 16 * (size_t) p.k * 2;
+        p.out = static_cast<char*>(p.out) + (size_t) 16 * (size_t) p.n * 2;
+    }
+}
+
 // launch shape: NS strips per wavefront, WAVES wavefronts per workgroup, PF tile rows in flight,
 // lds != 0: activations staged in LDS
 struct StreamShape
@@ -366,11 +404,17 @@ constexpr size_t kStreamMaxActLds = 96 * 1024;
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k);
 
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
+    bool GROUPED = false>
 int launch_stream_variant(StreamParams sp, hipStream_t stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    auto kernel = stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>;
+    auto kernel = [] {
+        if constexpr (GROUPED)
+            return stream_grouped_kernel<DT, BITS, GROUP, ZERO, NS, WAVES, PF, ALDS>;
+        else
+            return stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>;
+    }();
     size_t lds = 0;
     if constexpr (ALDS)
     {
@@ -389,7 +433,7 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
-    dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    dim3 grid(sp.groups_per_xcd * 8, GROUPED ? sp.num_experts : 1), block(WAVES * 64);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
@@ -430,6 +474,27 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
         sh.waves, sh.pf, sh.lds);
 }
 
+// grouped problems: the launch shapes the table picks for one 16-row tile
+template <int DT, int BITS, int GROUP, bool ZERO>
+int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
+{
+    constexpr int TK = BITS == 4 ? 128 : 64;
+    // every expert's column groups run side by side: the grid is num_experts times taller
+    StreamShape const sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK);
+#define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                                   \
+        return launch_stream_variant<DT, BITS, GROUP, false, ZERO, 1, NS_, WAVES_, PF_, LDS_, true>(sp, s);
+    WOQ_SHAPE(1, 8, 4, true)
+    WOQ_SHAPE(2, 8, 4, true)
+    WOQ_SHAPE(4, 8, 2, true)
+    WOQ_SHAPE(1, 8, 4, false)
+    WOQ_SHAPE(2, 8, 2, false)
+    WOQ_SHAPE(4, 4, 2, false)
+#undef WOQ_SHAPE
+    return fail(WOQ_ERR_UNSUPPORTED, "grouped stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated", sh.ns,
+        sh.waves, sh.pf, sh.lds);
+}
+
 template <int DT, int BITS>
 int launch_stream_typed(MatmulProblem const& p, void* stream)
 {
@@ -449,10 +514,28 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.k_tiles = (p.k + TK - 1) / TK;
     sp.strips = p.n / kTileN;
     sp.groups = sp.groups_per_xcd = 0;
+    sp.expert_rows = p.expert_rows;
+    sp.num_experts = p.num_experts;
+    sp.weight_stride = p.weight_stride;
+    sp.scale_stride = p.scale_stride;
     auto s = static_cast<hipStream_t>(stream);
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;
     bool const zero = p.zeros != nullptr;
+    if (p.expert_rows)
+    {
+        switch (p.group_size)
+        {
+        case 0: return launch_stream_grouped<DT, BITS, 0, false>(sp, s);
+        case 64:
+            return zero ? launch_stream_grouped<DT, BITS, 64, true>(sp, s)
+                        : launch_stream_grouped<DT, BITS, 64, false>(sp, s);
+        case 128:
+            return zero ? launch_stream_grouped<DT, BITS, 128, true>(sp, s)
+                        : launch_stream_grouped<DT, BITS, 128, false>(sp, s);
+        default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
+        }
+    }
 
 #define WOQ_STREAM_PQS(G)                                                                                              \
     if (pqs)                                                                                                           \

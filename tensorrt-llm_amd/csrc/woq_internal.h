@@ -48,6 +48,11 @@ struct MatmulProblem
     bool w4a8;
     void* workspace;
     size_t workspace_bytes;
+    // grouped (mixture-of-experts) problems: rows sorted by expert, expert_rows[e] = rows of experts
+    // 0..e (device memory); m is then the total row count and the strides are bytes per expert
+    int64_t const* expert_rows = nullptr;
+    int num_experts = 0;
+    size_t weight_stride = 0, scale_stride = 0;
 };
 
 // kernel launchers (each returns a woq_status)

@@ -145,3 +145,29 @@ def test_last_error_is_per_thread(pkg):
     t.join()
     assert seen["msg"] == ""
     assert "group_size" in (L.lib.woq_last_error() or b"").decode()
+
+
+def test_grouped_matmul_validation(pkg):
+    """woq_grouped_matmul_check: the single-matrix checks on `base` plus the grouping arguments."""
+    import ctypes
+    L = pkg._lib
+
+    def gstatus(num_experts=4, total=0x7000, **kw):
+        g = L.GroupedMatmulArgs(base=make_args(L, **kw), total_rows_before_expert=total, num_experts=num_experts)
+        return L.lib.woq_grouped_matmul_check(ctypes.byref(g)), (L.lib.woq_last_error() or b"").decode()
+
+    assert gstatus()[0] == 0
+    assert gstatus(m=5000, regime=1)[0] == 0            # streaming passes cover any row count per expert
+    assert gstatus(bias=0x5000, quant_algo=L.ALGO_BIAS, group_size=0)[0] == 0
+    rc, msg = gstatus(total=None)
+    assert rc == -1 and "total_rows_before_expert" in msg
+    assert gstatus(total=None, m=0)[0] == 0             # nothing to do, nothing to read
+    rc, msg = gstatus(num_experts=0)
+    assert rc == -2 and "num_experts" in msg
+    rc, msg = gstatus(quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3)
+    assert rc == -3 and "not supported" in msg
+    rc, msg = gstatus(pre_quant_scale=0x5000, quant_algo=L.ALGO_PRE_QUANT_SCALE)
+    assert rc == -3 and "not supported" in msg
+    rc, msg = gstatus(k=96)                             # base checks still apply
+    assert rc == -2
+    assert L.lib.woq_grouped_matmul_check(None) == -1

@@ -188,3 +188,22 @@ def test_c_dequant_matmul_matches_numpy(oracle, oracle_c):
                                        ctypes.c_size_t(K), ctypes.c_size_t(G))
     w = q.astype(np.float32) * np.repeat(s, G, 0) + np.repeat(z, G, 0)
     assert oracle.max_rel_err(out, a.astype(np.float64) @ w.astype(np.float64)) < 1e-5
+
+
+def test_grouped_matmul_ref_is_a_per_row_expert_gather(oracle):
+    """The grouped reference against an independent formulation: every row multiplied with the
+    dequantized matrix of the expert that owns it (rows -> expert by searching the prefix sums)."""
+    rng = np.random.default_rng(5)
+    E, K, N = 4, 128, 32
+    rows = [3, 0, 5, 2]
+    total = np.cumsum(np.asarray(rows, np.int64))
+    q = rng.integers(-8, 8, size=(E, K, N)).astype(np.int8)
+    s = oracle.round_to(rng.uniform(0.01, 0.1, (E, K // 64, N)).astype(np.float32), "fp16")
+    z = oracle.round_to(rng.standard_normal((E, K // 64, N)).astype(np.float32) * 0.1, "fp16")
+    b = oracle.round_to(rng.standard_normal((E, N)).astype(np.float32), "fp16")
+    a = oracle.round_to(rng.standard_normal((10, K)).astype(np.float32), "fp16")
+    got = oracle.grouped_matmul_ref(a, q, s, z, b, total, 64, "fp16")
+    owner = np.searchsorted(total, np.arange(10), side="right")
+    w = np.stack([oracle.dequantize(q[e], s[e], z[e], 64, "fp16") for e in range(E)]).astype(np.float64)
+    want = np.einsum("rk,rkn->rn", a.astype(np.float64), w[owner]) + b[owner]
+    assert np.allclose(got, want, rtol=0, atol=1e-9)
