@@ -356,7 +356,8 @@ def run_moe_sweep(pkg, dev):
     rows + scales + activations + outputs) and TFLOP/s."""
     F = pkg.functional
     experts, top_k = 8, 2
-    for name, k, n in [("fc1 gate_up", 4096, 28672), ("fc2 down", 14336, 4096)]:
+    for name, k, n, activation in [("fc1 gate_up", 4096, 28672, "identity"), ("fc1 gate_up + swiglu", 4096, 28672, "swiglu"),
+                                   ("fc2 down", 14336, 4096, "identity")]:
         layers = [make_layer(pkg, dev, k, n, 6000 + e) for e in range(experts)]
         copies = copies_beyond_cache(experts * k * n // 2)
         weight = [torch.stack([l["weight"] for l in layers]).roll(r, 0).contiguous() for r in range(copies)]
@@ -370,18 +371,19 @@ def run_moe_sweep(pkg, dev):
             total = torch.cumsum(rows, 0).to(torch.int64).to(dev)
             m = int(rows.sum())
             act = torch.randn((m, k), device=dev).to(torch.bfloat16)
-            out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            n_out = n // 2 if activation == "swiglu" else n
+            out = torch.empty((m, n_out), dtype=torch.bfloat16, device=dev)
             reps = 20 if m <= 512 else 4
 
             def run(r):
                 F.woq_grouped_matmul_raw(act, weight[r % copies], scales, zeros, None, total, n=n, k=k,
-                                         group_size=GROUP, quant_algo=F.ZERO, out=out)
+                                         group_size=GROUP, quant_algo=F.ZERO, activation=activation, out=out)
             run(0)
             torch.cuda.synchronize()
             _, sec, launches = time_graph(lambda: [run(r) for r in range(reps)], reps, repeats=3)
             us = sec / launches * 1e6
             active = int((rows > 0).sum())
-            by = active * (k * n // 2 + (k // GROUP) * n * 4) + m * k * 2 + m * n * 2
+            by = active * (k * n // 2 + (k // GROUP) * n * 4) + m * k * 2 + m * n_out * 2
             print(json.dumps({"sweep": "moe", "shape": name, "k": k, "n": n, "experts": experts, "tokens": tokens,
                               "rows": m, "rows_per_expert": rows.tolist(), "us": round(us, 2),
                               "gbs": round(by / us / 1e3, 1), "tflops": round(2.0 * m * n * k / us / 1e6, 1)}),

@@ -158,18 +158,41 @@ size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, 
  *   total_rows_before_expert   device memory, int64 [num_experts]: rows of experts 0..e
  *                (inclusive prefix sums, non-decreasing, last = total_rows; the reference's
  *                total_tokens_including_expert); experts may own no rows
- * pre_quant_scale, FP8_ALPHA and the workspace are not used (must be NULL / unset).
+ *                With num_experts == 1 it may be NULL: the one expert owns all base.m rows
+ *                (the plain matmul with a fused activation).
+ *   activation   WOQ_ACT_* applied to (acc + bias) in float32, as moeGemmBiasAct's activation_type.
+ *                Gated ones (SWIGLU, GEGLU) read value column j and gate column j + n/2 and write
+ *                out [total_rows, n/2] = value * f(gate), the reference's chunk order
+ *                (functional.py:804-821, tests/functional/test_moe.py:186-190); n % 32 == 0 then.
+ *   base.workspace   only for a gated activation in the GEMM regime:
+ *                woq_grouped_workspace_bytes() bytes hold the [total_rows, n] pre-activation
+ *                values (the streaming regime applies every activation in its epilogue).
+ * pre_quant_scale and FP8_ALPHA are not supported (must be NULL / unset).
  * AUTO regime: the streaming kernel while the average expert has at most 16 rows (an expert with
  * more streams its weights once per 16 rows), tiled MFMA kernels above.
  */
+typedef enum woq_activation /* values of the reference's ActivationType (moe_gemm_kernels.h:197-206) */
+{
+    WOQ_ACT_GELU = 0,
+    WOQ_ACT_RELU = 1,
+    WOQ_ACT_SILU = 2,
+    WOQ_ACT_SWIGLU = 3,
+    WOQ_ACT_GEGLU = 4,
+    WOQ_ACT_IDENTITY = 5
+} woq_activation;
+
 typedef struct woq_grouped_matmul_args
 {
     woq_matmul_args base;
     const int64_t* total_rows_before_expert;
     int32_t num_experts;
+    int32_t activation; /* woq_activation; note that 0 is GELU, as in the reference */
 } woq_grouped_matmul_args;
 
 int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);
+
+/* Workspace a woq_grouped_matmul call may need (see base.workspace above); 0 unless gated. */
+size_t woq_grouped_workspace_bytes(int64_t total_rows, int32_t n, int32_t activation);
 
 /* Validation only (no launch): what woq_grouped_matmul would return for these arguments. */
 int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);

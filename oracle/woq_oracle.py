@@ -467,13 +467,28 @@ def woq_matmul_ref(act, q, scales, zeros=None, bias=None, pre_quant_scale=None, 
     return out
 
 
+def activation_ref(x, name: str) -> np.ndarray:
+    """The MoE activations in float64 (tests/functional/test_moe.py:173-190: torch gelu is the erf
+    form; a gated activation takes value = first half, gate = second half of the last axis and
+    returns value * f(gate), functional.py:804-821)."""
+    from scipy.special import erf
+    x = np.asarray(x, np.float64)
+    f = {"gelu": lambda v: 0.5 * v * (1.0 + erf(v / np.sqrt(2.0))), "relu": lambda v: np.maximum(v, 0.0),
+         "silu": lambda v: v / (1.0 + np.exp(-v)), "identity": lambda v: v}
+    if name in ("swiglu", "geglu"):
+        half = x.shape[-1] // 2
+        return x[..., :half] * f["silu" if name == "swiglu" else "gelu"](x[..., half:])
+    return f[name](x)
+
+
 def grouped_matmul_ref(act, q, scales, zeros, bias, total_rows_before_expert, group_size: int = 0,
-                       act_dtype: str = "bf16") -> np.ndarray:
-    """The MoE expert GEMM (MoeGemmRunner::moeGemm / moeGemmBiasAct without activation,
+                       act_dtype: str = "bf16", activation: str = "identity") -> np.ndarray:
+    """The MoE expert GEMM (MoeGemmRunner::moeGemm / moeGemmBiasAct,
     kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:235-244; the CUTLASS problem visitor
-    gives expert e the rows [total[e-1], total[e]), cutlass_extensions/gemm/kernel/moe_problem_visitor.h):
-    rows of expert e times ITS dequantized weight, plus its bias row.  q [E, K, N], scales / zeros
-    [E, N] or [E, K/g, N], bias [E, N]; float64 accumulation, not rounded."""
+    gives expert e the rows [total[e-1], total[e]), cutlass_extensions/gemm/kernel/moe_problem_visitor.h:163-176):
+    rows of expert e times ITS dequantized weight, plus its bias row, then the activation on the
+    unrounded sums (the fused epilogue's order, fused_moe_kernel_routine.cuh:380-400).  q [E, K, N],
+    scales / zeros [E, N] or [E, K/g, N], bias [E, N]; float64 accumulation, not rounded."""
     act = np.asarray(act, np.float32)
     total = np.asarray(total_rows_before_expert, np.int64)
     out = np.zeros((act.shape[0], np.asarray(q).shape[2]), np.float64)
@@ -484,7 +499,7 @@ def grouped_matmul_ref(act, q, scales, zeros, bias, total_rows_before_expert, gr
             out[begin:end] = woq_matmul_ref(act[begin:end], q[e], scales[e], None if zeros is None else zeros[e],
                                             None if bias is None else bias[e], None, 1.0, group_size, act_dtype)
         begin = end
-    return out
+    return activation_ref(out, activation)
 
 
 def max_rel_err(out, ref) -> float:

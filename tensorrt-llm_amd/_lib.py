@@ -13,6 +13,9 @@ FP16, BF16, FP8_E4M3, FP32 = 0, 1, 2, 3
 W8_A16, W4_A16, W4_AFP8 = 0, 1, 2
 ALGO_BIAS, ALGO_ZERO, ALGO_PRE_QUANT_SCALE, ALGO_FP8_ALPHA, ALGO_INT8_WEIGHT = 1, 2, 4, 8, 16
 REGIME_AUTO, REGIME_STREAM, REGIME_GEMM = 0, 1, 2
+ACT_GELU, ACT_RELU, ACT_SILU, ACT_SWIGLU, ACT_GEGLU, ACT_IDENTITY = 0, 1, 2, 3, 4, 5
+ACTIVATIONS = {"gelu": ACT_GELU, "relu": ACT_RELU, "silu": ACT_SILU, "swiglu": ACT_SWIGLU, "geglu": ACT_GEGLU,
+               "identity": ACT_IDENTITY}
 
 STATUS_NAMES = {
     0: "WOQ_OK", -1: "WOQ_ERR_INVALID_ARGUMENT", -2: "WOQ_ERR_BAD_SHAPE", -3: "WOQ_ERR_UNSUPPORTED",
@@ -41,7 +44,8 @@ class MatmulArgs(ctypes.Structure):
 
 
 class GroupedMatmulArgs(ctypes.Structure):
-    _fields_ = [("base", MatmulArgs), ("total_rows_before_expert", ctypes.c_void_p), ("num_experts", ctypes.c_int32)]
+    _fields_ = [("base", MatmulArgs), ("total_rows_before_expert", ctypes.c_void_p), ("num_experts", ctypes.c_int32),
+                ("activation", ctypes.c_int32)]
 
 
 def lib_path() -> str:
@@ -60,6 +64,7 @@ def _load():
         "woq_matmul_check": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
         "woq_grouped_matmul": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs), vp]),
         "woq_grouped_matmul_check": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs)]),
+        "woq_grouped_workspace_bytes": (sz, [i64, i32, i32]),
         "woq_workspace_bytes": (sz, [i32, i32, i32, i32, i32]),
         "woq_select_regime": (ctypes.c_int, [i32, i32, i32, i32]),
         "woq_preprocessed_bytes": (sz, [i64, i64, i32]),

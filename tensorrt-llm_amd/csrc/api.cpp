@@ -57,7 +57,7 @@ int launch_stream(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_stream_w4a8(p, stream);
-    if (!p.expert_rows && p.m > kStreamMaxM) // a grouped problem runs 16-row passes per expert
+    if (!p.num_experts && p.m > kStreamMaxM) // a grouped problem runs 16-row passes per expert
         return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the streaming kernel covers m <= %d (got %d)", kStreamMaxM,
             p.m);
     if (p.out_dtype == WOQ_BF16)
@@ -362,6 +362,13 @@ GemmPlan plan_grouped(int total_rows, int num_experts, int n)
 }
 } // namespace
 
+extern "C" size_t woq_grouped_workspace_bytes(int64_t total_rows, int32_t n, int32_t activation)
+{
+    if (total_rows <= 0 || n <= 0 || !(activation == WOQ_ACT_SWIGLU || activation == WOQ_ACT_GEGLU))
+        return 0;
+    return (size_t) total_rows * (size_t) n * 2;
+}
+
 extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
 {
     if (!args)
@@ -373,11 +380,24 @@ extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
         return fail(WOQ_ERR_UNSUPPORTED, "grouped matmul: FP8_ALPHA and PRE_QUANT_SCALE are not supported");
     if (args->num_experts <= 0)
         return fail(WOQ_ERR_BAD_SHAPE, "num_experts must be positive (got %d)", args->num_experts);
-    if (p.m > 0 && !args->total_rows_before_expert)
-        return fail(WOQ_ERR_INVALID_ARGUMENT, "total_rows_before_expert must not be NULL");
+    if (p.m > 0 && !args->total_rows_before_expert && args->num_experts != 1)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "total_rows_before_expert must not be NULL (unless num_experts is 1)");
+    int const act = args->activation;
+    if (act < WOQ_ACT_GELU || act > WOQ_ACT_IDENTITY)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown activation %d", act);
+    bool const gated = act == WOQ_ACT_SWIGLU || act == WOQ_ACT_GEGLU;
+    if (gated && p.n % 32)
+        return fail(WOQ_ERR_BAD_SHAPE, "a gated activation needs n %% 32 == 0 (got %d)", p.n);
     int const r = args->base.regime;
     if (r != WOQ_REGIME_AUTO && r != WOQ_REGIME_STREAM && r != WOQ_REGIME_GEMM)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", r);
+    if (p.m > 0 && gated && grouped_regime(args) == WOQ_REGIME_GEMM)
+    {
+        size_t const need = woq_grouped_workspace_bytes(p.m, p.n, act);
+        if (!p.workspace || p.workspace_bytes < need)
+            return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
+                p.workspace ? p.workspace_bytes : (size_t) 0);
+    }
     return WOQ_OK;
 }
 
@@ -389,15 +409,33 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     validate(&args->base, p);
     if (p.m == 0)
         return WOQ_OK;
-    p.expert_rows = args->total_rows_before_expert;
-    p.num_experts = args->num_experts;
     p.weight_stride = woq_preprocessed_bytes(p.k, p.n, p.bits == 8 ? WOQ_W8_A16 : WOQ_W4_A16);
     p.scale_stride = (size_t) (p.group_size ? p.k / p.group_size : 1) * (size_t) p.n * 2;
-    p.workspace = nullptr;
+    int const act = args->activation;
+    bool const gated = act == WOQ_ACT_SWIGLU || act == WOQ_ACT_GEGLU;
+    // without the prefix sums (one expert owning every row) the kernels take the row count from m
+    bool const single = !args->total_rows_before_expert;
+    p.expert_rows = args->total_rows_before_expert;
+    p.num_experts = args->num_experts;
+    void* const final_out = p.out;
+    void* const scratch = p.workspace;
+    p.workspace = nullptr; // K is never split here
     p.workspace_bytes = 0;
     if (grouped_regime(args) == WOQ_REGIME_STREAM)
+    {
+        p.activation = act; // the grouped streaming kernel carries the activation epilogue
         return launch_stream(p, stream);
-    return launch_gemm_planned(p, plan_grouped(p.m, p.num_experts, p.n), stream);
+    }
+    if (gated)
+        p.out = scratch; // pre-activation values [m, n]; the activation pass writes [m, n/2]
+    GemmPlan plan = single ? plan_gemm(p.m, p.n, p.k, p.bits) : plan_grouped(p.m, p.num_experts, p.n);
+    plan.k_splits = 1;
+    plan.ws_bytes = 0;
+    if (int rc = launch_gemm_planned(p, plan, stream))
+        return rc;
+    if (act == WOQ_ACT_IDENTITY)
+        return WOQ_OK;
+    return launch_activation(final_out, p.out, p.m, p.n, act, p.out_dtype, stream);
 }
 
 extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,

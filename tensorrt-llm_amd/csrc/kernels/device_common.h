@@ -261,6 +261,41 @@ __device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc,
     return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int) byte_offset, 0, 0);
 }
 
+// ---- epilogue activations (values of the reference's ActivationType,
+// kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:197-206) -------------------------
+constexpr int kActGelu = 0, kActRelu = 1, kActSilu = 2, kActSwiglu = 3, kActGeglu = 4, kActIdentity = 5;
+
+__host__ __device__ __forceinline__ bool act_is_gated(int act)
+{
+    return act == kActSwiglu || act == kActGeglu;
+}
+
+// erf by Abramowitz & Stegun 7.1.26 (|error| < 1.5e-7, far below the 16-bit output rounding)
+__device__ __forceinline__ float erf_approx(float x)
+{
+    float const ax = __builtin_fabsf(x);
+    float const t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, ax, 1.f));
+    float poly = __builtin_fmaf(1.061405429f, t, -1.453152027f);
+    poly = __builtin_fmaf(poly, t, 1.421413741f);
+    poly = __builtin_fmaf(poly, t, -0.284496736f);
+    poly = __builtin_fmaf(poly, t, 0.254829592f);
+    float const r = 1.f - poly * t * __expf(-ax * ax);
+    return __builtin_copysignf(r, x);
+}
+
+// the non-gated function of an activation (Swiglu -> silu, Geglu -> gelu), in float32 as the
+// reference's epilogues compute it (fused_moe_kernel_routine.cuh:393-400)
+__device__ __forceinline__ float apply_act(int act, float v)
+{
+    if (act == kActGelu || act == kActGeglu)
+        return 0.5f * v * (1.f + erf_approx(v * 0.70710678118654752f));
+    if (act == kActRelu)
+        return __builtin_fmaxf(v, 0.f);
+    if (act == kActSilu || act == kActSwiglu)
+        return v * __builtin_amdgcn_rcpf(1.f + __expf(-v));
+    return v;
+}
+
 // A pointer (or count) that is the same in every lane but was computed from loaded values: moved
 // into scalar registers, so that buffer descriptors built from it stay scalar too.
 template <typename T>

@@ -43,10 +43,12 @@ struct StreamParams
     int groups;         // ceil(strips / NS): column groups, one workgroup each
     int groups_per_xcd; // ceil(groups / 8)
     // grouped problems (rows sorted by expert, expert_rows[e] = rows of experts 0..e, device
-    // memory): blockIdx.y is the expert, strides are bytes per expert, m is unused
+    // memory): blockIdx.y is the expert, strides are bytes per expert; m is the total row count
+    // (and, without expert_rows, the row count of the only expert)
     int64_t const* expert_rows = nullptr;
     int num_experts = 0;
     size_t weight_stride = 0, scale_stride = 0;
+    int activation = kActIdentity; // epilogue activation (grouped kernel only)
 };
 
 // Everything one wavefront needs for one tile row (NS tiles side by side), fetched together so
@@ -66,7 +68,10 @@ struct StreamStage
 // WAVES wavefronts per workgroup; they split K (tile row kt goes to wave kt % WAVES)
 // PF    tile rows in flight per wavefront
 // ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
+// ACT   the epilogue applies p.activation; a gated activation (value column j, gate column j + n/2) pairs
+//       the strips of a wavefront (even slot: value half, odd slot: gate half), output [m, n/2]
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
+    bool ACT = false>
 __device__ __forceinline__ void stream_body(StreamParams const& p)
 {
     static_assert(!ALDS || MT == 1, "LDS-staged activations are for M <= 16");
@@ -122,12 +127,20 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
 
     // strips past the end of N (last group only) are clamped for loads and skipped at the store
+    bool const gated = ACT && act_is_gated(p.activation);
+    int const half_strips = p.strips / 2;
     int strip_of[NS];
     uint32_t wlane[NS]; // byte offset of this lane's 16 bytes in tile row 0 of each strip
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        if (gated)
+        {
+            int const pair = strip0 / 2 + s / 2; // NS is even: this group's pairs are strip0/2 ..
+            strip_of[s] = (pair < half_strips ? pair : half_strips - 1) + (s & 1) * half_strips;
+        }
+        else
+            strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
         wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
     }
 
@@ -333,6 +346,39 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     __syncthreads();
 
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    if (gated)
+    {
+        // value and gate sums sit in neighbouring strip slots: out = (x + bias_x) * f(g + bias_g)
+        if constexpr (ACT && NS % 2 == 0)
+        {
+            int const n_out = p.n / 2;
+            for (int e = threadIdx.x; e < SLOTS / 2 * 64; e += WAVES * 64)
+            {
+                int const pslot = e >> 6, ln = e & 63; // (pair, mt, r)
+                int const ps = pslot / (MT * 4), mt = (pslot >> 2) % MT, r = pslot & 3;
+                int const row = mt * 16 + (ln >> 4) * 4 + r;
+                int const pair = strip0 / 2 + ps;
+                if (row >= p.m || pair >= half_strips)
+                    continue;
+                int const slot_x = ((2 * ps) * MT + mt) * 4 + r, slot_g = ((2 * ps + 1) * MT + mt) * 4 + r;
+                float x = 0.f, g = 0.f;
+#pragma unroll
+                for (int w2 = 0; w2 < WAVES; ++w2)
+                {
+                    x += red[w2][slot_x][ln];
+                    g += red[w2][slot_g][ln];
+                }
+                int const ocol = pair * 16 + (ln & 15);
+                if (p.bias)
+                {
+                    x += E::load(p.bias, ocol);
+                    g += E::load(p.bias, ocol + n_out);
+                }
+                out16[(size_t) row * n_out + ocol] = E::store(x * apply_act(p.activation, g));
+            }
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < SLOTS * 64; e += WAVES * 64)
     {
         int const slot = e >> 6, ln = e & 63;
@@ -348,6 +394,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         float v = p.alpha * sum;
         if (p.bias)
             v += E::load(p.bias, ocol);
+        if constexpr (ACT)
+            v = apply_act(p.activation, v);
         out16[(size_t) row * p.n + ocol] = E::store(v);
     }
 }
@@ -365,10 +413,16 @@ template <int DT, int BITS, int GROUP, bool ZERO, int NS, int WAVES, int PF, boo
 __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams p)
 {
     int const e = (int) blockIdx.y;
-    int64_t const begin = e ? p.expert_rows[e - 1] : 0;
-    int rows_left = __builtin_amdgcn_readfirstlane((int) (p.expert_rows[e] - begin));
+    int64_t begin = 0;
+    int rows_left = p.m; // no prefix sums: one expert owns every row
+    if (p.expert_rows)
+    {
+        begin = e ? p.expert_rows[e - 1] : 0;
+        rows_left = __builtin_amdgcn_readfirstlane((int) (p.expert_rows[e] - begin));
+    }
     p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
-    p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) p.n * 2);
+    int const n_out = act_is_gated(p.activation) ? p.n / 2 : p.n;
+    p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) n_out * 2);
     p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
     p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
     if (ZERO)
@@ -378,10 +432,10 @@ __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams
     for (; rows_left > 0; rows_left -= 16)
     {
         p.m = rows_left;
-        stream_body<DT, BITS, GROUP, false, ZERO, 1, NS, WAVES, PF, ALDS>(p);
+        stream_body<DT, BITS, GROUP, false, ZERO, 1, NS, WAVES, PF, ALDS, true>(p);
         __syncthreads(); // this pass is done with the LDS areas
         p.act = static_cast<char const*>(p.act) + (size_t) 16 * (size_t) p.k * 2;
-        p.out = static_cast<char*>(p.out) + (size_t) 16 * (size_t) p.n * 2;
+        p.out = static_cast<char*>(p.out) + (size_t) 16 * (size_t) n_out * 2;
     }
 }
 
@@ -480,7 +534,9 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
     // every expert's column groups run side by side: the grid is num_experts times taller
-    StreamShape const sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK);
+    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK);
+    if (act_is_gated(sp.activation) && sh.ns == 1) // value and gate strips pair up inside a wavefront
+        sh = sh.lds ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, 0};
 #define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
     if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                                   \
         return launch_stream_variant<DT, BITS, GROUP, false, ZERO, 1, NS_, WAVES_, PF_, LDS_, true>(sp, s);
@@ -518,11 +574,12 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.num_experts = p.num_experts;
     sp.weight_stride = p.weight_stride;
     sp.scale_stride = p.scale_stride;
+    sp.activation = p.activation;
     auto s = static_cast<hipStream_t>(stream);
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;
     bool const zero = p.zeros != nullptr;
-    if (p.expert_rows)
+    if (p.num_experts)
     {
         switch (p.group_size)
         {

@@ -27,27 +27,27 @@ def grouped_problem(oracle, rows, K, N, bits, group, dtype, zero, bias, seed):
     return p
 
 
-def run_grouped(pkg, oracle, dev, p, regime=0):
+def run_grouped(pkg, oracle, dev, p, regime=0, activation="identity", single=False):
     F = pkg.functional
     dt = p["dtype"]
     w = torch.stack([preprocess(pkg, oracle, p["q"][e], p["bits"]) for e in range(len(p["rows"]))]).to(dev)
     algo = (F.INT8_WEIGHT if p["bits"] == 8 else 0) | (F.ZERO if p["zeros"] is not None else 0) \
         | (F.BIAS if p["bias"] is not None else 0)
     opt = lambda x: None if x is None else to_dev(x, dt, dev)
-    total = torch.from_numpy(p["total"]).to(dev)
-    # a recognisable fill: rows that belong to no expert must stay untouched (there are none), and
-    # every row that does must be written
-    out = torch.full((p["act"].shape[0], p["N"]), float("nan"), dtype=TORCH_DT[dt], device=dev)
+    total = None if single else torch.from_numpy(p["total"]).to(dev)
+    # a recognisable fill: every row belongs to some expert and must be written
+    n_out = p["N"] // 2 if activation in ("swiglu", "geglu") else p["N"]
+    out = torch.full((p["act"].shape[0], n_out), float("nan"), dtype=TORCH_DT[dt], device=dev)
     F.woq_grouped_matmul_raw(to_dev(p["act"], dt, dev), w, to_dev(p["scales"], dt, dev), opt(p["zeros"]),
                              opt(p["bias"]), total, n=p["N"], k=p["K"], group_size=p["group"], quant_algo=algo,
-                             regime=regime, out=out)
+                             activation=activation, regime=regime, out=out)
     torch.cuda.synchronize()
     return out.float().cpu().numpy()
 
 
-def reference(oracle, p):
+def reference(oracle, p, activation="identity"):
     return oracle.grouped_matmul_ref(p["act"], p["q"], p["scales"], p["zeros"], p["bias"], p["total"], p["group"],
-                                     p["dtype"])
+                                     p["dtype"], activation)
 
 
 @pytest.mark.parametrize("rows", [[3, 0, 16, 1], [40, 0, 5, 17], [0, 0, 7, 0], [1, 1, 1, 1, 1, 1, 1, 1]])
@@ -103,6 +103,37 @@ def test_grouped_single_expert_equals_plain_matmul(pkg, oracle, dev):
     # the plain call may split K (fewer tiles than CUs), the grouped one never does: same bar, not same bits
     assert oracle.max_rel_err(out, plain.float().cpu().numpy()) < 2e-3
     assert oracle.max_rel_err(out, reference(oracle, p)) < TOL
+
+
+@pytest.mark.parametrize("activation", ["gelu", "relu", "silu", "swiglu", "geglu"])
+@pytest.mark.parametrize("rows", [[3, 0, 16, 1], [40, 5], [90, 0, 70, 33]])
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_grouped_activations(pkg, oracle, dev, activation, rows, dtype):
+    """moeGemmBiasAct's activations: fused into the streaming kernel's epilogue (few rows per expert,
+    with strips paired for the gated ones) or applied by the activation pass behind the tiled
+    kernels.  N = 544: a gated output of 272 columns, the last workgroup's strips only partly there."""
+    p = grouped_problem(oracle, rows, 512, 544, 4, 128, dtype, True, True, seed=len(activation) + sum(rows))
+    out = run_grouped(pkg, oracle, dev, p, activation=activation)
+    assert np.isfinite(out).all()
+    assert oracle.max_rel_err(out, reference(oracle, p, activation)) < TOL
+
+
+@pytest.mark.parametrize("regime", [STREAM, GEMM])
+@pytest.mark.parametrize("bits,group", [(8, 0), (4, 64)])
+def test_grouped_swiglu_forced_regimes(pkg, oracle, dev, regime, bits, group):
+    p = grouped_problem(oracle, [7, 20, 0, 9], 1024, 288, bits, group, "bf16", group != 0, True, seed=31)
+    out = run_grouped(pkg, oracle, dev, p, regime=regime, activation="swiglu")
+    assert oracle.max_rel_err(out, reference(oracle, p, "swiglu")) < TOL
+
+
+@pytest.mark.parametrize("M", [1, 9, 300])
+@pytest.mark.parametrize("activation", ["identity", "swiglu", "gelu"])
+def test_single_expert_without_prefix_sums(pkg, oracle, dev, M, activation):
+    """num_experts = 1 and no prefix sums: the plain matmul with a fused activation."""
+    p = grouped_problem(oracle, [M], 512, 544, 4, 128, "bf16", True, True, seed=M)
+    out = run_grouped(pkg, oracle, dev, p, activation=activation, single=True)
+    assert np.isfinite(out).all()
+    assert oracle.max_rel_err(out, reference(oracle, p, activation)) < TOL
 
 
 def test_grouped_rejections(pkg, oracle, dev):

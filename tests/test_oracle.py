@@ -207,3 +207,18 @@ def test_grouped_matmul_ref_is_a_per_row_expert_gather(oracle):
     w = np.stack([oracle.dequantize(q[e], s[e], z[e], 64, "fp16") for e in range(E)]).astype(np.float64)
     want = np.einsum("rk,rkn->rn", a.astype(np.float64), w[owner]) + b[owner]
     assert np.allclose(got, want, rtol=0, atol=1e-9)
+
+
+def test_activation_ref_known_values(oracle):
+    """Closed-form points of the activation restatement: silu(0) = 0, silu(x) - silu(-x) = x,
+    gelu(x) - gelu(-x) = x, gelu(1) = Phi(1), relu; the gated forms take value = first half."""
+    x = np.array([-3.0, -1.0, 0.0, 0.5, 1.0, 4.0])
+    silu, gelu = oracle.activation_ref(x, "silu"), oracle.activation_ref(x, "gelu")
+    assert silu[2] == 0 and np.allclose(silu - oracle.activation_ref(-x, "silu"), x)
+    assert np.allclose(gelu - oracle.activation_ref(-x, "gelu"), x)
+    assert abs(gelu[4] - 0.8413447460685429) < 1e-12 and abs(silu[4] - 0.7310585786300049) < 1e-12
+    assert (oracle.activation_ref(x, "relu") == np.maximum(x, 0)).all()
+    assert (oracle.activation_ref(x, "identity") == x).all()
+    pair = np.array([[2.0, 3.0, 1.0, -1.0]])  # value (2, 3), gate (1, -1)
+    assert np.allclose(oracle.activation_ref(pair, "swiglu"), [[2.0 * silu[4], 3.0 * silu[1]]])
+    assert np.allclose(oracle.activation_ref(pair, "geglu"), [[2.0 * gelu[4], 3.0 * gelu[1]]])
