@@ -270,6 +270,37 @@ def run_for_counters(pkg, dev, mode, reps=20):
         print(json.dumps({"mode": "copy", "bytes_read_per_launch": 256 << 20, "bytes_written_per_launch": 256 << 20,
                           "launches": reps}))
         return
+    if mode == "w4a8_decode":
+        _, k, n = SHAPES_70B[2]
+        copies = copies_beyond_cache(k * n // 2)
+        run = w4a8_setup(pkg, dev, 1, k, n, copies=copies)
+        for r in range(reps):
+            run(r)
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": mode, "kernel": "W4A8 streaming kernel on 70B gate_up K=8192 N=57344 M=1",
+                          "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n, 4, GROUP, 1, 1), "launches": reps}))
+        return
+    if mode == "moe_decode":
+        F = pkg.functional
+        experts, k, n = 8, 4096, 28672
+        layers = [make_layer(pkg, dev, k, n, 6000 + e) for e in range(experts)]
+        copies = copies_beyond_cache(experts * k * n // 2)
+        weight = [torch.stack([l["weight"] for l in layers]).roll(r, 0).contiguous() for r in range(copies)]
+        scales = torch.stack([l["scales"] for l in layers]).contiguous()
+        zeros = torch.stack([l["zeros"] for l in layers]).contiguous()
+        rows = torch.tensor([5, 1, 4, 4, 6, 3, 8, 1])
+        total = torch.cumsum(rows, 0).to(torch.int64).to(dev)
+        act = torch.randn((int(rows.sum()), k), device=dev).to(torch.bfloat16)
+        out = torch.empty((act.shape[0], n // 2), dtype=torch.bfloat16, device=dev)
+        for r in range(reps):
+            F.woq_grouped_matmul_raw(act, weight[r % copies], scales, zeros, None, total, n=n, k=k, group_size=GROUP,
+                                     quant_algo=F.ZERO, activation="swiglu", out=out)
+        torch.cuda.synchronize()
+        by = experts * (k * n // 2 + (k // GROUP) * n * 4) + act.numel() * 2 + out.numel() * 2
+        print(json.dumps({"mode": mode, "kernel": "grouped streaming kernel, 8 experts K=4096 N=28672 + swiglu, "
+                                                  "32 rows (16 tokens, top-2)",
+                          "algorithmic_bytes_per_launch": by, "launches": reps}))
+        return
     _, k, n = SHAPES_8B[2]
     if mode == "w4a8_4096":
         run = w4a8_setup(pkg, dev, 4096, k, n)
@@ -399,7 +430,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "sweep"],
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "w4a8_decode", "moe_decode",
+                                       "sweep"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
