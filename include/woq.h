@@ -164,10 +164,7 @@ size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, 
  *                Gated ones (SWIGLU, GEGLU) read value column j and gate column j + n/2 and write
  *                out [total_rows, n/2] = value * f(gate), the reference's chunk order
  *                (functional.py:804-821, tests/functional/test_moe.py:186-190); n % 32 == 0 then.
- *   base.workspace   only for a gated activation in the GEMM regime:
- *                woq_grouped_workspace_bytes() bytes hold the [total_rows, n] pre-activation
- *                values (the streaming regime applies every activation in its epilogue).
- * pre_quant_scale and FP8_ALPHA are not supported (must be NULL / unset).
+ * pre_quant_scale, FP8_ALPHA and the workspace are not used (must be NULL / unset).
  * AUTO regime: the streaming kernel while the average expert has at most 16 rows (an expert with
  * more streams its weights once per 16 rows), tiled MFMA kernels above.
  */
@@ -190,9 +187,6 @@ typedef struct woq_grouped_matmul_args
 } woq_grouped_matmul_args;
 
 int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);
-
-/* Workspace a woq_grouped_matmul call may need (see base.workspace above); 0 unless gated. */
-size_t woq_grouped_workspace_bytes(int64_t total_rows, int32_t n, int32_t activation);
 
 /* Validation only (no launch): what woq_grouped_matmul would return for these arguments. */
 int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);

@@ -64,7 +64,6 @@ def _load():
         "woq_matmul_check": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
         "woq_grouped_matmul": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs), vp]),
         "woq_grouped_matmul_check": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs)]),
-        "woq_grouped_workspace_bytes": (sz, [i64, i32, i32]),
         "woq_workspace_bytes": (sz, [i32, i32, i32, i32, i32]),
         "woq_select_regime": (ctypes.c_int, [i32, i32, i32, i32]),
         "woq_preprocessed_bytes": (sz, [i64, i64, i32]),

@@ -362,13 +362,6 @@ GemmPlan plan_grouped(int total_rows, int num_experts, int n)
 }
 } // namespace
 
-extern "C" size_t woq_grouped_workspace_bytes(int64_t total_rows, int32_t n, int32_t activation)
-{
-    if (total_rows <= 0 || n <= 0 || !(activation == WOQ_ACT_SWIGLU || activation == WOQ_ACT_GEGLU))
-        return 0;
-    return (size_t) total_rows * (size_t) n * 2;
-}
-
 extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
 {
     if (!args)
@@ -391,13 +384,6 @@ extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
     int const r = args->base.regime;
     if (r != WOQ_REGIME_AUTO && r != WOQ_REGIME_STREAM && r != WOQ_REGIME_GEMM)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", r);
-    if (p.m > 0 && gated && grouped_regime(args) == WOQ_REGIME_GEMM)
-    {
-        size_t const need = woq_grouped_workspace_bytes(p.m, p.n, act);
-        if (!p.workspace || p.workspace_bytes < need)
-            return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
-                p.workspace ? p.workspace_bytes : (size_t) 0);
-    }
     return WOQ_OK;
 }
 
@@ -417,25 +403,21 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     bool const single = !args->total_rows_before_expert;
     p.expert_rows = args->total_rows_before_expert;
     p.num_experts = args->num_experts;
-    void* const final_out = p.out;
-    void* const scratch = p.workspace;
     p.workspace = nullptr; // K is never split here
     p.workspace_bytes = 0;
-    if (grouped_regime(args) == WOQ_REGIME_STREAM)
-    {
-        p.activation = act; // the grouped streaming kernel carries the activation epilogue
+    // every kernel applies a gated activation in its epilogue; the streaming kernel the others too
+    bool const streaming = grouped_regime(args) == WOQ_REGIME_STREAM;
+    p.activation = (streaming || gated) ? act : WOQ_ACT_IDENTITY;
+    if (streaming)
         return launch_stream(p, stream);
-    }
-    if (gated)
-        p.out = scratch; // pre-activation values [m, n]; the activation pass writes [m, n/2]
     GemmPlan plan = single ? plan_gemm(p.m, p.n, p.k, p.bits) : plan_grouped(p.m, p.num_experts, p.n);
     plan.k_splits = 1;
     plan.ws_bytes = 0;
     if (int rc = launch_gemm_planned(p, plan, stream))
         return rc;
-    if (act == WOQ_ACT_IDENTITY)
+    if (act == WOQ_ACT_IDENTITY || gated)
         return WOQ_OK;
-    return launch_activation(final_out, p.out, p.m, p.n, act, p.out_dtype, stream);
+    return launch_activation(p.out, p.out, p.m, p.n, act, p.out_dtype, stream); // elementwise, in place
 }
 
 extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,

@@ -28,10 +28,30 @@ struct GemmParams
     int64_t const* expert_rows = nullptr;
     int num_experts = 0;
     size_t weight_stride = 0, scale_stride = 0;
+    // kActSwiglu / kActGeglu: the epilogue multiplies value column j with f(gate column j + n/2)
+    // and writes [m, n/2]; the strips of a wavefront then alternate between the two halves of N
+    // (see paired_strip).  Other activations are applied by a separate pass.
+    int activation = kActIdentity;
 };
+
+// Strip slot s of a wavefront whose first slot is `first` (even): without a gated activation strip
+// first + s; with one, slots pair up - even slot: pair (first + s) / 2 in the value half, odd
+// slot: the same pair in the gate half, `half` strips further.  `valid`: the slot's strip exists.
+__device__ __forceinline__ int paired_strip(bool gated, int first, int s, int strips, bool& valid)
+{
+    if (!gated)
+    {
+        valid = first + s < strips;
+        return valid ? first + s : strips - 1;
+    }
+    int const half = strips / 2, pair = first / 2 + s / 2;
+    valid = pair < half;
+    return (valid ? pair : half - 1) + (s & 1) * half;
+}
 
 inline void set_group_fields(GemmParams& gp, MatmulProblem const& p, int tile_rows)
 {
+    gp.activation = act_is_gated(p.activation) ? p.activation : kActIdentity;
     gp.expert_rows = p.expert_rows;
     gp.num_experts = p.num_experts;
     gp.weight_stride = p.weight_stride;
@@ -56,7 +76,8 @@ __device__ __forceinline__ bool select_expert(GemmParams& p, int& tm, int tile_r
         if (tm < first_tile + tiles)
         {
             p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
-            p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) p.n * 2);
+            p.out = uniform_ptr(static_cast<char*>(p.out)
+                + (size_t) begin * (size_t) (act_is_gated(p.activation) ? p.n / 2 : p.n) * 2);
             p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
             p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
             if (p.zeros)

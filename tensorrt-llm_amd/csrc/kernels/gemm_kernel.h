@@ -21,6 +21,8 @@
 #pragma once
 
 #include "dequant_math.h"
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace woq
@@ -86,12 +88,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
 
+    bool const gated = !SPLITK && act_is_gated(p.activation);
+    bool strip_ok[NS];
     int strip_of[NS];
     uint32_t wlane[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        strip_of[s] = paired_strip(gated, strip0, s, p.strips, strip_ok[s]);
         wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
     }
 
@@ -347,12 +351,48 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    if (gated)
+    {
+        // value and gate sums of an output element sit in neighbouring strip slots of this lane
+        if constexpr (!SPLITK)
+        {
+            int const n_out = p.n / 2;
+            auto gated_epilogue = [&](auto act_tag)
+            {
+                constexpr int ACT = decltype(act_tag)::value;
+#pragma unroll
+                for (int s = 0; s < NS; s += 2)
+                {
+                    if (!strip_ok[s])
+                        continue;
+                    int const col = strip_of[s] * 16 + c; // strip_of[s] is the pair index (value half)
+                    float const bias_x = p.bias ? E::load(p.bias, col) : 0.f;
+                    float const bias_g = p.bias ? E::load(p.bias, col + n_out) : 0.f;
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                        {
+                            int const row = m0 + rt * 16 + kg * 4 + r;
+                            if (row < p.m)
+                                out16[(size_t) row * n_out + col] = E::store(
+                                    (acc[rt][s][r] + bias_x) * apply_act(ACT, acc[rt][s + 1][r] + bias_g));
+                        }
+                }
+            };
+            if (p.activation == kActSwiglu)
+                gated_epilogue(std::integral_constant<int, kActSwiglu>{});
+            else
+                gated_epilogue(std::integral_constant<int, kActGeglu>{});
+        }
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        if (strip0 + s >= p.strips)
+        if (!strip_ok[s])
             continue;
-        int const col = (strip0 + s) * 16 + c;
+        int const col = strip_of[s] * 16 + c;
         float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)

@@ -16,6 +16,8 @@
 // of the lane that feeds them to the matrix core.
 #pragma once
 
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace woq
@@ -80,12 +82,14 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
 
+    bool const gated = !SPLITK && act_is_gated(p.activation);
+    bool strip_ok[NS];
     int strip_of[NS];
     uint32_t wlane[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
+        strip_of[s] = paired_strip(gated, strip0, s, p.strips, strip_ok[s]);
         wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
     }
 
@@ -141,8 +145,8 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
 
     // Scales (and zeros) of the wavefront's 16*NS columns for one group, fetched by the first 8*NS
     // lanes as dwords straight into LDS (the other lanes get zeros from an out-of-range offset).
-    int const col0 = strip0 * 16;
-    uint32_t const sc_lane_col = (uint32_t) (col0 + 2 * (lane & 31));
+    static_assert(NS == 2, "the scale fetch below picks between two strips");
+    uint32_t const sc_lane_col = (uint32_t) (((lane & 31) < 8 ? strip_of[0] : strip_of[1]) * 16 + 2 * (lane & 7));
     uint32_t const sc_lane_oob = (lane >= 8 * NS || (int) sc_lane_col >= p.n) ? kOob : 0u;
 
     auto fetch_b = [&](Stage& st, int buf, int kt)
@@ -355,12 +359,54 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
 
     // ---- epilogue ----------------------------------------------------------------------------
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    // finished sum of (row tile, strip slot, register): per-channel scales are applied here
+    auto finished = [&](int rt, int s, int r, float pc) -> float
+    {
+        float v = acc[rt][s][r];
+        if constexpr (GROUP == 0)
+            v = __builtin_fmaf(pc, v, (-OFF * pc) * acc_s[rt][r]);
+        return v;
+    };
+    if (gated)
+    {
+        // value and gate sums of an output element sit in the two strip slots of this lane
+        if constexpr (!SPLITK)
+        {
+            int const n_out = p.n / 2;
+            auto gated_epilogue = [&](auto act_tag)
+            {
+                constexpr int ACT = decltype(act_tag)::value;
+                if (!strip_ok[0])
+                    return;
+                int const col = strip_of[0] * 16 + c; // strip_of[0] is the pair index (value half)
+                float const bias_x = p.bias ? E::load(p.bias, col) : 0.f;
+                float const bias_g = p.bias ? E::load(p.bias, col + n_out) : 0.f;
+                [[maybe_unused]] float const pc_x = GROUP == 0 ? E::load(p.scales, col) : 0.f;
+                [[maybe_unused]] float const pc_g = GROUP == 0 ? E::load(p.scales, col + n_out) : 0.f;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                    {
+                        int const row = m0 + rt * 16 + kg * 4 + r;
+                        if (row < p.m)
+                            out16[(size_t) row * n_out + col] = E::store((finished(rt, 0, r, pc_x) + bias_x)
+                                * apply_act(ACT, finished(rt, 1, r, pc_g) + bias_g));
+                    }
+            };
+            if (p.activation == kActSwiglu)
+                gated_epilogue(std::integral_constant<int, kActSwiglu>{});
+            else
+                gated_epilogue(std::integral_constant<int, kActGeglu>{});
+        }
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        if (strip0 + s >= p.strips)
+        if (!strip_ok[s])
             continue;
-        int const col = (strip0 + s) * 16 + c;
+        int const col = strip_of[s] * 16 + c;
         float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
         [[maybe_unused]] float const pc = GROUP == 0 ? E::load(p.scales, col) : 0.f;
 #pragma unroll
@@ -370,9 +416,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             for (int r = 0; r < 4; ++r)
             {
                 int const row = m0 + rt * 16 + kg * 4 + r;
-                float v = acc[rt][s][r];
-                if constexpr (GROUP == 0)
-                    v = __builtin_fmaf(pc, v, (-OFF * pc) * acc_s[rt][r]);
+                float const v = finished(rt, s, r, pc);
                 if (row < p.m)
                 {
                     if constexpr (SPLITK)

@@ -87,13 +87,11 @@ def woq_grouped_matmul_raw(act, weight, scales, zeros, bias, total_rows_before_e
     n_out = n // 2 if activation in ("swiglu", "geglu") else n
     if out is None:
         out = torch.empty((act.shape[0], n_out), dtype=act.dtype, device=act.device)
-    need = lib.woq_grouped_workspace_bytes(act.shape[0], n, act_id)
-    workspace = torch.empty(need, dtype=torch.uint8, device=act.device) if need else None
     base = MatmulArgs(
         act=_ptr(act), pre_quant_scale=None, weight=_ptr(weight), scales=_ptr(scales), zeros=_ptr(zeros),
         bias=_ptr(bias), out=_ptr(out), alpha=1.0, m=act.shape[0], n=n, k=k, group_size=group_size,
         quant_algo=quant_algo, act_dtype=_WOQ_DT[act.dtype], out_dtype=_WOQ_DT[act.dtype], regime=regime,
-        workspace=_ptr(workspace), workspace_bytes=need)
+        workspace=None, workspace_bytes=0)
     experts = 1 if total_rows_before_expert is None else total_rows_before_expert.numel()
     args = GroupedMatmulArgs(base=base, total_rows_before_expert=_ptr(total_rows_before_expert), num_experts=experts,
                              activation=act_id)

@@ -174,16 +174,11 @@ def test_grouped_matmul_validation(pkg):
     assert L.lib.woq_grouped_matmul_check(None) == -1
     # one expert may come without prefix sums; more may not
     assert gstatus(num_experts=1, total=None)[0] == 0
-    # activations: every value of the reference's enum; gated ones need n % 32 == 0 and, in the GEMM
-    # regime, a workspace for the pre-activation values
+    # activations: every value of the reference's enum; gated ones need n % 32 == 0
     for act in range(6):
         assert gstatus(activation=act, n=256)[0] == 0
     rc, msg = gstatus(activation=6)
     assert rc == -1 and "activation" in msg
     rc, msg = gstatus(activation=L.ACT_SWIGLU, n=48)
     assert rc == -2 and "32" in msg
-    rc, msg = gstatus(activation=L.ACT_SWIGLU, m=4096, n=256)
-    assert rc == -4 and "workspace" in msg
-    need = L.lib.woq_grouped_workspace_bytes(4096, 256, L.ACT_SWIGLU)
-    assert need == 4096 * 256 * 2 and L.lib.woq_grouped_workspace_bytes(4096, 256, L.ACT_GELU) == 0
-    assert gstatus(activation=L.ACT_SWIGLU, m=4096, n=256, workspace=0x9000, workspace_bytes=need)[0] == 0
+    assert gstatus(activation=L.ACT_SWIGLU, m=4096, n=256)[0] == 0
