@@ -437,8 +437,8 @@ def main():
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the op shards with no "
-                 "communication inside it, see DESIGN.md")
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1): the op contains no communication, a "
+                 "tensor-parallel model gives each GPU its own column or row slice of the weights")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the matmul has no CPU path")
     pkg = import_package()

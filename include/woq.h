@@ -164,6 +164,9 @@ size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, 
  *                Gated ones (SWIGLU, GEGLU) read value column j and gate column j + n/2 and write
  *                out [total_rows, n/2] = value * f(gate), the reference's chunk order
  *                (functional.py:804-821, tests/functional/test_moe.py:186-190); n % 32 == 0 then.
+ *   residual     optional [total_rows, n_out], same type as out: out = T(f(acc + bias) + residual),
+ *                the skip connection behind o_proj / down projections (no counterpart in the
+ *                reference's GEMM runners, which leave it to a following elementwise layer).
  * pre_quant_scale, FP8_ALPHA and the workspace are not used (must be NULL / unset).
  * AUTO regime: the streaming kernel while the average expert has at most 16 rows (an expert with
  * more streams its weights once per 16 rows), tiled MFMA kernels above.
@@ -183,7 +186,8 @@ typedef struct woq_grouped_matmul_args
     woq_matmul_args base;
     const int64_t* total_rows_before_expert;
     int32_t num_experts;
-    int32_t activation; /* woq_activation; note that 0 is GELU, as in the reference */
+    int32_t activation;   /* woq_activation; note that 0 is GELU, as in the reference */
+    const void* residual; /* NULL, or [total_rows, n_out] in the output type: added after the activation */
 } woq_grouped_matmul_args;
 
 int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);

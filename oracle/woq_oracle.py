@@ -482,13 +482,14 @@ def activation_ref(x, name: str) -> np.ndarray:
 
 
 def grouped_matmul_ref(act, q, scales, zeros, bias, total_rows_before_expert, group_size: int = 0,
-                       act_dtype: str = "bf16", activation: str = "identity") -> np.ndarray:
+                       act_dtype: str = "bf16", activation: str = "identity", residual=None) -> np.ndarray:
     """The MoE expert GEMM (MoeGemmRunner::moeGemm / moeGemmBiasAct,
     kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:235-244; the CUTLASS problem visitor
     gives expert e the rows [total[e-1], total[e]), cutlass_extensions/gemm/kernel/moe_problem_visitor.h:163-176):
     rows of expert e times ITS dequantized weight, plus its bias row, then the activation on the
     unrounded sums (the fused epilogue's order, fused_moe_kernel_routine.cuh:380-400).  q [E, K, N],
-    scales / zeros [E, N] or [E, K/g, N], bias [E, N]; float64 accumulation, not rounded."""
+    scales / zeros [E, N] or [E, K/g, N], bias [E, N]; float64 accumulation, not rounded.  `residual`
+    (an extension of this library, the skip connection) is added last."""
     act = np.asarray(act, np.float32)
     total = np.asarray(total_rows_before_expert, np.int64)
     out = np.zeros((act.shape[0], np.asarray(q).shape[2]), np.float64)
@@ -499,7 +500,8 @@ def grouped_matmul_ref(act, q, scales, zeros, bias, total_rows_before_expert, gr
             out[begin:end] = woq_matmul_ref(act[begin:end], q[e], scales[e], None if zeros is None else zeros[e],
                                             None if bias is None else bias[e], None, 1.0, group_size, act_dtype)
         begin = end
-    return activation_ref(out, activation)
+    out = activation_ref(out, activation)
+    return out if residual is None else out + np.asarray(residual, np.float64)
 
 
 def max_rel_err(out, ref) -> float:

@@ -45,7 +45,7 @@ class MatmulArgs(ctypes.Structure):
 
 class GroupedMatmulArgs(ctypes.Structure):
     _fields_ = [("base", MatmulArgs), ("total_rows_before_expert", ctypes.c_void_p), ("num_experts", ctypes.c_int32),
-                ("activation", ctypes.c_int32)]
+                ("activation", ctypes.c_int32), ("residual", ctypes.c_void_p)]
 
 
 def lib_path() -> str:

@@ -384,6 +384,9 @@ extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
     int const r = args->base.regime;
     if (r != WOQ_REGIME_AUTO && r != WOQ_REGIME_STREAM && r != WOQ_REGIME_GEMM)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", r);
+    // the kernels address the residual with 32-bit byte offsets
+    if (args->residual && (uint64_t) p.m * (uint64_t) p.n * 2 >= ((uint64_t) 1 << 32))
+        return fail(WOQ_ERR_UNSUPPORTED, "residual: total_rows * n * 2 must stay below 4 GiB (got %d x %d)", p.m, p.n);
     return WOQ_OK;
 }
 
@@ -408,16 +411,20 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     // every kernel applies a gated activation in its epilogue; the streaming kernel the others too
     bool const streaming = grouped_regime(args) == WOQ_REGIME_STREAM;
     p.activation = (streaming || gated) ? act : WOQ_ACT_IDENTITY;
+    p.residual = args->residual;
     if (streaming)
         return launch_stream(p, stream);
     GemmPlan plan = single ? plan_gemm(p.m, p.n, p.k, p.bits) : plan_grouped(p.m, p.num_experts, p.n);
     plan.k_splits = 1;
     plan.ws_bytes = 0;
+    bool const two_pass = act != WOQ_ACT_IDENTITY && !gated;
+    if (two_pass)
+        p.residual = nullptr; // added behind the activation, by the pass below
     if (int rc = launch_gemm_planned(p, plan, stream))
         return rc;
-    if (act == WOQ_ACT_IDENTITY || gated)
+    if (!two_pass)
         return WOQ_OK;
-    return launch_activation(p.out, p.out, p.m, p.n, act, p.out_dtype, stream); // elementwise, in place
+    return launch_activation(p.out, p.out, args->residual, p.m, p.n, act, p.out_dtype, stream); // in place
 }
 
 extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m,

@@ -10,7 +10,8 @@ namespace woq
 {
 
 template <int DT>
-__global__ void __launch_bounds__(256) activation_kernel(void* out, void const* in, long m, int n_in, int act)
+__global__ void __launch_bounds__(256) activation_kernel(
+    void* out, void const* in, void const* residual, long m, int n_in, int act)
 {
     using E = Elem<DT>;
     bool const gated = act_is_gated(act);
@@ -22,33 +23,33 @@ __global__ void __launch_bounds__(256) activation_kernel(void* out, void const* 
     for (long row = blockIdx.y; row < m; row += gridDim.y)
     {
         uint16_t const* src = static_cast<uint16_t const*>(in) + row * n_in + (long) col8 * 8;
-        u32x4 x = *reinterpret_cast<u32x4 const*>(src);
-        if (gated)
-        {
-            u32x4 const g = *reinterpret_cast<u32x4 const*>(src + n_out);
+        long const o = row * n_out + (long) col8 * 8;
+        u32x4 const x = *reinterpret_cast<u32x4 const*>(src);
+        u32x4 const g = gated ? *reinterpret_cast<u32x4 const*>(src + n_out) : x;
+        u32x4 const res = residual ? *reinterpret_cast<u32x4 const*>(static_cast<uint16_t const*>(residual) + o)
+                                   : u32x4{0u, 0u, 0u, 0u}; // +0.0 in both 16-bit formats
+        u32x4 y;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                x[r] = E::pack(E::lo(x[r]) * apply_act(act, E::lo(g[r])), E::hi(x[r]) * apply_act(act, E::hi(g[r])));
-        }
-        else
+        for (int r = 0; r < 4; ++r)
         {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                x[r] = E::pack(apply_act(act, E::lo(x[r])), apply_act(act, E::hi(x[r])));
+            float const lo = gated ? E::lo(x[r]) * apply_act(act, E::lo(g[r])) : apply_act(act, E::lo(x[r]));
+            float const hi = gated ? E::hi(x[r]) * apply_act(act, E::hi(g[r])) : apply_act(act, E::hi(x[r]));
+            y[r] = E::pack(lo + E::lo(res[r]), hi + E::hi(res[r]));
         }
-        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(out) + row * n_out + (long) col8 * 8) = x;
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(out) + o) = y;
     }
 }
 
-int launch_activation(void* out, void const* in, long m, int n_in, int act, int dtype, void* stream)
+int launch_activation(void* out, void const* in, void const* residual, long m, int n_in, int act, int dtype,
+    void* stream)
 {
     auto s = static_cast<hipStream_t>(stream);
     int const n_out = act_is_gated(act) ? n_in / 2 : n_in;
     dim3 block(256), grid((n_out / 8 + 255) / 256, (unsigned) (m < 4096 ? m : 4096));
     if (dtype == WOQ_BF16)
-        hipLaunchKernelGGL((activation_kernel<WOQ_BF16>), grid, block, 0, s, out, in, m, n_in, act);
+        hipLaunchKernelGGL((activation_kernel<WOQ_BF16>), grid, block, 0, s, out, in, residual, m, n_in, act);
     else
-        hipLaunchKernelGGL((activation_kernel<WOQ_FP16>), grid, block, 0, s, out, in, m, n_in, act);
+        hipLaunchKernelGGL((activation_kernel<WOQ_FP16>), grid, block, 0, s, out, in, residual, m, n_in, act);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "activation kernel launch failed: %s", hipGetErrorString(err));

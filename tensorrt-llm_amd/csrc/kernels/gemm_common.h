@@ -32,6 +32,7 @@ struct GemmParams
     // and writes [m, n/2]; the strips of a wavefront then alternate between the two halves of N
     // (see paired_strip).  Other activations are applied by a separate pass.
     int activation = kActIdentity;
+    void const* residual = nullptr; // [m, n_out] in the output type, added last (no split-K with it)
 };
 
 // Strip slot s of a wavefront whose first slot is `first` (even): without a gated activation strip
@@ -52,6 +53,8 @@ __device__ __forceinline__ int paired_strip(bool gated, int first, int s, int st
 inline void set_group_fields(GemmParams& gp, MatmulProblem const& p, int tile_rows)
 {
     gp.activation = act_is_gated(p.activation) ? p.activation : kActIdentity;
+    // behind a non-gated activation the residual is added by the activation pass, not here
+    gp.residual = (p.activation == kActIdentity || act_is_gated(p.activation)) ? p.residual : nullptr;
     gp.expert_rows = p.expert_rows;
     gp.num_experts = p.num_experts;
     gp.weight_stride = p.weight_stride;
@@ -76,8 +79,10 @@ __device__ __forceinline__ bool select_expert(GemmParams& p, int& tm, int tile_r
         if (tm < first_tile + tiles)
         {
             p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
-            p.out = uniform_ptr(static_cast<char*>(p.out)
-                + (size_t) begin * (size_t) (act_is_gated(p.activation) ? p.n / 2 : p.n) * 2);
+            size_t const out_off = (size_t) begin * (size_t) (act_is_gated(p.activation) ? p.n / 2 : p.n) * 2;
+            p.out = uniform_ptr(static_cast<char*>(p.out) + out_off);
+            if (p.residual)
+                p.residual = uniform_ptr(static_cast<char const*>(p.residual) + out_off);
             p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
             p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
             if (p.zeros)

@@ -351,33 +351,49 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    int const n_out = gated ? p.n / 2 : p.n;
+    // The residual is read through a descriptor (rows >= m read zeros, so no branches) and one row
+    // tile at a time, all loads of the tile in flight before the first is used.
+    auto const res_rsrc = make_rsrc(p.residual ? p.residual : p.out, (uint32_t) p.m * (uint32_t) n_out * 2u);
     if (gated)
     {
         // value and gate sums of an output element sit in neighbouring strip slots of this lane
         if constexpr (!SPLITK)
         {
-            int const n_out = p.n / 2;
             auto gated_epilogue = [&](auto act_tag)
             {
                 constexpr int ACT = decltype(act_tag)::value;
+                int col[NS / 2];
+                float bias_x[NS / 2], bias_g[NS / 2];
 #pragma unroll
-                for (int s = 0; s < NS; s += 2)
+                for (int i = 0; i < NS / 2; ++i)
                 {
-                    if (!strip_ok[s])
-                        continue;
-                    int const col = strip_of[s] * 16 + c; // strip_of[s] is the pair index (value half)
-                    float const bias_x = p.bias ? E::load(p.bias, col) : 0.f;
-                    float const bias_g = p.bias ? E::load(p.bias, col + n_out) : 0.f;
+                    col[i] = strip_of[2 * i] * 16 + c; // strip_of[even slot] is the pair index (value half)
+                    bias_x[i] = p.bias ? E::load(p.bias, col[i]) : 0.f;
+                    bias_g[i] = p.bias ? E::load(p.bias, col[i] + n_out) : 0.f;
+                }
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt)
+                for (int rt = 0; rt < RT; ++rt)
+                {
+                    int const row0 = m0 + rt * 16 + kg * 4;
+                    float res[NS / 2][4] = {};
+                    if (p.residual)
+                    {
+#pragma unroll
+                        for (int i = 0; i < NS / 2; ++i)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                res[i][r] = E::from_bits(buffer_load_u16(res_rsrc,
+                                    ((uint32_t) (row0 + r) * (uint32_t) n_out + (uint32_t) col[i]) * 2u));
+                    }
+#pragma unroll
+                    for (int i = 0; i < NS / 2; ++i)
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                        {
-                            int const row = m0 + rt * 16 + kg * 4 + r;
-                            if (row < p.m)
-                                out16[(size_t) row * n_out + col] = E::store(
-                                    (acc[rt][s][r] + bias_x) * apply_act(ACT, acc[rt][s + 1][r] + bias_g));
-                        }
+                            if (strip_ok[2 * i] && row0 + r < p.m)
+                                out16[(size_t) (row0 + r) * n_out + col[i]] = E::store((acc[rt][2 * i][r] + bias_x[i])
+                                        * apply_act(ACT, acc[rt][2 * i + 1][r] + bias_g[i])
+                                    + res[i][r]);
                 }
             };
             if (p.activation == kActSwiglu)
@@ -387,29 +403,40 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         return;
     }
+    int col[NS];
+    float bias[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        if (!strip_ok[s])
-            continue;
-        int const col = strip_of[s] * 16 + c;
-        float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
+        col[s] = strip_of[s] * 16 + c;
+        bias[s] = (!SPLITK && p.bias) ? E::load(p.bias, col[s]) : 0.f;
+    }
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
+    {
+        int const row0 = m0 + rt * 16 + kg * 4;
+        float res[NS][4] = {};
+        if (!SPLITK && p.residual)
         {
 #pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    res[s][r] = E::from_bits(
+                        buffer_load_u16(res_rsrc, ((uint32_t) (row0 + r) * (uint32_t) p.n + (uint32_t) col[s]) * 2u));
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
             for (int r = 0; r < 4; ++r)
-            {
-                int const row = m0 + rt * 16 + kg * 4 + r;
-                if (row < p.m)
+                if (strip_ok[s] && row0 + r < p.m)
                 {
                     if constexpr (SPLITK)
-                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, acc[rt][s][r]);
+                        unsafeAtomicAdd(p.partial + (size_t) (row0 + r) * p.n + col[s], acc[rt][s][r]);
                     else
-                        out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias));
+                        out16[(size_t) (row0 + r) * p.n + col[s]]
+                            = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias[s]) + res[s][r]);
                 }
-            }
-        }
     }
 }
 

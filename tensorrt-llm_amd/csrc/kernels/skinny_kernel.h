@@ -367,12 +367,15 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             v = __builtin_fmaf(pc, v, (-OFF * pc) * acc_s[rt][r]);
         return v;
     };
+    int const n_out = gated ? p.n / 2 : p.n;
+    // The residual is read through a descriptor (rows >= m read zeros, so no branches) and one row
+    // tile at a time, all loads of the tile in flight before the first is used.
+    auto const res_rsrc = make_rsrc(p.residual ? p.residual : p.out, (uint32_t) p.m * (uint32_t) n_out * 2u);
     if (gated)
     {
         // value and gate sums of an output element sit in the two strip slots of this lane
         if constexpr (!SPLITK)
         {
-            int const n_out = p.n / 2;
             auto gated_epilogue = [&](auto act_tag)
             {
                 constexpr int ACT = decltype(act_tag)::value;
@@ -385,14 +388,23 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 [[maybe_unused]] float const pc_g = GROUP == 0 ? E::load(p.scales, col + n_out) : 0.f;
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
+                {
+                    int const row0 = m0 + rt * 16 + kg * 4;
+                    float res[4] = {};
+                    if (p.residual)
+                    {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            res[r] = E::from_bits(buffer_load_u16(
+                                res_rsrc, ((uint32_t) (row0 + r) * (uint32_t) n_out + (uint32_t) col) * 2u));
+                    }
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                    {
-                        int const row = m0 + rt * 16 + kg * 4 + r;
-                        if (row < p.m)
-                            out16[(size_t) row * n_out + col] = E::store((finished(rt, 0, r, pc_x) + bias_x)
-                                * apply_act(ACT, finished(rt, 1, r, pc_g) + bias_g));
-                    }
+                        if (row0 + r < p.m)
+                            out16[(size_t) (row0 + r) * n_out + col] = E::store((finished(rt, 0, r, pc_x) + bias_x)
+                                    * apply_act(ACT, finished(rt, 1, r, pc_g) + bias_g)
+                                + res[r]);
+                }
             };
             if (p.activation == kActSwiglu)
                 gated_epilogue(std::integral_constant<int, kActSwiglu>{});
@@ -401,31 +413,44 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         }
         return;
     }
+    int col[NS];
+    float bias[NS];
+    [[maybe_unused]] float pc[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        if (!strip_ok[s])
-            continue;
-        int const col = strip_of[s] * 16 + c;
-        float const bias = (!SPLITK && p.bias) ? E::load(p.bias, col) : 0.f;
-        [[maybe_unused]] float const pc = GROUP == 0 ? E::load(p.scales, col) : 0.f;
+        col[s] = strip_of[s] * 16 + c;
+        bias[s] = (!SPLITK && p.bias) ? E::load(p.bias, col[s]) : 0.f;
+        pc[s] = GROUP == 0 ? E::load(p.scales, col[s]) : 0.f;
+    }
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
+    {
+        int const row0 = m0 + rt * 16 + kg * 4;
+        float res[NS][4] = {};
+        if (!SPLITK && p.residual)
         {
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    res[s][r] = E::from_bits(
+                        buffer_load_u16(res_rsrc, ((uint32_t) (row0 + r) * (uint32_t) p.n + (uint32_t) col[s]) * 2u));
+        }
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
             {
-                int const row = m0 + rt * 16 + kg * 4 + r;
-                float const v = finished(rt, s, r, pc);
-                if (row < p.m)
+                float const v = finished(rt, s, r, pc[s]);
+                if (strip_ok[s] && row0 + r < p.m)
                 {
                     if constexpr (SPLITK)
-                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, v);
+                        unsafeAtomicAdd(p.partial + (size_t) (row0 + r) * p.n + col[s], v);
                     else
-                        out16[(size_t) row * p.n + col] = E::store(__builtin_fmaf(p.alpha, v, bias));
+                        out16[(size_t) (row0 + r) * p.n + col[s]] = E::store(__builtin_fmaf(p.alpha, v, bias[s]) + res[s][r]);
                 }
             }
-        }
     }
 }
 

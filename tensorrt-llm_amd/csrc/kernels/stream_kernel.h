@@ -48,7 +48,8 @@ struct StreamParams
     int64_t const* expert_rows = nullptr;
     int num_experts = 0;
     size_t weight_stride = 0, scale_stride = 0;
-    int activation = kActIdentity; // epilogue activation (grouped kernel only)
+    int activation = kActIdentity;  // epilogue activation (grouped kernel only)
+    void const* residual = nullptr; // [rows, n_out], added after the activation (grouped kernel only)
 };
 
 // Everything one wavefront needs for one tile row (NS tiles side by side), fetched together so
@@ -374,7 +375,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                     x += E::load(p.bias, ocol);
                     g += E::load(p.bias, ocol + n_out);
                 }
-                out16[(size_t) row * n_out + ocol] = E::store(x * apply_act(p.activation, g));
+                float v = x * apply_act(p.activation, g);
+                if (p.residual)
+                    v += E::load(p.residual, (size_t) row * n_out + ocol);
+                out16[(size_t) row * n_out + ocol] = E::store(v);
             }
         }
         return;
@@ -395,7 +399,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         if (p.bias)
             v += E::load(p.bias, ocol);
         if constexpr (ACT)
+        {
             v = apply_act(p.activation, v);
+            if (p.residual)
+                v += E::load(p.residual, (size_t) row * p.n + ocol);
+        }
         out16[(size_t) row * p.n + ocol] = E::store(v);
     }
 }
@@ -423,6 +431,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams
     p.act = uniform_ptr(static_cast<char const*>(p.act) + (size_t) begin * (size_t) p.k * 2);
     int const n_out = act_is_gated(p.activation) ? p.n / 2 : p.n;
     p.out = uniform_ptr(static_cast<char*>(p.out) + (size_t) begin * (size_t) n_out * 2);
+    if (p.residual)
+        p.residual = uniform_ptr(static_cast<char const*>(p.residual) + (size_t) begin * (size_t) n_out * 2);
     p.weight = uniform_ptr(static_cast<char const*>(p.weight) + (size_t) e * p.weight_stride);
     p.scales = uniform_ptr(static_cast<char const*>(p.scales) + (size_t) e * p.scale_stride);
     if (ZERO)
@@ -436,6 +446,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams
         __syncthreads(); // this pass is done with the LDS areas
         p.act = static_cast<char const*>(p.act) + (size_t) 16 * (size_t) p.k * 2;
         p.out = static_cast<char*>(p.out) + (size_t) 16 * (size_t) n_out * 2;
+        if (p.residual)
+            p.residual = static_cast<char const*>(p.residual) + (size_t) 16 * (size_t) n_out * 2;
     }
 }
 
@@ -575,6 +587,7 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.weight_stride = p.weight_stride;
     sp.scale_stride = p.scale_stride;
     sp.activation = p.activation;
+    sp.residual = p.residual;
     auto s = static_cast<hipStream_t>(stream);
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;

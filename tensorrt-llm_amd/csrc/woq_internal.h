@@ -53,7 +53,8 @@ struct MatmulProblem
     int64_t const* expert_rows = nullptr;
     int num_experts = 0;
     size_t weight_stride = 0, scale_stride = 0;
-    int activation = 5; // WOQ_ACT_IDENTITY; applied by the grouped streaming kernel's epilogue
+    int activation = 5;             // WOQ_ACT_IDENTITY; see woq_grouped_matmul
+    void const* residual = nullptr; // [m, n_out] in the output type, added after the activation
 };
 
 // kernel launchers (each returns a woq_status)
@@ -61,7 +62,8 @@ int launch_stream(MatmulProblem const& p, void* stream);
 int launch_gemm(MatmulProblem const& p, void* stream);
 int launch_prequant(void* out, void const* act, void const* scale, int m, int k, int in_dtype, int out_dtype,
     void* stream);
-int launch_activation(void* out, void const* in, long m, int n_in, int act, int dtype, void* stream);
+int launch_activation(void* out, void const* in, void const* residual, long m, int n_in, int act, int dtype,
+    void* stream);
 int launch_dequant(void* out, void const* weight, void const* scales, void const* zeros, int k, int n, int group_size,
     int bits, int dtype, void* stream);
 

@@ -68,15 +68,15 @@ def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int,
 
 
 def woq_grouped_matmul_raw(act, weight, scales, zeros, bias, total_rows_before_expert, *, n: int, k: int,
-                           group_size: int, quant_algo: int, activation: str = "identity", regime: int = 0,
-                           out=None) -> torch.Tensor:
+                           group_size: int, quant_algo: int, activation: str = "identity", residual=None,
+                           regime: int = 0, out=None) -> torch.Tensor:
     """One call of woq_grouped_matmul (the MoE expert GEMM: moe_gemm_kernels.h:235-244 with weight-only
     scales).  `act` is [total_rows, k] sorted by expert, `weight` the preprocessed [E, ...] tensor,
     `scales` / `zeros` [E, n] or [E, k/group, n], `bias` [E, n], `total_rows_before_expert` an int64
     device tensor [E] of inclusive prefix sums (None: one expert owns every row).  `activation` is one
     of gelu / relu / silu / swiglu / geglu / identity (tensorrt_llm/layers/moe.py activation names);
-    the gated ones return [total_rows, n/2]."""
-    _require_gpu(act, weight, scales, zeros, bias, total_rows_before_expert, out)
+    the gated ones return [total_rows, n/2].  `residual` [total_rows, n_out] is added after the activation."""
+    _require_gpu(act, weight, scales, zeros, bias, total_rows_before_expert, residual, out)
     if total_rows_before_expert is not None and total_rows_before_expert.dtype != torch.int64:
         raise RuntimeError("total_rows_before_expert must be int64")
     if act.dim() != 2 or act.shape[1] != k:
@@ -87,6 +87,8 @@ def woq_grouped_matmul_raw(act, weight, scales, zeros, bias, total_rows_before_e
     n_out = n // 2 if activation in ("swiglu", "geglu") else n
     if out is None:
         out = torch.empty((act.shape[0], n_out), dtype=act.dtype, device=act.device)
+    if residual is not None and (tuple(residual.shape) != (act.shape[0], n_out) or residual.dtype != act.dtype):
+        raise RuntimeError("residual must be [%d, %d] of the activation dtype" % (act.shape[0], n_out))
     base = MatmulArgs(
         act=_ptr(act), pre_quant_scale=None, weight=_ptr(weight), scales=_ptr(scales), zeros=_ptr(zeros),
         bias=_ptr(bias), out=_ptr(out), alpha=1.0, m=act.shape[0], n=n, k=k, group_size=group_size,
@@ -94,7 +96,7 @@ def woq_grouped_matmul_raw(act, weight, scales, zeros, bias, total_rows_before_e
         workspace=None, workspace_bytes=0)
     experts = 1 if total_rows_before_expert is None else total_rows_before_expert.numel()
     args = GroupedMatmulArgs(base=base, total_rows_before_expert=_ptr(total_rows_before_expert), num_experts=experts,
-                             activation=act_id)
+                             activation=act_id, residual=_ptr(residual))
     check(lib.woq_grouped_matmul(ctypes.byref(args), _stream_handle(act.device)))
     return out
 

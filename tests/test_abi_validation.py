@@ -152,9 +152,9 @@ def test_grouped_matmul_validation(pkg):
     import ctypes
     L = pkg._lib
 
-    def gstatus(num_experts=4, total=0x7000, activation=L.ACT_IDENTITY, **kw):
+    def gstatus(num_experts=4, total=0x7000, activation=L.ACT_IDENTITY, residual=None, **kw):
         g = L.GroupedMatmulArgs(base=make_args(L, **kw), total_rows_before_expert=total, num_experts=num_experts,
-                                activation=activation)
+                                activation=activation, residual=residual)
         return L.lib.woq_grouped_matmul_check(ctypes.byref(g)), (L.lib.woq_last_error() or b"").decode()
 
     assert gstatus()[0] == 0
@@ -182,3 +182,4 @@ def test_grouped_matmul_validation(pkg):
     rc, msg = gstatus(activation=L.ACT_SWIGLU, n=48)
     assert rc == -2 and "32" in msg
     assert gstatus(activation=L.ACT_SWIGLU, m=4096, n=256)[0] == 0
+    assert gstatus(residual=0xA000)[0] == 0

@@ -27,7 +27,7 @@ def grouped_problem(oracle, rows, K, N, bits, group, dtype, zero, bias, seed):
     return p
 
 
-def run_grouped(pkg, oracle, dev, p, regime=0, activation="identity", single=False):
+def run_grouped(pkg, oracle, dev, p, regime=0, activation="identity", single=False, residual=None):
     F = pkg.functional
     dt = p["dtype"]
     w = torch.stack([preprocess(pkg, oracle, p["q"][e], p["bits"]) for e in range(len(p["rows"]))]).to(dev)
@@ -40,14 +40,15 @@ def run_grouped(pkg, oracle, dev, p, regime=0, activation="identity", single=Fal
     out = torch.full((p["act"].shape[0], n_out), float("nan"), dtype=TORCH_DT[dt], device=dev)
     F.woq_grouped_matmul_raw(to_dev(p["act"], dt, dev), w, to_dev(p["scales"], dt, dev), opt(p["zeros"]),
                              opt(p["bias"]), total, n=p["N"], k=p["K"], group_size=p["group"], quant_algo=algo,
-                             activation=activation, regime=regime, out=out)
+                             activation=activation, residual=None if residual is None else to_dev(residual, dt, dev),
+                             regime=regime, out=out)
     torch.cuda.synchronize()
     return out.float().cpu().numpy()
 
 
-def reference(oracle, p, activation="identity"):
+def reference(oracle, p, activation="identity", residual=None):
     return oracle.grouped_matmul_ref(p["act"], p["q"], p["scales"], p["zeros"], p["bias"], p["total"], p["group"],
-                                     p["dtype"], activation)
+                                     p["dtype"], activation, residual)
 
 
 @pytest.mark.parametrize("rows", [[3, 0, 16, 1], [40, 0, 5, 17], [0, 0, 7, 0], [1, 1, 1, 1, 1, 1, 1, 1]])
@@ -134,6 +135,24 @@ def test_single_expert_without_prefix_sums(pkg, oracle, dev, M, activation):
     out = run_grouped(pkg, oracle, dev, p, activation=activation, single=True)
     assert np.isfinite(out).all()
     assert oracle.max_rel_err(out, reference(oracle, p, activation)) < TOL
+
+
+@pytest.mark.parametrize("activation", ["identity", "swiglu", "gelu"])
+@pytest.mark.parametrize("rows,single", [([9], True), ([300], True), ([700], True), ([3, 0, 16, 1], False),
+                                         ([40, 5], False), ([90, 0, 70, 33], False), ([600, 300, 0, 700], False)])
+def test_residual_is_added_after_the_activation(pkg, oracle, dev, activation, rows, single):
+    """out = T(f(acc + bias) + residual) on every kernel: streaming, 64-row tiles, 256-row tiles, with
+    the gated epilogue, and behind the separate activation pass."""
+    p = grouped_problem(oracle, rows, 512, 288, 4, 128, "bf16", True, True, seed=sum(rows) + len(activation))
+    n_out = 144 if activation == "swiglu" else 288
+    rng = np.random.default_rng(77)
+    residual = oracle.round_to(rng.standard_normal((sum(rows), n_out)).astype(np.float32) * 3.0, "bf16")
+    out = run_grouped(pkg, oracle, dev, p, activation=activation, single=single, residual=residual)
+    assert np.isfinite(out).all()
+    assert oracle.max_rel_err(out, reference(oracle, p, activation, residual)) < TOL
+    # and it is the residual that was added: the difference to a call without it is the residual itself
+    plain = run_grouped(pkg, oracle, dev, p, activation=activation, single=single)
+    assert np.abs((out - plain) - residual).max() <= 0.05 * np.abs(residual).max()
 
 
 def test_grouped_rejections(pkg, oracle, dev):
