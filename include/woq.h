@@ -245,6 +245,16 @@ int woq_unpack_int4(void* unpacked_int8, const void* packed, size_t n_packed);
 int woq_apply_per_channel_scale(void* out, const void* act, const void* per_channel_scale, int32_t m, int32_t k,
     int32_t in_dtype, int32_t out_dtype, void* stream);
 
+/* RMSNorm fused with the smoothing pass in front of the matmul (one pass over the activations):
+ *   normed = T(x * rsqrt(mean(x^2) + eps) * gamma [+ beta]),  out = T_out(T(normed * pre_quant_scale))
+ * with T = dtype (fp16 / bf16) and T_out = dtype or fp8 e4m3 (the W4A8 activation).  Replaces
+ * invokeGeneralRmsNorm (kernels/rmsnormKernels.cu:230-262, arithmetic at :29-38 and :83-124)
+ * followed by apply_per_channel_scale_kernel_launcher (kernels/preQuantScaleKernel.cu:137-149).
+ * x, out [m, k]; gamma, beta, pre_quant_scale [k] of dtype; beta and pre_quant_scale may be NULL.
+ * k % 8 == 0.  The sum of squares is accumulated in float32 in this kernel's own order. */
+int woq_rmsnorm_prequant(void* out, const void* x, const void* gamma, const void* beta, const void* pre_quant_scale,
+    float eps, int32_t m, int32_t k, int32_t dtype, int32_t out_dtype, void* stream);
+
 /* Materialises W[k, n] = T(q*scale + zero) from preprocessed weights with the same device code
  * the GEMM main loop uses (counterpart of the identity-activation round trip in
  * tests/quantization/test_weight_only_quant_matmul.py:147-164).  dtype fp16/bf16, or fp8 e4m3

@@ -450,6 +450,20 @@ def apply_per_channel_scale(act, pre_quant_scale, in_dtype: str, out_dtype: str 
     return round_to(t, out_dtype)
 
 
+def rmsnorm_ref(x, gamma, eps: float, dtype: str, beta=None) -> np.ndarray:
+    """T(x * rsqrt(mean(x^2) + eps) * gamma [+ beta]) with the reference kernel's float32 steps
+    (kernels/rmsnormKernels.cu:29-38 compute_rmsnorm: val * s_variance * gamma, then + beta, each a
+    float32 operation; :106-107 variance / hidden_dim, rsqrtf(variance + eps); :124 cast to T).  The
+    sum of squares is taken in float64 here: its float32 summation order is the kernel's own."""
+    x = np.asarray(x, np.float32)
+    var = (x.astype(np.float64) ** 2).sum(-1, keepdims=True) / x.shape[-1]
+    inv = (1.0 / np.sqrt(var.astype(np.float32) + np.float32(eps))).astype(np.float32)
+    y = (x * inv).astype(np.float32) * np.asarray(gamma, np.float32)
+    if beta is not None:
+        y = y.astype(np.float32) + np.asarray(beta, np.float32)
+    return round_to(y.astype(np.float32), dtype)
+
+
 def woq_matmul_ref(act, q, scales, zeros=None, bias=None, pre_quant_scale=None, alpha: float = 1.0,
                    group_size: int = 0, act_dtype: str = "bf16", w4a8: bool = False) -> np.ndarray:
     """The dequantize-then-matmul path with float64 accumulation (well inside "fp32 accumulated"):

@@ -74,6 +74,7 @@ def _load():
         "woq_pack_int4": (ctypes.c_int, [vp, vp, sz]),
         "woq_unpack_int4": (ctypes.c_int, [vp, vp, sz]),
         "woq_apply_per_channel_scale": (ctypes.c_int, [vp, vp, vp, i32, i32, i32, i32, vp]),
+        "woq_rmsnorm_prequant": (ctypes.c_int, [vp, vp, vp, vp, vp, ctypes.c_float, i32, i32, i32, i32, vp]),
         "woq_dequantize": (ctypes.c_int, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
         "woq_last_error": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),

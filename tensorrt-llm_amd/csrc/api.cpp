@@ -443,6 +443,22 @@ extern "C" int woq_apply_per_channel_scale(void* out, const void* act, const voi
     return launch_prequant(out, act, per_channel_scale, m, k, in_dtype, out_dtype, stream);
 }
 
+extern "C" int woq_rmsnorm_prequant(void* out, const void* x, const void* gamma, const void* beta,
+    const void* pre_quant_scale, float eps, int32_t m, int32_t k, int32_t dtype, int32_t out_dtype, void* stream)
+{
+    if (!out || !x || !gamma)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_rmsnorm_prequant: null pointer");
+    if (dtype != WOQ_FP16 && dtype != WOQ_BF16)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "input dtype must be fp16 or bf16");
+    if (out_dtype != dtype && out_dtype != WOQ_FP8_E4M3)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "output dtype must be the input dtype or fp8 e4m3");
+    if (m < 0 || k <= 0 || k % 8)
+        return fail(WOQ_ERR_BAD_SHAPE, "m >= 0 and k %% 8 == 0 required (got %d, %d)", m, k);
+    if (m == 0)
+        return WOQ_OK;
+    return launch_rmsnorm_prequant(out, x, gamma, beta, pre_quant_scale, eps, m, k, dtype, out_dtype, stream);
+}
+
 extern "C" int woq_dequantize(void* out, const void* weight, const void* scales, const void* zeros, int32_t k,
     int32_t n, int32_t group_size, int32_t quant_type, int32_t dtype, void* stream)
 {

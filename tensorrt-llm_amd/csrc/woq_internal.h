@@ -62,6 +62,8 @@ int launch_stream(MatmulProblem const& p, void* stream);
 int launch_gemm(MatmulProblem const& p, void* stream);
 int launch_prequant(void* out, void const* act, void const* scale, int m, int k, int in_dtype, int out_dtype,
     void* stream);
+int launch_rmsnorm_prequant(void* out, void const* x, void const* gamma, void const* beta, void const* scale, float eps,
+    int m, int k, int dtype, int out_dtype, void* stream);
 int launch_activation(void* out, void const* in, void const* residual, long m, int n_in, int act, int dtype,
     void* stream);
 int launch_dequant(void* out, void const* weight, void const* scales, void const* zeros, int k, int n, int group_size,

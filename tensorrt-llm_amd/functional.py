@@ -147,6 +147,20 @@ def apply_per_channel_scale(act: torch.Tensor, per_channel_scale: torch.Tensor, 
     return out
 
 
+def rmsnorm_prequant(x: torch.Tensor, gamma: torch.Tensor, pre_quant_scale=None, eps: float = 1e-6, beta=None,
+                     out_dtype=None) -> torch.Tensor:
+    """RMSNorm (kernels/rmsnormKernels.cu:29-124) fused with the smoothing pass
+    (kernels/preQuantScaleKernel.cu:42-149): T_out(T(T(rmsnorm(x)) * pre_quant_scale)), T_out = x.dtype or
+    fp8 e4m3.  `pre_quant_scale` and `beta` may be None."""
+    _require_gpu(x, gamma, pre_quant_scale, beta)
+    out_dtype = out_dtype or x.dtype
+    k = x.shape[-1]
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    check(lib.woq_rmsnorm_prequant(_ptr(out), _ptr(x), _ptr(gamma), _ptr(beta), _ptr(pre_quant_scale), float(eps),
+                                   x.numel() // k, k, _WOQ_DT[x.dtype], _WOQ_DT[out_dtype], _stream_handle(x.device)))
+    return out
+
+
 def dequantize_weights(weights: torch.Tensor, scales: torch.Tensor, zeros, *, k: int, n: int, group_size: int,
                        quant_type: int, dtype: torch.dtype) -> torch.Tensor:
     """W[k, n] = dtype(q * scale + zero) from preprocessed weights (woq_dequantize)."""

@@ -183,3 +183,14 @@ def test_grouped_matmul_validation(pkg):
     assert rc == -2 and "32" in msg
     assert gstatus(activation=L.ACT_SWIGLU, m=4096, n=256)[0] == 0
     assert gstatus(residual=0xA000)[0] == 0
+
+
+def test_rmsnorm_prequant_validation(pkg):
+    L = pkg._lib
+    f = L.lib.woq_rmsnorm_prequant
+    err = lambda: (L.lib.woq_last_error() or b"").decode()
+    assert f(None, 0x1000, 0x2000, None, None, 1e-5, 4, 64, L.BF16, L.BF16, None) == -1 and "null" in err()
+    assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 4, 60, L.BF16, L.BF16, None) == -2
+    assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 4, 64, L.FP8_E4M3, L.BF16, None) == -1
+    assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 4, 64, L.BF16, L.FP16, None) == -1
+    assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 0, 64, L.BF16, L.FP8_E4M3, None) == 0  # m == 0: nothing to do

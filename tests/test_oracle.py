@@ -222,3 +222,23 @@ def test_activation_ref_known_values(oracle):
     pair = np.array([[2.0, 3.0, 1.0, -1.0]])  # value (2, 3), gate (1, -1)
     assert np.allclose(oracle.activation_ref(pair, "swiglu"), [[2.0 * silu[4], 3.0 * silu[1]]])
     assert np.allclose(oracle.activation_ref(pair, "geglu"), [[2.0 * gelu[4], 3.0 * gelu[1]]])
+
+
+def test_rmsnorm_ref_against_torch_and_closed_forms(oracle):
+    """rmsnorm_ref: a row of equal values c normalises to sign(c) * gamma / sqrt(1 + eps / c^2); scaling
+    a row leaves the result unchanged (eps = 0); and it agrees with torch's float32 rms_norm rounded
+    to the type, up to the last place."""
+    import torch
+    k = 256
+    gamma = oracle.round_to(np.linspace(0.5, 1.5, k).astype(np.float32), "bf16")
+    x = np.full((1, k), -2.0, np.float32)
+    want = oracle.round_to((-gamma / np.sqrt(1.0 + 1e-5 / 4.0)).astype(np.float32), "bf16")
+    assert (oracle.rmsnorm_ref(x, gamma, 1e-5, "bf16") == want).all()
+    rng = np.random.default_rng(2)
+    x = oracle.round_to(rng.standard_normal((4, k)).astype(np.float32), "fp16")
+    assert (oracle.rmsnorm_ref(x, gamma, 0.0, "fp16") == oracle.rmsnorm_ref(4.0 * x, gamma, 0.0, "fp16")).all()
+    beta = oracle.round_to(rng.standard_normal(k).astype(np.float32), "fp16")
+    t = torch.nn.functional.rms_norm(torch.from_numpy(x), (k,), torch.from_numpy(gamma), 1e-5) + torch.from_numpy(beta)
+    want = t.to(torch.float16).float().numpy()
+    got = oracle.rmsnorm_ref(x, gamma, 1e-5, "fp16", beta)
+    assert (got == want).mean() > 0.99 and np.abs(got - want).max() <= 2.0 ** -10 * np.abs(want).max()
