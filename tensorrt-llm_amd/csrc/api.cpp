@@ -176,6 +176,18 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
         return fail(WOQ_ERR_BAD_SHAPE, "n must be a multiple of %d (got %d)", kTileN, a->n);
     if (a->regime != WOQ_REGIME_AUTO && a->regime != WOQ_REGIME_STREAM && a->regime != WOQ_REGIME_GEMM)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown regime %d", a->regime);
+    {
+        // the kernels address every operand through buffer descriptors with 31-bit byte offsets
+        // (the top bit marks a deliberately out-of-range access)
+        uint64_t const limit = (uint64_t) 1 << 31;
+        uint64_t const act_bytes = (uint64_t) a->m * a->k * (a->act_dtype == WOQ_FP8_E4M3 ? 1 : 2);
+        uint64_t const weight_bytes = (uint64_t) a->k * a->n * ((algo & WOQ_ALGO_INT8_WEIGHT) ? 2 : 1) / 2;
+        uint64_t const scale_bytes = (uint64_t) (a->group_size ? a->k / a->group_size : 1) * a->n * 2;
+        if (act_bytes >= limit || weight_bytes >= limit || scale_bytes >= limit)
+            return fail(WOQ_ERR_UNSUPPORTED,
+                "operand too large: activations, one weight matrix and its scales must each stay below 2 GiB "
+                "(m=%d n=%d k=%d)", a->m, a->n, a->k);
+    }
 
     p.act = a->act;
     p.pre_quant_scale = a->pre_quant_scale;

@@ -54,6 +54,8 @@ def test_valid_combinations(pkg):
     (dict(act_dtype=2), -1, "FP8_ALPHA"),
     (dict(regime=1, m=129), -3, "unsupported m"),
     (dict(regime=7), -1, "regime"),
+    (dict(m=300000, k=4096), -3, "2 GiB"),                  # activations: 300000 * 4096 * 2 bytes
+    (dict(n=65536, k=65536), -3, "2 GiB"),                  # one int4 weight matrix of 2 GiB
     (dict(m=-1), -2, "non-negative"),
     (dict(quant_algo=64), -1, "quant_algo"),
 ])
