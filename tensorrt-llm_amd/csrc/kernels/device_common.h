@@ -256,6 +256,11 @@ __device__ __forceinline__ u32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t rsrc, uin
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) byte_offset, 0, 0);
 }
 
+__device__ __forceinline__ u32x2 buffer_load_x2(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int) byte_offset, 0, 0);
+}
+
 __device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
 {
     return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int) byte_offset, 0, 0);

@@ -316,7 +316,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                 {
-                    E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
+                    // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block,
+                    // lane (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c, so the
+                    // epilogue moves 8 bytes per lane and block instead of 2
+                    E::mma_acc(b_cur[s], a_cur, acc[rt][s]);
                     conv_stage(s);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -352,9 +355,27 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     mma_drain();
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
     int const n_out = gated ? p.n / 2 : p.n;
+    // acc[rt][s][r] = output (row m0 + rt*16 + c, column strip*16 + kg*4 + r): four consecutive
+    // columns per lane, moved as one 8-byte access (output, bias and residual alike).
     // The residual is read through a descriptor (rows >= m read zeros, so no branches) and one row
     // tile at a time, all loads of the tile in flight before the first is used.
     auto const res_rsrc = make_rsrc(p.residual ? p.residual : p.out, (uint32_t) p.m * (uint32_t) n_out * 2u);
+    auto load4 = [&](void const* base, int col) -> f32x4 // four consecutive 16-bit values as floats
+    {
+        u32x2 const v = *reinterpret_cast<u32x2 const*>(static_cast<uint16_t const*>(base) + col);
+        return f32x4{E::lo(v[0]), E::hi(v[0]), E::lo(v[1]), E::hi(v[1])};
+    };
+    auto store4 = [&](int row, int col, f32x4 v)
+    {
+        u32x2 const o = {E::pack(v[0], v[1]), E::pack(v[2], v[3])};
+        *reinterpret_cast<u32x2*>(out16 + (size_t) row * n_out + col) = o;
+    };
+    auto residual4 = [&](int row, int col) -> f32x4
+    {
+        u32x2 const v = buffer_load_x2(res_rsrc, ((uint32_t) row * (uint32_t) n_out + (uint32_t) col) * 2u);
+        return f32x4{E::lo(v[0]), E::hi(v[0]), E::lo(v[1]), E::hi(v[1])};
+    };
+    f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
     if (gated)
     {
         // value and gate sums of an output element sit in neighbouring strip slots of this lane
@@ -364,36 +385,34 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             {
                 constexpr int ACT = decltype(act_tag)::value;
                 int col[NS / 2];
-                float bias_x[NS / 2], bias_g[NS / 2];
+                f32x4 bias_x[NS / 2], bias_g[NS / 2];
 #pragma unroll
                 for (int i = 0; i < NS / 2; ++i)
                 {
-                    col[i] = strip_of[2 * i] * 16 + c; // strip_of[even slot] is the pair index (value half)
-                    bias_x[i] = p.bias ? E::load(p.bias, col[i]) : 0.f;
-                    bias_g[i] = p.bias ? E::load(p.bias, col[i] + n_out) : 0.f;
+                    col[i] = strip_of[2 * i] * 16 + kg * 4; // strip_of[even slot] is the pair index (value half)
+                    bias_x[i] = p.bias ? load4(p.bias, col[i]) : zero4;
+                    bias_g[i] = p.bias ? load4(p.bias, col[i] + n_out) : zero4;
                 }
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
                 {
-                    int const row0 = m0 + rt * 16 + kg * 4;
-                    float res[NS / 2][4] = {};
-                    if (p.residual)
-                    {
-#pragma unroll
-                        for (int i = 0; i < NS / 2; ++i)
-#pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                res[i][r] = E::from_bits(buffer_load_u16(res_rsrc,
-                                    ((uint32_t) (row0 + r) * (uint32_t) n_out + (uint32_t) col[i]) * 2u));
-                    }
+                    int const row = m0 + rt * 16 + c;
+                    f32x4 res[NS / 2];
 #pragma unroll
                     for (int i = 0; i < NS / 2; ++i)
+                        res[i] = p.residual ? residual4(row, col[i]) : zero4;
+#pragma unroll
+                    for (int i = 0; i < NS / 2; ++i)
+                    {
+                        if (!strip_ok[2 * i] || row >= p.m)
+                            continue;
+                        f32x4 v;
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (strip_ok[2 * i] && row0 + r < p.m)
-                                out16[(size_t) (row0 + r) * n_out + col[i]] = E::store((acc[rt][2 * i][r] + bias_x[i])
-                                        * apply_act(ACT, acc[rt][2 * i + 1][r] + bias_g[i])
-                                    + res[i][r]);
+                            v[r] = (acc[rt][2 * i][r] + bias_x[i][r]) * apply_act(ACT, acc[rt][2 * i + 1][r] + bias_g[i][r])
+                                + res[i][r];
+                        store4(row, col[i], v);
+                    }
                 }
             };
             if (p.activation == kActSwiglu)
@@ -404,39 +423,41 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         return;
     }
     int col[NS];
-    float bias[NS];
+    f32x4 bias[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
-        col[s] = strip_of[s] * 16 + c;
-        bias[s] = (!SPLITK && p.bias) ? E::load(p.bias, col[s]) : 0.f;
+        col[s] = strip_of[s] * 16 + kg * 4;
+        bias[s] = (!SPLITK && p.bias) ? load4(p.bias, col[s]) : zero4;
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
     {
-        int const row0 = m0 + rt * 16 + kg * 4;
-        float res[NS][4] = {};
-        if (!SPLITK && p.residual)
-        {
-#pragma unroll
-            for (int s = 0; s < NS; ++s)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    res[s][r] = E::from_bits(
-                        buffer_load_u16(res_rsrc, ((uint32_t) (row0 + r) * (uint32_t) p.n + (uint32_t) col[s]) * 2u));
-        }
+        int const row = m0 + rt * 16 + c;
+        f32x4 res[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
+            res[s] = (!SPLITK && p.residual) ? residual4(row, col[s]) : zero4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (strip_ok[s] && row0 + r < p.m)
-                {
-                    if constexpr (SPLITK)
-                        unsafeAtomicAdd(p.partial + (size_t) (row0 + r) * p.n + col[s], acc[rt][s][r]);
-                    else
-                        out16[(size_t) (row0 + r) * p.n + col[s]]
-                            = E::store(__builtin_fmaf(p.alpha, acc[rt][s][r], bias[s]) + res[s][r]);
-                }
+        for (int s = 0; s < NS; ++s)
+        {
+            if (!strip_ok[s] || row >= p.m)
+                continue;
+            if constexpr (SPLITK)
+            {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    unsafeAtomicAdd(p.partial + (size_t) row * p.n + col[s] + r, acc[rt][s][r]);
+            }
+            else
+            {
+                f32x4 v;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    v[r] = __builtin_fmaf(p.alpha, acc[rt][s][r], bias[s][r]) + res[s][r];
+                store4(row, col[s], v);
+            }
+        }
     }
 }
 

@@ -22,11 +22,6 @@
 namespace woq
 {
 
-__device__ __forceinline__ u32x2 buffer_load_x2(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
-{
-    return __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int) byte_offset, 0, 0);
-}
-
 // ALDS: the workgroup stages the activation rows in LDS once (small M x K) and the lanes read
 // their A pieces from there; a pipeline stage then holds packed weights and scales only.
 template <int ODT, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
