@@ -319,7 +319,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block,
                     // lane (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c, so the
                     // epilogue moves 8 bytes per lane and block instead of 2
-                    E::mma_acc(b_cur[s], a_cur, acc[rt][s]);
+                    // (the split-K variant keeps the plain orientation: its float atomics coalesce
+                    // better with 16 consecutive columns per row and instruction)
+                    if constexpr (SPLITK)
+                        E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
+                    else
+                        E::mma_acc(b_cur[s], a_cur, acc[rt][s]);
                     conv_stage(s);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -353,6 +358,22 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
+    if constexpr (SPLITK)
+    {
+        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                {
+                    int const row = m0 + rt * 16 + kg * 4 + r;
+                    if (strip_ok[s] && row < p.m)
+                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + strip_of[s] * 16 + c, acc[rt][s][r]);
+                }
+        return;
+    }
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
     int const n_out = gated ? p.n / 2 : p.n;
     // acc[rt][s][r] = output (row m0 + rt*16 + c, column strip*16 + kg*4 + r): four consecutive
@@ -368,7 +389,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto store4 = [&](int row, int col, f32x4 v)
     {
         u32x2 const o = {E::pack(v[0], v[1]), E::pack(v[2], v[3])};
-        *reinterpret_cast<u32x2*>(out16 + (size_t) row * n_out + col) = o;
+        // the output pointer may have been computed (grouped problems): tell the compiler it is
+        // global memory, or it falls back to flat stores
+        typedef __attribute__((address_space(1))) u32x2 global_u32x2;
+        *(global_u32x2*) (out16 + (size_t) row * n_out + col) = o;
     };
     auto residual4 = [&](int row, int col) -> f32x4
     {
@@ -381,9 +405,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         // value and gate sums of an output element sit in neighbouring strip slots of this lane
         if constexpr (!SPLITK)
         {
-            auto gated_epilogue = [&](auto act_tag)
+            // (two instantiations each: without a residual the loop holds no loads at all, so that no
+            // wait for a load - which would also wait for the stores before it - sits between stores)
+            auto gated_epilogue = [&](auto act_tag, auto residual_tag)
             {
                 constexpr int ACT = decltype(act_tag)::value;
+                constexpr bool RESIDUAL = decltype(residual_tag)::value;
                 int col[NS / 2];
                 f32x4 bias_x[NS / 2], bias_g[NS / 2];
 #pragma unroll
@@ -400,7 +427,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     f32x4 res[NS / 2];
 #pragma unroll
                     for (int i = 0; i < NS / 2; ++i)
-                        res[i] = p.residual ? residual4(row, col[i]) : zero4;
+                        res[i] = RESIDUAL ? residual4(row, col[i]) : zero4;
 #pragma unroll
                     for (int i = 0; i < NS / 2; ++i)
                     {
@@ -415,10 +442,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     }
                 }
             };
-            if (p.activation == kActSwiglu)
-                gated_epilogue(std::integral_constant<int, kActSwiglu>{});
+            bool const swiglu = p.activation == kActSwiglu;
+            if (p.residual)
+                swiglu ? gated_epilogue(std::integral_constant<int, kActSwiglu>{}, std::true_type{})
+                       : gated_epilogue(std::integral_constant<int, kActGeglu>{}, std::true_type{});
             else
-                gated_epilogue(std::integral_constant<int, kActGeglu>{});
+                swiglu ? gated_epilogue(std::integral_constant<int, kActSwiglu>{}, std::false_type{})
+                       : gated_epilogue(std::integral_constant<int, kActGeglu>{}, std::false_type{});
         }
         return;
     }
@@ -430,6 +460,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         col[s] = strip_of[s] * 16 + kg * 4;
         bias[s] = (!SPLITK && p.bias) ? load4(p.bias, col[s]) : zero4;
     }
+    auto plain_epilogue = [&](auto residual_tag)
+    {
+    constexpr bool RESIDUAL = decltype(residual_tag)::value;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
     {
@@ -437,28 +470,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         f32x4 res[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            res[s] = (!SPLITK && p.residual) ? residual4(row, col[s]) : zero4;
+            res[s] = RESIDUAL ? residual4(row, col[s]) : zero4;
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
             if (!strip_ok[s] || row >= p.m)
                 continue;
-            if constexpr (SPLITK)
-            {
+            f32x4 v;
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    unsafeAtomicAdd(p.partial + (size_t) row * p.n + col[s] + r, acc[rt][s][r]);
-            }
-            else
-            {
-                f32x4 v;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    v[r] = __builtin_fmaf(p.alpha, acc[rt][s][r], bias[s][r]) + res[s][r];
-                store4(row, col[s], v);
-            }
+            for (int r = 0; r < 4; ++r)
+                v[r] = __builtin_fmaf(p.alpha, acc[rt][s][r], bias[s][r]) + res[s][r];
+            store4(row, col[s], v);
         }
     }
+    };
+    if (!SPLITK && p.residual)
+        plain_epilogue(std::true_type{});
+    else
+        plain_epilogue(std::false_type{});
 }
 
 template <int DT, int BITS, int GROUP, bool ZERO, int RT>

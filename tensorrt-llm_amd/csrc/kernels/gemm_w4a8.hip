@@ -191,7 +191,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int s = 0; s < NS; ++s)
             {
-                mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
+                // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block, lane
+                // (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c (8-byte epilogue accesses)
+                // (the split-K variant keeps the plain orientation: its float atomics coalesce better
+                // with 16 consecutive columns per row and instruction)
+                if constexpr (SPLITK)
+                    mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
+                else
+                    mma_fp8_acc(b_use[s], a_cur, acc[rt][s]);
                 constexpr int PER = UNITS / (RT * NS);
 #pragma unroll
                 for (int cu = (rt * NS + s) * PER; cu < (rt * NS + s + 1) * PER; ++cu)
@@ -239,29 +246,52 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
     mma_drain();
     fp8_saturation_off();
+    if constexpr (SPLITK)
+    {
+        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c)
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                {
+                    int const row = m0 + rt * 16 + kg * 4 + r;
+                    if (strip0 + s < p.strips && row < p.m)
+                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + (strip0 + s) * 16 + c, acc[rt][s][r]);
+                }
+        return;
+    }
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    // acc[rt][s][r] = output (row m0 + rt*16 + c, column strip*16 + kg*4 + r): four consecutive
+    // columns per lane, written as one 8-byte store
+    typedef __attribute__((address_space(1))) u32x2 global_u32x2;
 #pragma unroll
     for (int s = 0; s < NS; ++s)
     {
         if (strip0 + s >= p.strips)
             continue;
-        int const col = (strip0 + s) * 16 + c;
-        float const bias = (!SPLITK && p.bias) ? EO::load(p.bias, col) : 0.f;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+        int const col = (strip0 + s) * 16 + kg * 4;
+        float bias[4] = {0.f, 0.f, 0.f, 0.f};
+        if (!SPLITK && p.bias)
+        {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-            {
-                int const row = m0 + rt * 16 + kg * 4 + r;
-                if (row < p.m)
-                {
-                    if constexpr (SPLITK)
-                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + col, acc[rt][s][r]);
-                    else
-                        out16[(size_t) row * p.n + col]
-                            = EO::store(after_mode_change(__builtin_fmaf(p.alpha, acc[rt][s][r], bias)));
-                }
-            }
+                bias[r] = EO::load(p.bias, col + r);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+        {
+            int const row = m0 + rt * 16 + c;
+            if (row >= p.m)
+                continue;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                v[r] = after_mode_change(__builtin_fmaf(p.alpha, acc[rt][s][r], bias[r]));
+            u32x2 const o = {EO::pack(v[0], v[1]), EO::pack(v[2], v[3])};
+            *(global_u32x2*) (out16 + (size_t) row * p.n + col) = o;
+        }
     }
 }
 
