@@ -68,7 +68,9 @@ struct StreamStage
 //       the row-sum MFMA
 // WAVES wavefronts per workgroup; they split K (tile row kt goes to wave kt % WAVES)
 // PF    tile rows in flight per wavefront
-// ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1
+// ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1.  The group
+//       scales and zeros of the workgroup's columns are staged with them (one 16-byte load per
+//       eight columns instead of a 2-byte load per lane, tile and strip inside the K loop)
 // ACT   the epilogue applies p.activation; a gated activation (value column j, gate column j + n/2) pairs
 //       the strips of a wavefront (even slot: value half, odd slot: gate half), output [m, n/2]
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
@@ -84,7 +86,9 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     constexpr int SEGS = TK / SEG;
     constexpr float OFF = Offset<DT, BITS>::value;
     using Stage = StreamStage<NS, SLABS, SEGS, MT, PQS, ALDS>;
-    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (KT*TK*2 + 16) bytes
+    constexpr bool SLDS = ALDS && GROUP != 0; // group scales / zeros live in LDS as well
+    constexpr int THREADS = WAVES * 64;
+    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (KT*TK*2 + 16) bytes, then scales, then zeros
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
     if (group >= p.groups)
@@ -150,6 +154,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     uint32_t const lds_row = (uint32_t) KT * TK * 2u + 16u; // +16: rows start in different banks
     int const a_row = c < p.m ? c : p.m - 1;
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
+    // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
+    // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
+    int const act_rows = p.m < 16 ? p.m : 16;
+    int const sc_rows = SLDS ? (KT * TK + (GROUP ? GROUP : 1) - 1) / (GROUP ? GROUP : 1) : 0;
+    constexpr uint32_t SC_ROW = NS * 32u;
+    char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
+    char* const zr_lds = sc_lds + (uint32_t) sc_rows * SC_ROW;
 
     auto fetch = [&](Stage& st, int kt)
     {
@@ -175,7 +186,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 }
             }
         }
-        if constexpr (GROUP != 0)
+        if constexpr (GROUP != 0 && !SLDS)
         {
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
@@ -244,8 +255,23 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
 #pragma unroll
                     for (int s = 0; s < NS; ++s)
                     {
-                        float const sc = E::from_bits(st.s[s][seg]);
-                        float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits(st.z[s][seg]) : 0.f);
+                        uint16_t s_raw, z_raw = 0;
+                        if constexpr (SLDS)
+                        {
+                            uint32_t const at
+                                = (uint32_t) ((kt * TK + seg * SEG) / (GROUP ? GROUP : 1)) * SC_ROW + (s * 16 + c) * 2u;
+                            s_raw = *reinterpret_cast<uint16_t const*>(sc_lds + at);
+                            if constexpr (ZERO)
+                                z_raw = *reinterpret_cast<uint16_t const*>(zr_lds + at);
+                        }
+                        else
+                        {
+                            s_raw = st.s[s][seg];
+                            if constexpr (ZERO)
+                                z_raw = st.z[s][seg];
+                        }
+                        float const sc = E::from_bits(s_raw);
+                        float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits(z_raw) : 0.f);
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt)
                         {
@@ -273,32 +299,119 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // the compiler's wait-count tracking stays exact: compute(st[i]) waits only for its own
     // stage while the PF-1 younger stages stay in flight.  The scheduling barriers keep the
     // compiler from sinking the prefetch below the compute (it would, to save registers).
+#ifdef WOQ_K_BLOCKED
+    int const k_per = (KT + WAVES - 1) / WAVES;
+    int const n_left = KT - wave * k_per;
+    int const n_my = n_left < 0 ? 0 : (n_left < k_per ? n_left : k_per);
+    auto kt_of = [&](int it) { return it < n_my ? wave * k_per + it : KT; };
+#else
     int const n_my = (KT - wave + WAVES - 1) / WAVES;
+    auto kt_of = [&](int it) { return wave + it * WAVES; };
+#endif
     Stage st[PF];
-#pragma unroll
-    for (int i = 0; i < PF; ++i)
-        fetch(st[i], wave + i * WAVES);
-    __builtin_amdgcn_sched_barrier(0);
-
-    if constexpr (ALDS)
+    if constexpr (!ALDS)
     {
-        // Stage the activations (smoothed if a pre-quant scale is given) behind the first weight
-        // prefetches: both are in flight together, the activations come from L2 and land first.
-        int const rows = p.m < 16 ? p.m : 16;
-        int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
-        for (int idx = threadIdx.x; idx < rows * chunks_per_row; idx += WAVES * 64)
-        {
-            int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
-            bool const k_ok = ch * 8 < K;
-            u32x4 v = buffer_load_x4(act_rsrc, k_ok ? ((uint32_t) row * (uint32_t) K + (uint32_t) ch * 8u) * 2u : kOob);
-            if constexpr (PQS)
-            {
-                u32x4 const sm = buffer_load_x4(pqs_rsrc, (uint32_t) ch * 16u);
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    v[r] = E::mul2(v[r], sm[r]);
+        for (int i = 0; i < PF; ++i)
+            fetch(st[i], kt_of(i));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    else
+    {
+        // Staged operands (activations - smoothed if a pre-quant scale is given - and the group
+        // scales / zeros of this workgroup's columns) are requested FIRST, the weight prefetch
+        // right behind them: loads complete in order, so the LDS writes and the barrier wait for
+        // the small staged loads only while the weights stay in flight.  Each thread holds up to
+        // UA + 2 staged chunks in registers across the prefetch; anything beyond that (long K,
+        // many rows) is staged by a plain loop after it.
+        constexpr int UA = 2;
+        int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
+        int const act_chunks = act_rows * chunks_per_row;
+        int const sc_chunks = sc_rows * NS * 2; // 8 columns each
+        auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch)
+        {
+            int const row = act_rows == 1 ? 0 : idx / chunks_per_row;
+            ch = (uint32_t) (idx - row * chunks_per_row);
+            lds_at = (uint32_t) row * lds_row + ch * 16u;
+            bool const ok = idx < act_chunks && (int) ch * 8 < K;
+            return ok ? ((uint32_t) row * (uint32_t) K + ch * 8u) * 2u : kOob;
+        };
+        auto sc_offset = [&](int idx, uint32_t& lds_at)
+        {
+            int const row = idx / (NS * 2), piece = idx - row * (NS * 2); // piece = strip slot * 2 + half
+            int strip = strip0 + (piece >> 1);
+            if (gated)
+            {
+                int const pair = strip0 / 2 + (piece >> 2);
+                strip = (pair < half_strips ? pair : half_strips - 1) + ((piece >> 1) & 1) * half_strips;
             }
-            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + (uint32_t) row * lds_row + (uint32_t) ch * 16u) = v;
+            else if (strip >= p.strips)
+                strip = p.strips - 1;
+            lds_at = (uint32_t) row * SC_ROW + (uint32_t) piece * 16u;
+            return idx < sc_chunks ? ((uint32_t) row * (uint32_t) p.n + (uint32_t) (strip * 16 + (piece & 1) * 8)) * 2u
+                                   : kOob;
+        };
+        auto smooth = [&](u32x4 v, u32x4 sm)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                v[r] = E::mul2(v[r], sm[r]);
+            return v;
+        };
+
+        u32x4 av[UA], pv[UA], sv, zv;
+        uint32_t a_at[UA], s_at = 0;
+#pragma unroll
+        for (int u = 0; u < UA; ++u)
+        {
+            uint32_t ch;
+            av[u] = buffer_load_x4(act_rsrc, act_offset(threadIdx.x + u * THREADS, a_at[u], ch));
+            if constexpr (PQS)
+                pv[u] = buffer_load_x4(pqs_rsrc, ch * 16u);
+        }
+        if constexpr (SLDS)
+        {
+            uint32_t const off = sc_offset(threadIdx.x, s_at);
+            sv = buffer_load_x4(sc_rsrc, off);
+            if constexpr (ZERO)
+                zv = buffer_load_x4(zr_rsrc, off);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+            fetch(st[i], kt_of(i));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < UA; ++u)
+            if ((int) threadIdx.x + u * THREADS < act_chunks)
+                *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = PQS ? smooth(av[u], pv[u]) : av[u];
+        if constexpr (SLDS)
+        {
+            if ((int) threadIdx.x < sc_chunks)
+            {
+                *reinterpret_cast<u32x4*>(sc_lds + s_at) = sv;
+                if constexpr (ZERO)
+                    *reinterpret_cast<u32x4*>(zr_lds + s_at) = zv;
+            }
+        }
+        for (int idx = threadIdx.x + UA * THREADS; idx < act_chunks; idx += THREADS)
+        {
+            uint32_t at, ch;
+            u32x4 v = buffer_load_x4(act_rsrc, act_offset(idx, at, ch));
+            if constexpr (PQS)
+                v = smooth(v, buffer_load_x4(pqs_rsrc, ch * 16u));
+            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + at) = v;
+        }
+        if constexpr (SLDS)
+        {
+            for (int idx = threadIdx.x + THREADS; idx < sc_chunks; idx += THREADS)
+            {
+                uint32_t at;
+                uint32_t const off = sc_offset(idx, at);
+                *reinterpret_cast<u32x4*>(sc_lds + at) = buffer_load_x4(sc_rsrc, off);
+                if constexpr (ZERO)
+                    *reinterpret_cast<u32x4*>(zr_lds + at) = buffer_load_x4(zr_rsrc, off);
+            }
         }
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
@@ -310,9 +423,9 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         for (int i = 0; i < PF; ++i)
         {
             if (it + i < n_my)
-                compute(st[i], wave + (it + i) * WAVES);
+                compute(st[i], kt_of(it + i));
             __builtin_amdgcn_sched_barrier(0);
-            fetch(st[i], wave + (it + i + PF) * WAVES);
+            fetch(st[i], kt_of(it + i + PF));
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -465,7 +578,15 @@ inline size_t stream_act_lds_bytes(int m, int k, int tile_k)
     return (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
 }
 
-constexpr size_t kStreamMaxActLds = 96 * 1024;
+// bytes of LDS the staged group scales (and zeros) of ns strips take
+inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool zeros)
+{
+    if (group == 0)
+        return 0;
+    size_t const k_padded = (size_t) ((k + tile_k - 1) / tile_k) * tile_k;
+    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1);
+}
+
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k);
@@ -484,7 +605,7 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     size_t lds = 0;
     if constexpr (ALDS)
     {
-        lds = stream_act_lds_bytes(sp.m, sp.k, TK);
+        lds = stream_act_lds_bytes(sp.m, sp.k, TK) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO);
         if (lds > kStreamMaxActLds)
             return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
         static bool raised = false; // benign race: the attribute call is idempotent
@@ -524,6 +645,7 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
     WOQ_SHAPE(1, 4, 4, 2, true)
     WOQ_SHAPE(1, 4, 4, 4, true)
     WOQ_SHAPE(1, 4, 8, 2, true)
+    WOQ_SHAPE(1, 4, 8, 4, true)
     // decode, activations in registers (M x K too large for LDS)
     WOQ_SHAPE(1, 1, 8, 4, false)
     WOQ_SHAPE(1, 2, 8, 2, false)

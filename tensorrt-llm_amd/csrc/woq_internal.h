@@ -205,5 +205,7 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;
 constexpr int kStreamW4a8MaxM = 16;
+// most LDS a streaming workgroup stages its operands in (activations, group scales and zeros)
+constexpr size_t kStreamMaxActLds = 96 * 1024;
 
 } // namespace woq
