@@ -87,14 +87,15 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         int const rows = m < 16 ? m : 16;
         size_t const act_lds = (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
         // beyond ~48 KiB the staging area costs more in resident workgroups than the L2 reads it saves;
-        // the group scales and zeros are staged next to the activations (at most k * ns bytes)
+        // the group scales and zeros are staged next to the activations (at most k * ns bytes, and k
+        // more for the activation row sums)
         if (act_lds <= 48 * 1024)
         {
             StreamShape const sh = strips >= 1024 ? StreamShape{4, 8, 2, 1}
                                                   : (strips >= 384 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
-            if (act_lds + (size_t) k * sh.ns <= kStreamMaxActLds)
+            if (act_lds + (size_t) k * (sh.ns + 1) <= kStreamMaxActLds)
                 return sh;
-            if (act_lds + (size_t) k <= kStreamMaxActLds)
+            if (act_lds + (size_t) k * 2 <= kStreamMaxActLds)
                 return {1, 8, 4, 1};
         }
         if (strips >= 1024)

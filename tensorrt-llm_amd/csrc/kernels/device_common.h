@@ -315,6 +315,14 @@ __device__ __forceinline__ T* uniform_ptr(T* ptr)
 // Workgroups are handed to the 8 XCDs round-robin.  Mapping block b to
 // strip (b % 8) * strips_per_xcd + b / 8 keeps neighbouring 16-column strips (which share
 // 128-byte lines of the scale / zero rows) on one XCD, hence in one L2.
+// v + (v of the lane a DPP control selects); every lane of the 16-lane row must be active
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v)
+{
+    int const x = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+    return v + __builtin_bit_cast(float, x);
+}
+
 __device__ __forceinline__ int xcd_strip(int block, int strips_per_xcd)
 {
     return (block & 7) * strips_per_xcd + (block >> 3);

@@ -70,7 +70,9 @@ struct StreamStage
 // PF    tile rows in flight per wavefront
 // ALDS  activations (m <= 16 rows) are staged in LDS by the workgroup; requires MT == 1.  The group
 //       scales and zeros of the workgroup's columns are staged with them (one 16-byte load per
-//       eight columns instead of a 2-byte load per lane, tile and strip inside the K loop)
+//       eight columns instead of a 2-byte load per lane, tile and strip inside the K loop), and
+//       the activation row sums S of every segment are formed once while staging, which takes
+//       the all-ones MFMA out of the K loop
 // ACT   the epilogue applies p.activation; a gated activation (value column j, gate column j + n/2) pairs
 //       the strips of a wavefront (even slot: value half, odd slot: gate half), output [m, n/2]
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
@@ -161,6 +163,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     constexpr uint32_t SC_ROW = NS * 32u;
     char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
     char* const zr_lds = sc_lds + (uint32_t) sc_rows * SC_ROW;
+    // activation row sums of segment i (SEG rows of K): 16 floats (one per row of the M-tile) at i * 64
+    char* const sum_lds = zr_lds + (ZERO ? (uint32_t) sc_rows * SC_ROW : 0u);
 
     auto fetch = [&](Stage& st, int kt)
     {
@@ -229,7 +233,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                                 a[mt][r] = E::mul2(a[mt][r], st.sm[j][r]);
                         }
                     }
-                    acc_s[mt] = E::mma(a[mt], ones, acc_s[mt]);
+                    if constexpr (!SLDS)
+                        acc_s[mt] = E::mma(a[mt], ones, acc_s[mt]);
                 }
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
@@ -249,6 +254,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 // a segment past the end of K carries zero activations, scale 0 and zero 0.
                 // Lane (kg, c) register r is output row kg*4 + r: with a single row (decode,
                 // m == 1) only r == 0 is ever stored, so the other three are not scaled.
+                if constexpr (SLDS) // rows kg*4 .. kg*4+3 of this segment's sums
+                    acc_s[0] = *reinterpret_cast<f32x4 const*>(sum_lds + (uint32_t) (kt * SEGS + seg) * 64u + kg * 16u);
                 auto scale_rows = [&](auto rows_tag)
                 {
                     constexpr int ROWS = decltype(rows_tag)::value;
@@ -299,15 +306,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // the compiler's wait-count tracking stays exact: compute(st[i]) waits only for its own
     // stage while the PF-1 younger stages stay in flight.  The scheduling barriers keep the
     // compiler from sinking the prefetch below the compute (it would, to save registers).
-#ifdef WOQ_K_BLOCKED
-    int const k_per = (KT + WAVES - 1) / WAVES;
-    int const n_left = KT - wave * k_per;
-    int const n_my = n_left < 0 ? 0 : (n_left < k_per ? n_left : k_per);
-    auto kt_of = [&](int it) { return it < n_my ? wave * k_per + it : KT; };
-#else
     int const n_my = (KT - wave + WAVES - 1) / WAVES;
     auto kt_of = [&](int it) { return wave + it * WAVES; };
-#endif
     Stage st[PF];
     if constexpr (!ALDS)
     {
@@ -328,11 +328,12 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
         int const act_chunks = act_rows * chunks_per_row;
         int const sc_chunks = sc_rows * NS * 2; // 8 columns each
-        auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch)
+        auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
         {
             int const row = act_rows == 1 ? 0 : idx / chunks_per_row;
             ch = (uint32_t) (idx - row * chunks_per_row);
             lds_at = (uint32_t) row * lds_row + ch * 16u;
+            sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;
             bool const ok = idx < act_chunks && (int) ch * 8 < K;
             return ok ? ((uint32_t) row * (uint32_t) K + ch * 8u) * 2u : kOob;
         };
@@ -358,14 +359,31 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 v[r] = E::mul2(v[r], sm[r]);
             return v;
         };
+        // Sum of the SEG activations of one segment: the SEG/8 consecutive lanes that hold its
+        // chunks add their eight values each and combine across lanes; every lane of a 16-lane
+        // row is active here (rows of lanes enter or leave the staging loops together).
+        auto stage_sum = [&](u32x4 v, int idx, uint32_t sum_at)
+        {
+            float t = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                t += E::from_bits((uint16_t) (v[r] & 0xFFFFu)) + E::from_bits((uint16_t) (v[r] >> 16));
+            t = dpp_add<0xB1>(t);  // quad_perm [1,0,3,2]
+            t = dpp_add<0x4E>(t);  // quad_perm [2,3,0,1]
+            t = dpp_add<0x141>(t); // row_half_mirror
+            if constexpr (SEG == 128)
+                t = dpp_add<0x140>(t); // row_mirror
+            if ((threadIdx.x & (SEG / 8 - 1)) == 0 && idx < act_chunks)
+                *reinterpret_cast<float*>(sum_lds + sum_at) = t;
+        };
 
         u32x4 av[UA], pv[UA], sv, zv;
-        uint32_t a_at[UA], s_at = 0;
+        uint32_t a_at[UA], sum_at[UA], s_at = 0;
 #pragma unroll
         for (int u = 0; u < UA; ++u)
         {
             uint32_t ch;
-            av[u] = buffer_load_x4(act_rsrc, act_offset(threadIdx.x + u * THREADS, a_at[u], ch));
+            av[u] = buffer_load_x4(act_rsrc, act_offset(threadIdx.x + u * THREADS, a_at[u], ch, sum_at[u]));
             if constexpr (PQS)
                 pv[u] = buffer_load_x4(pqs_rsrc, ch * 16u);
         }
@@ -383,8 +401,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < UA; ++u)
+        {
+            u32x4 const v = PQS ? smooth(av[u], pv[u]) : av[u];
             if ((int) threadIdx.x + u * THREADS < act_chunks)
-                *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = PQS ? smooth(av[u], pv[u]) : av[u];
+                *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = v;
+            if constexpr (SLDS)
+                stage_sum(v, threadIdx.x + u * THREADS, sum_at[u]);
+        }
         if constexpr (SLDS)
         {
             if ((int) threadIdx.x < sc_chunks)
@@ -396,11 +419,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         for (int idx = threadIdx.x + UA * THREADS; idx < act_chunks; idx += THREADS)
         {
-            uint32_t at, ch;
-            u32x4 v = buffer_load_x4(act_rsrc, act_offset(idx, at, ch));
+            uint32_t at, ch, sum_at;
+            u32x4 v = buffer_load_x4(act_rsrc, act_offset(idx, at, ch, sum_at));
             if constexpr (PQS)
                 v = smooth(v, buffer_load_x4(pqs_rsrc, ch * 16u));
             *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + at) = v;
+            if constexpr (SLDS)
+                stage_sum(v, idx, sum_at);
         }
         if constexpr (SLDS)
         {
@@ -578,13 +603,14 @@ inline size_t stream_act_lds_bytes(int m, int k, int tile_k)
     return (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
 }
 
-// bytes of LDS the staged group scales (and zeros) of ns strips take
+// bytes of LDS the staged group scales (and zeros) of ns strips and the activation row sums take
 inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool zeros)
 {
     if (group == 0)
         return 0;
     size_t const k_padded = (size_t) ((k + tile_k - 1) / tile_k) * tile_k;
-    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1);
+    size_t const seg = group > tile_k ? tile_k : group; // rows of K per activation row sum
+    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1) + k_padded / seg * 64;
 }
 
 
