@@ -130,7 +130,7 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
     assert oracle.max_rel_err(outg.float().cpu().numpy(), reference(oracle, pg)) < TOL
 
 
-STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,1", "4,4,4,1", "4,8,2,1",
+STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,1", "4,4,4,1", "4,8,2,1", "4,8,4,1",
                  "1,8,4,0", "2,8,2,0", "4,4,2,0"]
 
 
@@ -151,6 +151,18 @@ def test_stream_every_launch_shape(pkg, oracle, dev, monkeypatch, shape, M):
 def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
     """Wide outputs take the multi-strip launch shapes of the heuristic."""
     p = random_problem(oracle, 1, 512, N, 4, 128, "bf16", zero=True, seed=N)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("M,K,group,bits", [(1, 8192, 64, 4), (3, 8192, 64, 4), (2, 4160, 64, 4), (5, 4096, 128, 8)])
+def test_stream_long_k_staged_operands(pkg, oracle, dev, M, K, group, bits):
+    """Long K with four strips per wavefront: the activations, the group scales / zeros and the
+    activation row sums staged in LDS exceed what a thread keeps in registers across the weight
+    prefetch (the staging tail loops run), take more than 64 KiB of LDS, and K = 4160 ends in half
+    a weight tile whose scales, zeros and row sums must read as zero."""
+    N = 16384
+    p = random_problem(oracle, M, K, N, bits, group, "bf16", zero=True, pqs=True, seed=K + M)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
     assert err < TOL, err
 
