@@ -94,6 +94,52 @@ __device__ __forceinline__ void int8_pair(uint32_t w0, uint32_t w1, int p, int& 
     q1 = (int) ((w >> (sh + 8)) & 0xFF) - 128;
 }
 
+// The same two values divided by 16, as floats: v_cvt_off_f32_i4 converts the signed nibble in
+// bits [3:0] of its operand to q/16, and a byte select on the source reaches the low nibble of any
+// byte without a shift; the odd nibbles are the low nibbles of the bytes of t >> 4.  The caller
+// multiplies by 16*s, so fma(q/16, 16*s, z) rounds the same real number as fma(q, s, z).
+// (The byte select is written out: left to the compiler, a third of these conversions end up
+// behind a separate bit-field extract.)
+__device__ __forceinline__ float cvt_off_f32_i4_byte(uint32_t t, int byte)
+{
+    float x;
+    switch (byte)
+    {
+    case 0: x = __builtin_amdgcn_cvt_off_f32_i4((int) t); break; // the instruction reads bits [3:0] only
+    case 1: asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(x) : "v"(t)); break;
+    case 2: asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(x) : "v"(t)); break;
+    default: asm("v_cvt_off_f32_i4_sdwa %0, %1 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(x) : "v"(t)); break;
+    }
+    return x;
+}
+
+__device__ __forceinline__ void int4_pair_sixteenths(uint32_t t, int p, float& x0, float& x1)
+{
+    uint32_t const src = (p & 1) ? t >> 4 : t;
+    x0 = cvt_off_f32_i4_byte(src, p >> 1);
+    x1 = cvt_off_f32_i4_byte(src, 2 + (p >> 1));
+}
+
+// signed values of bytes 2h and 2h+1 of an int8 dword `t` (the stored dword XOR 0x80808080), as
+// floats: sign-extending byte converts
+__device__ __forceinline__ void int8_pair_float(uint32_t t, int h, float& x0, float& x1)
+{
+    x0 = (float) (int) (signed char) (t >> (16 * h));
+    x1 = (float) (int) (signed char) (t >> (16 * h + 8));
+}
+
+// packed half-precision helpers on raw 32-bit pairs
+__device__ __forceinline__ uint32_t half2_add(uint32_t a, float b)
+{
+    f16x2 const b2 = {(_Float16) b, (_Float16) b};
+    return bit_cast<uint32_t>(bit_cast<f16x2>(a) + b2);
+}
+
+__device__ __forceinline__ uint32_t half2_fma(uint32_t a, uint32_t b, uint32_t c)
+{
+    return bit_cast<uint32_t>(__builtin_elementwise_fma(bit_cast<f16x2>(a), bit_cast<f16x2>(b), bit_cast<f16x2>(c)));
+}
+
 template <int DT>
 __device__ __forceinline__ uint32_t dequant_pair(int q0, int q1, float s, float z);
 

@@ -108,11 +108,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     // per-column scale of the per-channel mode (GROUP == 0) is loaded once
     float pc_scale[NS];
+    uint32_t pc_scale2[NS]; // the raw 16-bit value in both halves
     if constexpr (GROUP == 0)
     {
 #pragma unroll
         for (int s = 0; s < NS; ++s)
+        {
             pc_scale[s] = E::load(p.scales, strip_of[s] * 16 + c);
+            pc_scale2[s] = (uint32_t) static_cast<uint16_t const*>(p.scales)[strip_of[s] * 16 + c] * 0x10001u;
+        }
     }
 
     // A tile -> LDS.  Fragment f = rt * SLABS + j is 1 KiB: the 16 rows x 32 k that one MFMA
@@ -228,6 +232,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
     };
 
+    // the same as packed half-precision pairs (s, s) and (z, z), from the raw 16-bit values
+    auto scale_pair_of = [&](BStage const& st, int s, int seg, uint32_t& s2, uint32_t& z2)
+    {
+        if constexpr (GROUP != 0)
+        {
+            s2 = (uint32_t) st.s[s][seg] * 0x10001u;
+            z2 = ZERO ? (uint32_t) st.z[s][seg] * 0x10001u : 0u;
+        }
+        else
+        {
+            s2 = pc_scale2[s];
+            z2 = 0u;
+        }
+    };
+
     auto compute = [&](auto const* buf, BStage const& st, BStage& st_next, auto* buf_next, int kt_next)
     {
         char const* a_base = reinterpret_cast<char const*>(buf) + a_lane_off;
@@ -265,8 +284,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 // after each of the 4 MFMAs: a wavefront issues in order, so VALU work only runs
                 // under the matrix core when it sits between the matrix instructions.
                 constexpr int CONV = 16 / RT;
-                int q0[CONV], q1[CONV];
+                // bf16: q/16 as float (v_cvt_off_f32_i4 / sign-extending byte converts, with byte
+                // selects on the source), float32 FMA with 16*s, packed round to bf16.
+                // fp16: the exponent-magic pair (BASE + u), one packed subtract to the exact q and
+                // one packed half-precision FMA.
                 float t0[CONV], t1[CONV], sc[CONV], zr[CONV];
+                uint32_t h2[CONV], s2[CONV], z2[CONV];
                 auto conv_stage = [&](int stage)
                 {
 #pragma unroll
@@ -276,39 +299,43 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                         bool const same_step = j + 1 < SLABS;
                         BStage const& src = same_step ? st : st_next;
                         int const jn = same_step ? j + 1 : 0;
-                        if (stage == 0)
+                        if constexpr (DT == WOQ_BF16)
                         {
-                            scale_of(src, s, jn / SEG_SLABS, sc[x], zr[x]);
-                            if constexpr (BITS == 4)
-                                int4_pair(src.w[s][jn] ^ 0x88888888u, pr, q0[x], q1[x]);
-                            else
-                                int8_pair(src.w[s][2 * jn], src.w[s][2 * jn + 1], pr, q0[x], q1[x]);
-                        }
-                        else if (stage == 1)
-                        {
-                            t0[x] = (float) q0[x];
-                            t1[x] = (float) q1[x];
-                        }
-                        else if (stage == 2)
-                        {
-                            if constexpr (DT == WOQ_BF16)
+                            if (stage == 0)
+                            {
+                                scale_of(src, s, jn / SEG_SLABS, sc[x], zr[x]);
+                                sc[x] *= BITS == 4 ? 16.f : 1.f;
+                            }
+                            else if (stage == 1)
+                            {
+                                if constexpr (BITS == 4)
+                                    int4_pair_sixteenths(src.w[s][jn] ^ 0x88888888u, pr, t0[x], t1[x]);
+                                else
+                                    int8_pair_float(src.w[s][2 * jn + pr / 2] ^ 0x80808080u, pr & 1, t0[x], t1[x]);
+                            }
+                            else if (stage == 2)
                             {
                                 t0[x] = __builtin_fmaf(t0[x], sc[x], zr[x]);
                                 t1[x] = __builtin_fmaf(t1[x], sc[x], zr[x]);
                             }
+                            else
+                                b_nxt[s][pr] = E::pack(t0[x], t1[x]);
                         }
                         else
                         {
-                            if constexpr (DT == WOQ_BF16)
-                                b_nxt[s][pr] = E::pack(t0[x], t1[x]);
-                            else
+                            if (stage == 0)
+                                scale_pair_of(src, s, jn / SEG_SLABS, s2[x], z2[x]);
+                            else if (stage == 1)
                             {
-                                // half-precision FMA (single rounding), as dequant_pair<WOQ_FP16>
-                                f16x2 const q2 = {(_Float16) t0[x], (_Float16) t1[x]};
-                                f16x2 const s2 = {(_Float16) sc[x], (_Float16) sc[x]};
-                                f16x2 const z2 = {(_Float16) zr[x], (_Float16) zr[x]};
-                                b_nxt[s][pr] = bit_cast<uint32_t>(__builtin_elementwise_fma(q2, s2, z2));
+                                if constexpr (BITS == 4)
+                                    h2[x] = ((src.w[s][jn] >> (4 * pr)) & 0x000F000Fu) | E::kMagic4;
+                                else
+                                    h2[x] = expand_int8_reg<WOQ_FP16>(src.w[s][2 * jn + pr / 2], pr & 1);
                             }
+                            else if (stage == 2)
+                                h2[x] = half2_add(h2[x], -Offset<DT, BITS>::value);
+                            else
+                                b_nxt[s][pr] = half2_fma(h2[x], s2[x], z2[x]);
                         }
                     }
                 };
