@@ -18,14 +18,16 @@ template <bool ZERO, bool CLAMP = true>
 __device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h, int p, float s, float z)
 {
     float v0, v1;
-    int const e0 = 4 * h + 2 * p; // even element: nibble slot e0/2; the odd one after it: slot 4 + e0/2
+    // elements e0 = 4h + 2p and e0 + 1 sit in nibble slots e0/2 and 4 + e0/2
     if constexpr (ZERO)
     {
+        // q/16 straight from the nibble (see int4_pair_sixteenths), times 16 s: the same rounding.
+        // Slots e0/2 and 4 + e0/2 are the low nibbles of bytes h and h+2 of t (p = 0) or t >> 4 (p = 1).
         uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
-        int const q0 = (int) (t << (28 - 4 * (e0 / 2))) >> 28;
-        int const q1 = (int) (t << (12 - 4 * (e0 / 2))) >> 28;
-        v0 = __builtin_fmaf((float) q0, s, z);
-        v1 = __builtin_fmaf((float) q1, s, z);
+        uint32_t const src = p == 0 ? t : t >> 4;
+        float const s16 = 16.f * s;
+        v0 = __builtin_fmaf(cvt_off_f32_i4_byte(src, h), s16, z);
+        v1 = __builtin_fmaf(cvt_off_f32_i4_byte(src, h + 2), s16, z);
     }
     else
     {
@@ -55,11 +57,12 @@ __device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, flo
     float v[4]; // elements 4h, 4h+1, 4h+2, 4h+3: nibble slots 2h, 4+2h, 2h+1, 5+2h
     if constexpr (ZERO)
     {
-        uint32_t const t = w ^ 0x88888888u; // biased -> two's complement nibbles
-        int const slot[4] = {2 * h, 4 + 2 * h, 2 * h + 1, 5 + 2 * h};
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            v[i] = __builtin_fmaf((float) ((int) (t << (28 - 4 * slot[i])) >> 28), s, z);
+        uint32_t const t = w ^ 0x88888888u, t4 = t >> 4; // biased -> two's complement nibbles
+        float const s16 = 16.f * s;
+        v[0] = __builtin_fmaf(cvt_off_f32_i4_byte(t, h), s16, z);
+        v[1] = __builtin_fmaf(cvt_off_f32_i4_byte(t, h + 2), s16, z);
+        v[2] = __builtin_fmaf(cvt_off_f32_i4_byte(t4, h), s16, z);
+        v[3] = __builtin_fmaf(cvt_off_f32_i4_byte(t4, h + 2), s16, z);
     }
     else
     {
@@ -111,7 +114,6 @@ __device__ __forceinline__ T after_mode_change(T v)
 }
 
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
-typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // c += a x b (32 e4m3 values per lane each), accumulator tied to one AGPR quad (see Elem::mma_acc)
