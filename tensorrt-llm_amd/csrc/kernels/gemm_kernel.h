@@ -375,10 +375,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             scale_of(st0, s, 0, sc, zr);
             b_cur[s][pr] = dequant_operand_reg<DT, BITS>(st0.w[s], 0, pr, sc, zr);
         }
+    // Before each barrier a wavefront waits for its own A-tile DMAs explicitly: the wait the
+    // compiler derives for them may be placed behind the barrier, where it no longer says anything
+    // about the fragments the OTHER wavefronts moved.
     for (int kt = kt_begin; kt < KT; kt += 2)
     {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
         compute(a_buf0, st0, st1, a_buf1, kt + 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         compute(a_buf1, st1, st0, a_buf0, kt + 2); // past the end of K both operands read as zeros: no branch needed
     }
