@@ -39,7 +39,7 @@ CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # calibrated with a 256 MiB copy (profiles/stream_gemv_gate_up_m1_hbm_traffic.md); counters cannot
 # be read from inside this process, so the figure is the recorded one
-DOMINANT_TRAFFIC_BYTES = 62_613_000
+DOMINANT_TRAFFIC_BYTES = 62_640_000
 
 
 def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
