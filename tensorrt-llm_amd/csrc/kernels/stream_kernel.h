@@ -632,15 +632,22 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     if constexpr (ALDS)
     {
         lds = stream_act_lds_bytes(sp.m, sp.k, TK) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO);
-        if (lds > kStreamMaxActLds)
+        // the reduction buffer of the epilogue is static LDS of this variant and shares the CU's 160 KiB
+        constexpr size_t kStaticLds = (size_t) WAVES * NS * MT * 4 * 64 * sizeof(float);
+        constexpr size_t kMaxDynamic = stream_max_staged_lds(NS * MT, WAVES);
+        static_assert(kStaticLds + kMaxDynamic <= 160 * 1024, "LDS of one CU");
+        if (lds > kMaxDynamic)
             return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
         static bool raised = false; // benign race: the attribute call is idempotent
         if (lds > 32 * 1024 && !raised)
         {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kStreamMaxActLds);
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxDynamic);
             if (e != hipSuccess)
+            {
+                (void) hipGetLastError(); // do not leave the error for the caller's next runtime call
                 return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            }
             raised = true;
         }
     }

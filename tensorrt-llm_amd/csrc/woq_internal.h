@@ -205,7 +205,12 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;
 constexpr int kStreamW4a8MaxM = 16;
-// most LDS a streaming workgroup stages its operands in (activations, group scales and zeros)
-constexpr size_t kStreamMaxActLds = 96 * 1024;
+// most LDS a streaming workgroup stages its operands in (activations, group scales and zeros, row
+// sums): what the CU's 160 KiB leave next to the static reduction buffer of the epilogue
+// (`slots` = strips per wavefront x 16-row tiles, 256 floats per slot and wavefront)
+constexpr size_t stream_max_staged_lds(int slots, int waves)
+{
+    return (size_t) 160 * 1024 - (size_t) waves * slots * 1024 - 2048;
+}
 
 } // namespace woq

@@ -167,6 +167,15 @@ def test_stream_long_k_staged_operands(pkg, oracle, dev, M, K, group, bits):
     assert err < TOL, err
 
 
+@pytest.mark.parametrize("M", [2, 4])
+def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, M):
+    """Few column groups and a long K (a down projection at M = 2..4): the activations are staged in
+    LDS although they take 57 / 115 KiB, since one workgroup per CU covers the problem anyway."""
+    p = random_problem(oracle, M, 14336, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
 def test_stream_activations_too_large_for_lds(pkg, oracle, dev):
     """M x K beyond the LDS staging area falls back to register-held activation fragments."""
     p = random_problem(oracle, 16, 4096, 64, 4, 128, "bf16", zero=True, seed=77)
