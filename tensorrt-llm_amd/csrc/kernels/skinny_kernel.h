@@ -7,7 +7,9 @@
 // kernel's arithmetic on a GEMM skeleton:
 //   * the packed integers are expanded to the activation type by one bit operation per pair
 //     (value q + OFFSET, exact) and multiplied as they are; per scale group the matrix core
-//     produces P = sum a * (q + OFFSET) and, against an all-ones operand, S = sum a;
+//     produces P = sum a * (q + OFFSET) and, against an all-ones operand, S = sum a (the row sums
+//     are the same for every wavefront of the workgroup: with group scales each (group, row
+//     tile) is summed by ONE wavefront, a step ahead, and shared through LDS);
 //   * the scale is applied to the float32 sums, once per group and output element:
 //     acc += s * P + (z - OFFSET * s) * S.
 // Output tile 64 (32 for M <= 32, int4) rows x 256 columns; 8 wavefronts side by side along N,
@@ -45,14 +47,27 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // One LDS object per step in flight.  They are separate variables on purpose: the compiler
     // orders an LDS read after the DMA writes to the SAME variable only, so reading step kt's
     // buffer does not wait for the DMA just issued into another one.
-    struct StageLds
+    // (The A tile and the scale slots of a step are separate objects too: the row sums of step kt+1
+    // are formed from its A tile while its scales are still in flight.)
+    struct StageA
     {
         u32x4 a[A_BYTES / 16];
+    };
+    struct StageSc
+    {
         u32x4 sc[kSkinnyWaves][(SC_SLOTS ? SC_SLOTS : 1) * 16];
     };
     static_assert(DEPTH + 1 <= 7, "seven stage buffers are declared");
-    __shared__ StageLds lds0, lds1, lds2, lds3, lds4, lds5, lds6;
-    StageLds* const stage_lds[7] = {&lds0, &lds1, &lds2, &lds3, &lds4, &lds5, &lds6};
+    __shared__ StageA lda0, lda1, lda2, lda3, lda4, lda5, lda6;
+    __shared__ StageSc ldc0, ldc1, ldc2, ldc3, ldc4, ldc5, ldc6;
+    StageA* const stage_a[7] = {&lda0, &lda1, &lda2, &lda3, &lda4, &lda5, &lda6};
+    StageSc* const stage_sc[7] = {&ldc0, &ldc1, &ldc2, &ldc3, &ldc4, &ldc5, &ldc6};
+    // row sums S of the activations: per step slot, (group of the step, row tile), 16 rows.
+    // (Spreading the work over all eight wavefronts - two slabs each, partial sums added by the
+    // readers - measured slower than leaving it to SEGS * RT of them.)
+    constexpr int SUM_UNITS = GROUP != 0 ? SEGS * RT : 1;
+    static_assert(SUM_UNITS <= kSkinnyWaves, "one wavefront per (group, row tile)");
+    __shared__ f32x4 sum_lds[7][SUM_UNITS][4];
 
     int t;
     if (!xcd_tile(p.tiles_m * p.tiles_n, t))
@@ -130,7 +145,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             uint32_t const off
                 = ((row * (uint32_t) K + (uint32_t) kk) * 2u) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(act_rsrc,
-                (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(stage_lds[buf]->a) + f * 1024), 16,
+                (__attribute__((address_space(3))) void*) (reinterpret_cast<char*>(stage_a[buf]->a) + f * 1024), 16,
                 (int) off, 0, 0, 0);
         }
     };
@@ -163,7 +178,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             {
                 uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
                 uint32_t const off = ((grow * (uint32_t) p.n + sc_lane_col) * 2u) | past | sc_lane_oob;
-                char* slot = reinterpret_cast<char*>(stage_lds[buf]->sc[wave]) + seg * (ZERO ? 512 : 256);
+                char* slot = reinterpret_cast<char*>(stage_sc[buf]->sc[wave]) + seg * (ZERO ? 512 : 256);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
                     sc_rsrc, (__attribute__((address_space(3))) void*) slot, 4, (int) off, 0, 0, 0);
                 if constexpr (ZERO)
@@ -218,10 +233,31 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             return expand_int8_reg<DT>(w[2 * j + pr / 2], pr % 2);
     };
 
-    auto compute = [&](int buf, Stage const& st)
+    // Row sums of the step whose A tile sits in buffer `buf`: wavefront w < SUM_UNITS sums (group
+    // w / RT, row tile w % RT) against the all-ones operand and leaves the 16 sums in that slot.
+    auto form_sums = [&](int buf)
     {
-        char const* a_base = reinterpret_cast<char const*>(stage_lds[buf]->a) + a_lane_off;
-        [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_lds[buf]->sc[wave]) + c * 2;
+        if constexpr (GROUP != 0)
+        {
+            if (wave < SUM_UNITS)
+            {
+                int const seg = wave / RT, rt = wave % RT; // wave-uniform
+                char const* frag
+                    = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off + (rt * SLABS + seg * SEG_SLABS) * 1024;
+                f32x4 sum = zero4;
+#pragma unroll
+                for (int js = 0; js < SEG_SLABS; ++js)
+                    sum = E::mma(*reinterpret_cast<u32x4 const*>(frag + js * 1024), ones, sum);
+                if (c == 0) // every column of the block holds the same sums; rows kg*4 .. kg*4+3
+                    sum_lds[buf][wave][kg] = sum;
+            }
+        }
+    };
+
+    auto compute = [&](int buf, int buf_next, Stage const& st)
+    {
+        char const* a_base = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off;
+        [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_sc[buf]->sc[wave]) + c * 2;
         u32x4 a[RT][SLABS];
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
@@ -260,27 +296,37 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 }
         }
 
-        // S of every group of the step (per-channel mode: the running S); the first B operand is
-        // expanded underneath
         u32x4 b_cur, b_nxt;
+        if constexpr (GROUP != 0)
+        {
+            // this wavefront's share of the NEXT step's S, from the next A tile (it has landed: see
+            // WAIT); this step's S was formed during the previous step and is read when the first
+            // strip is done (until then the registers still hold the previous step's)
+            form_sums(buf_next);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < SLABS; ++j)
+            for (int x = 0; x < 4; ++x)
+                b_cur[x] = expand_reg(st.w[0], 0, x);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        else
+        {
+            // per-channel mode: the running S; the first B operand is expanded underneath
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-            {
-                if constexpr (GROUP != 0)
-                    part_s[j / SEG_SLABS][rt]
-                        = E::mma(a[rt][j], ones, j % SEG_SLABS == 0 ? zero4 : part_s[j / SEG_SLABS][rt]);
-                else
-                    acc_s[rt] = E::mma(a[rt][j], ones, acc_s[rt]);
-                if (j == SLABS - 1)
+            for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
                 {
+                    acc_s[rt] = E::mma(a[rt][j], ones, acc_s[rt]);
+                    if (j == SLABS - 1)
+                    {
 #pragma unroll
-                    for (int x = rt * PER_B; x < (rt + 1) * PER_B; ++x)
-                        b_cur[x] = expand_reg(st.w[0], 0, x);
+                        for (int x = rt * PER_B; x < (rt + 1) * PER_B; ++x)
+                            b_cur[x] = expand_reg(st.w[0], 0, x);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-            }
+        }
 
 #pragma unroll
         for (int s = 0; s < NS; ++s)
@@ -305,6 +351,17 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                         else if (s + 1 < NS)
                             b_nxt[x] = expand_reg(st.w[s + 1], 0, x);
                     }
+                    if constexpr (GROUP != 0)
+                    {
+                        if (s == 0 && j == SLABS - 1 && rt == RT - 1)
+                        {
+#pragma unroll
+                            for (int seg = 0; seg < SEGS; ++seg)
+#pragma unroll
+                                for (int rt2 = 0; rt2 < RT; ++rt2)
+                                    part_s[seg][rt2] = sum_lds[buf][seg * RT + rt2][kg];
+                        }
+                    }
                     if (s > 0)
                     {
                         constexpr int BLOCKS = SLABS * RT; // mini-blocks per strip
@@ -327,8 +384,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // goes into the buffer A(kt-1) used), compute step kt.
     // Vector-memory operations retire in order, so "step kt has landed" is "at most the requests
     // of the DEPTH-1 younger steps are outstanding".
-    constexpr int WAIT = (DEPTH - 1) * (FETCH_OPS + DMA_OPS);
-    static_assert(WAIT < 64, "vmcnt is a 6-bit counter");
+    // With group scales the A tile of step kt+1 must have landed as well (its row sums are formed
+    // during step kt): a step's requests are its A DMAs followed by its weight-side requests, so
+    // only the weight-side requests of step kt+1 may still be outstanding.
+    constexpr int WAIT = GROUP != 0 ? (DEPTH - 2) * (FETCH_OPS + DMA_OPS) + FETCH_OPS : (DEPTH - 1) * (FETCH_OPS + DMA_OPS);
+    static_assert(DEPTH >= 2 && WAIT < 64, "vmcnt is a 6-bit counter");
     Stage st[DEPTH + 1];
 #pragma unroll
     for (int i = 0; i < DEPTH; ++i)
@@ -337,18 +397,26 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         fetch_b(st[i], i, kt_begin + i);
         __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (GROUP != 0)
+    {
+        // row sums of the first step: its A tile has landed once at most the younger steps and its
+        // own weight-side requests are outstanding
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DEPTH - 1) * (FETCH_OPS + DMA_OPS) + FETCH_OPS) : "memory");
+        form_sums(0);
+    }
     for (int kt = kt_begin; kt < KT; kt += DEPTH + 1)
     {
 #pragma unroll
         for (int u = 0; u < DEPTH + 1; ++u)
         {
-            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WAIT) : "memory");
+            // (lgkmcnt: the row sums this wavefront wrote for step kt are in LDS before anyone reads them)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(WAIT) : "memory");
             __builtin_amdgcn_sched_barrier(0);
             dma_a((u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
             fetch_b(st[(u + DEPTH) % (DEPTH + 1)], (u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
             __builtin_amdgcn_sched_barrier(0);
             if (kt + u < KT) // uniform; the requests above go on (they read zeros past the end of K)
-                compute(u, st[u]);
+                compute(u, (u + 1) % (DEPTH + 1), st[u]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
