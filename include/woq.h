@@ -195,8 +195,8 @@ int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);
 /* Validation only (no launch): what woq_grouped_matmul would return for these arguments. */
 int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);
 
-/* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, < 2^26 for int8
- * weights; m <= 16 for W4A8), GEMM otherwise - crossovers measured on MI355X.  Counterpart of the tactic choice
+/* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, <= 2^26 for int8
+ * weights, m <= 64 for int8 when n*k <= 2^24; m <= 16 for W4A8), GEMM otherwise - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 

@@ -238,13 +238,15 @@ extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_
         return m <= kStreamW4a8MaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
     // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed; with two row
     // tiles the streaming kernel still wins on small matrices (it needs no split-K passes): up to
-    // 2^24 int4 weights, where the MFMA kernel has 32-row tiles, and below 2^26 int8 weights,
-    // where its tiles have 64 rows.  From 33 rows on the MFMA GEMM kernels are faster.
+    // 2^24 int4 weights and up to 2^26 int8 weights (up to 64 rows on int8 matrices of 2^24).
+    // Beyond that the MFMA GEMM kernels are faster.
     if (m <= 16)
         return WOQ_REGIME_STREAM;
     int64_t const weights = (int64_t) n * k;
-    bool const small = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? weights < ((int64_t) 1 << 26) : weights <= ((int64_t) 1 << 24);
-    if (m <= 32 && small)
+    bool const int8 = quant_algo & WOQ_ALGO_INT8_WEIGHT;
+    if (m <= 32 && weights <= ((int64_t) 1 << (int8 ? 26 : 24)))
+        return WOQ_REGIME_STREAM;
+    if (m <= 64 && int8 && weights <= ((int64_t) 1 << 24))
         return WOQ_REGIME_STREAM;
     return WOQ_REGIME_GEMM;
 }
@@ -287,10 +289,10 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     // the split-K region does not (large m does not split), so take its maximum over the row
     // counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
-    // the plan changes at multiples of the 64-row tile; kEnoughTiles or more tiles never split,
-    // which even one column of the tallest (256-row) tiles reaches at 256 * kEnoughTiles rows
+    // kEnoughTiles or more tiles never split, which even one column of the tallest (256-row) tiles
+    // reaches at 256 * kEnoughTiles rows; below that the plan may change at any row count
     size_t split = split_bytes(m, n, k, quant_algo);
-    for (int mm = 64; mm < m && mm <= 256 * (int) kEnoughTiles; mm += 64)
+    for (int mm = 1; mm < m && mm <= 256 * (int) kEnoughTiles; ++mm)
     {
         size_t const b = split_bytes(mm, n, k, quant_algo);
         split = b > split ? b : split;
@@ -352,10 +354,10 @@ extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
 
 namespace
 {
-// Kernel family and tile height of a grouped problem.  Only the total row count is known on the
-// host, so the choice goes by the average expert: streaming passes of 16 rows while that is at
-// most 16 rows; 64-row deferred-scale tiles up to 256; exact-dequantize 256-row tiles above (128
-// when those would not fill the chip).  K is never split.
+// Kernel family of a grouped problem.  Only the total row count is known on the host, so the choice
+// goes by the average expert: streaming passes of 16 rows while that is at most 16 rows, else the
+// tiled kernels (kernel and tile height by plan_gemm's estimate for the average expert; K is
+// never split).
 int grouped_regime(woq_grouped_matmul_args const* a)
 {
     int r = a->base.regime != WOQ_REGIME_AUTO ? a->base.regime : env_regime();
@@ -364,21 +366,6 @@ int grouped_regime(woq_grouped_matmul_args const* a)
     return r;
 }
 
-GemmPlan plan_grouped(int total_rows, int num_experts, int n)
-{
-    GemmPlan pl;
-    int const avg = (total_rows + num_experts - 1) / num_experts;
-    pl.skinny = avg <= 256;
-    if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
-        pl.skinny = !std::strcmp(e, "skinny");
-    if (pl.skinny)
-        pl.rt = 4;
-    else
-        pl.rt = (long) num_experts * gemm_tiles(avg, n, 16) >= kEnoughTiles ? 16 : 8;
-    pl.k_splits = 1;
-    pl.ws_bytes = 0;
-    return pl;
-}
 } // namespace
 
 extern "C" int woq_grouped_matmul_check(const woq_grouped_matmul_args* args)
@@ -433,9 +420,8 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     p.residual = args->residual;
     if (streaming)
         return launch_stream(p, stream);
-    GemmPlan plan = single ? plan_gemm(p.m, p.n, p.k, p.bits) : plan_grouped(p.m, p.num_experts, p.n);
-    plan.k_splits = 1;
-    plan.ws_bytes = 0;
+    // no K split: the tiles of one expert are not what is short here, and the epilogue fusions need the sums
+    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, p.bits, false, single ? 1 : p.num_experts);
     bool const two_pass = act != WOQ_ACT_IDENTITY && !gated;
     if (two_pass)
         p.residual = nullptr; // added behind the activation, by the pass below

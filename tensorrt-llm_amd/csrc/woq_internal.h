@@ -88,26 +88,6 @@ inline long gemm_tiles(int m, int n, int rt)
 // A launch fills the 256 CUs from about this many workgroups on; below it K is split.
 constexpr long kEnoughTiles = 160;
 
-// Tile height of the exact-dequantize kernels above 256 rows: the tallest tile amortises the
-// dequantize best (measured per-CU rates 1 : 0.87 : 0.58 for 256 : 128 : 64 rows), but only when
-// its tiles still fill the chip, and a partly filled last row tile is wasted matrix-core work.
-// Returns 0 when neither 256- nor 128-row tiles fill the chip.
-inline int tall_tile_rt(int m, int n)
-{
-    int best = 0;
-    double best_cost = 0;
-    for (int rt : {16, 8})
-    {
-        if (gemm_tiles(m, n, rt) < kEnoughTiles)
-            continue;
-        int const padded = (m + rt * 16 - 1) / (rt * 16) * (rt * 16);
-        double const cost = padded / (rt == 16 ? 1.0 : 0.87);
-        if (!best || cost < best_cost)
-            best = rt, best_cost = cost;
-    }
-    return best;
-}
-
 inline int auto_k_splits(long tiles, int k_tiles)
 {
     if (tiles >= kEnoughTiles || k_tiles < 8)
@@ -118,44 +98,81 @@ inline int auto_k_splits(long tiles, int k_tiles)
     return splits > 1 ? (int) splits : 1;
 }
 
-// Kernel, tile height and K split of a 16-bit GEMM-regime problem, from measured crossovers:
-//   * up to 256 rows the deferred-scale kernel (32-row tiles for int4 up to 32 rows, else 64-row);
-//   * above, the exact-dequantize kernel with the tallest tile that fills the chip; when neither
-//     256- nor 128-row tiles do, 128-row tiles with K split if K is long (>= 8192: the float32
-//     partial sums are then small next to the weight work), else the deferred-scale kernel.
+// Estimated time (microseconds) of a 16-bit GEMM-regime problem on one kernel and tile height, from
+// a model fitted to sweeps over the Llama-3-8B / 70B layer shapes (M = 32 .. 1024, int4 g64 / g128
+// and int8 per-channel; picking by it stays within 1 % of the best measured choice on average):
+//   * a workgroup spends c microseconds per tile row of K: c = a + b * rows for the exact-dequantize
+//     kernel (the dequantize is paid once per workgroup, the MFMAs per row), a constant for the
+//     deferred-scale kernel's 64-row (or 32-row) tile;
+//   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another;
+//   * splitting K costs two more launches and the float32 partial traffic.
+// `tiles` is the output tile count of that tile height (for a grouped problem: over all experts).
+inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, bool allow_split, int& splits)
+{
+    int const tk = tile_k_of_bits(bits);
+    int const k_tiles = (k + tk - 1) / tk;
+    double const per_k = bits == 4 ? 1.0 : 0.5; // a tile row of int8 covers half the K of an int4 one
+    double c;
+    if (skinny)
+        c = (bits == 4 ? 1.5 : 1.2) * per_k * (rt == 2 ? 0.72 : 1.0);
+    else
+        c = (0.8 + 0.007 * 16 * rt) * per_k;
+    splits = allow_split ? auto_k_splits(tiles, k_tiles) : 1;
+    long const rounds = (tiles * splits + 255) / 256;
+    int const steps = (k_tiles + splits - 1) / splits;
+    double t = (double) rounds * steps * c + 4.0;
+    if (splits > 1)
+        t += 5.0 + (double) m * n * 4.0 * (2 + 2 * splits) / (bits == 4 ? 1.5e6 : 2.5e6);
+    return t;
+}
+
+// Kernel, tile height and K split of a 16-bit GEMM-regime problem: the cheapest by gemm_cost_us of
+//   * the deferred-scale kernel (32-row tiles for int4 up to 32 rows, else 64-row tiles);
+//   * the exact-dequantize kernel with 64-, 128- or 256-row tiles.
 // Environment overrides for experiments: WOQ_GEMM_KERNEL=exact|skinny, WOQ_GEMM_RT=4|8|16 (exact
 // kernel), WOQ_GEMM_SPLITS=<n>
-inline GemmPlan plan_gemm(int m, int n, int k, int bits)
+inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true, int num_experts = 1)
 {
-    GemmPlan pl;
-    int exact_rt = m <= 64 ? 4 : (m <= 128 ? 8 : 16);
-    if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
-        pl.skinny = !std::strcmp(e, "skinny");
-    else if (m <= 256)
-        pl.skinny = true;
-    else if (int const rt = tall_tile_rt(m, n))
-        pl.skinny = false, exact_rt = rt;
-    else if (k >= 8192 && gemm_tiles(m, n, 8) >= 96)
-        pl.skinny = false, exact_rt = 8;
-    else
-        pl.skinny = true;
-    if (pl.skinny)
-        pl.rt = (m <= 32 && bits == 4) ? 2 : 4;
-    else
-        pl.rt = exact_rt;
+    // rows per expert of a grouped problem (its tiles do not straddle experts)
+    int const rows = num_experts > 1 ? (m + num_experts - 1) / num_experts : m;
+    int const skinny_rt = (rows <= 32 && bits == 4) ? 2 : 4;
+    char const* forced = std::getenv("WOQ_GEMM_KERNEL");
+    int forced_rt = 0;
     if (char const* r = std::getenv("WOQ_GEMM_RT"))
     {
         int const v = std::atoi(r);
-        if (!pl.skinny && (v == 4 || v == 8 || v == 16))
-            pl.rt = v;
+        if (v == 4 || v == 8 || v == 16)
+            forced_rt = v;
+    }
+    GemmPlan pl{};
+    double best = 0;
+    bool have = false;
+    for (int cand = 0; cand < 4; ++cand)
+    {
+        bool const skinny = cand == 0;
+        int const rt = skinny ? skinny_rt : (cand == 1 ? 4 : (cand == 2 ? 8 : 16));
+        if (forced && skinny != !std::strcmp(forced, "skinny"))
+            continue;
+        if (!skinny && forced_rt && rt != forced_rt)
+            continue;
+        int splits;
+        double const cost
+            = gemm_cost_us(skinny, rt, (long) num_experts * gemm_tiles(rows, n, rt), m, n, k, bits, allow_split, splits);
+        if (!have || cost < best)
+        {
+            have = true;
+            best = cost;
+            pl.skinny = skinny;
+            pl.rt = rt;
+            pl.k_splits = splits;
+        }
     }
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
-    pl.k_splits = auto_k_splits(gemm_tiles(m, n, pl.rt), k_tiles);
     if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
     {
         int const v = std::atoi(f);
-        if (v >= 1 && v <= k_tiles)
+        if (allow_split && v >= 1 && v <= k_tiles)
             pl.k_splits = v;
     }
     pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;

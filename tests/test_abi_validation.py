@@ -74,12 +74,16 @@ def test_workspace_rule(pkg):
     lib = L.lib
     algo = L.ALGO_PRE_QUANT_SCALE
     # the split-K partial buffer: none at m=4096 x n=4096 itself (256 tiles fill the chip), but the
-    # size covers every smaller m too, and up to 1152 rows (9 x 16 tiles of 128 rows) still split
-    split = 1152 * 4096 * 4
+    # size covers every smaller m too, and a few hundred rows still split K on this narrow N:
+    # whole float32 rows of the output, fewer than 4096 of them
+    split = lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16)
+    assert split % (4096 * 4) == 0 and 64 * 4096 * 4 <= split < 4096 * 4096 * 4
+    # the smoothed activations come on top
     assert lib.woq_workspace_bytes(4096, 4096, 8192, algo, L.BF16) == 4096 * 8192 * 2 + split
-    assert lib.woq_workspace_bytes(4096, 4096, 8192, 0, L.BF16) == split
     assert lib.woq_workspace_bytes(64, 4096, 8192, 0, L.BF16) == 64 * 4096 * 4
-    assert lib.woq_workspace_bytes(4096, 20480, 8192, 0, L.BF16) == 64 * 20480 * 4
+    # a wide N fills the chip with few rows: only the smallest row counts split
+    wide = lib.woq_workspace_bytes(4096, 20480, 8192, 0, L.BF16)
+    assert wide % (20480 * 4) == 0 and wide <= 128 * 20480 * 4
     # never shrinks as m grows
     sizes = [lib.woq_workspace_bytes(m, 1024, 4096, algo, L.FP16) for m in range(1, 3000, 37)]
     assert sizes == sorted(sizes)
@@ -112,7 +116,11 @@ def test_regime_table(pkg):
     assert sel(16, 28672, 4096, 0) == L.REGIME_STREAM
     assert sel(32, 6144, 4096, 0) == L.REGIME_GEMM  # int4: 32-row MFMA tiles win above 2^24 weights
     assert sel(32, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM
-    assert sel(32, 8192, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
+    assert sel(32, 8192, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM  # 2^26 int8 weights: still streaming
+    assert sel(32, 10240, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
+    assert sel(64, 4096, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM  # small int8 matrices stream up to 64 rows
+    assert sel(65, 4096, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
+    assert sel(64, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
     # W4A8: streaming kernel for one 16-row tile, the fp8 GEMM above
     assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
     assert sel(16, 57344, 8192, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
