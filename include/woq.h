@@ -74,8 +74,9 @@ typedef enum woq_regime
 {
     WOQ_REGIME_AUTO = 0,
     WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 16) */
-    WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMMs: 64-row deferred-scale tiles for skinny m, 256-row prefill
-                              tiles, the fp8 kernel for W4A8; may split K through the workspace */
+    WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMMs: deferred-scale 32/64-row tiles or exact-dequantize 64/128/256-row
+                              tiles (whichever is estimated cheaper for the shape), the fp8 kernel for W4A8;
+                              may split K through the workspace */
 } woq_regime;
 
 /*
