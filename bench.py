@@ -259,7 +259,7 @@ def bench_w4a8(pkg, dev, m=4096, reps=5):
 def run_for_counters(pkg, dev, mode, reps=20):
     """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
     dominant kernel (gate_up GEMV, rotating weight copies); `gemm<M>` launches the GEMM regime on
-    gate_up at M rows (prefill kernel at 4096, skinny kernel at 128); `copy` runs a plain device-to-device
+    gate_up at M rows (256-row tiles at 4096, 64-row tiles at 128); `copy` runs a plain device-to-device
     copy of a known size (256 MiB read + 256 MiB written per launch), whose FETCH_SIZE /
     WRITE_SIZE readings calibrate the counters."""
     if mode == "copy":
