@@ -65,7 +65,9 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // row sums S of the activations: per step slot, (group of the step, row tile), 16 rows.
     // (Spreading the work over all eight wavefronts - two slabs each, partial sums added by the
     // readers - measured slower than leaving it to SEGS * RT of them.)
-    constexpr int SUM_UNITS = GROUP != 0 ? SEGS * RT : 1;
+    // Per-channel scales need only the sums over the whole of K: every wavefront sums its share of
+    // each step's A fragments and the shares are added once, in the epilogue.
+    constexpr int SUM_UNITS = GROUP != 0 ? SEGS * RT : kSkinnyWaves;
     static_assert(SUM_UNITS <= kSkinnyWaves, "one wavefront per (group, row tile)");
     __shared__ f32x4 sum_lds[7][SUM_UNITS][4];
 
@@ -311,21 +313,19 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         }
         else
         {
-            // per-channel mode: the running S; the first B operand is expanded underneath
+            // per-channel mode: this wavefront's share of the running row sums (fragments
+            // wave * FPW .. of the step, all of one row tile), kept in acc_s[0] until the epilogue
+            // adds the shares up
+            constexpr int FPW = FRAGS / kSkinnyWaves;
+            static_assert(FPW >= 1 && SLABS % FPW == 0, "a wavefront's fragments belong to one row tile");
+            char const* frag = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off + wave * (FPW * 1024);
 #pragma unroll
-            for (int j = 0; j < SLABS; ++j)
+            for (int i = 0; i < FPW; ++i)
+                acc_s[0] = E::mma(*reinterpret_cast<u32x4 const*>(frag + i * 1024), ones, acc_s[0]);
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                {
-                    acc_s[rt] = E::mma(a[rt][j], ones, acc_s[rt]);
-                    if (j == SLABS - 1)
-                    {
-#pragma unroll
-                        for (int x = rt * PER_B; x < (rt + 1) * PER_B; ++x)
-                            b_cur[x] = expand_reg(st.w[0], 0, x);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+            for (int x = 0; x < 4; ++x)
+                b_cur[x] = expand_reg(st.w[0], 0, x);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
 #pragma unroll
@@ -421,6 +421,25 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // no DMA may still be writing LDS when the wavefront ends
+    if constexpr (GROUP == 0)
+    {
+        // row sums of the per-channel mode: add the wavefronts' shares (wavefront w summed row tile
+        // w * FPW / SLABS)
+        constexpr int FPW = FRAGS / kSkinnyWaves;
+        if (c == 0)
+            sum_lds[0][wave][kg] = acc_s[0];
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+        {
+            f32x4 t = zero4;
+#pragma unroll
+            for (int w = 0; w < kSkinnyWaves; ++w)
+                if (w * FPW / SLABS == rt)
+                    t += sum_lds[0][w][kg];
+            acc_s[rt] = t;
+        }
+    }
 #pragma unroll
     for (int u = 0; u < UNITS; ++u)
         apply_unit(NS - 1, u); // the last step's last strip
