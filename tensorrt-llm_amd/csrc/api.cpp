@@ -102,11 +102,13 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         }
         else if (strips <= 256 && rows <= 4 && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
             return {1, 8, 4, 1};
-        if (strips >= 1024)
-            return {4, 4, 2, 0};
-        if (strips >= 384)
-            return {2, 8, 2, 0};
-        return {1, 8, 4, 0};
+        // activations stay in registers; the group scales / zeros (at most k * ns bytes) are still
+        // staged while that leaves room for the resident workgroups the shape counts on
+        StreamShape reg = strips >= 1024 ? StreamShape{4, 4, 2, 0}
+                                         : (strips >= 384 ? StreamShape{2, 8, 2, 0} : StreamShape{1, 8, 4, 0});
+        if ((size_t) k * reg.ns <= (size_t) (reg.waves == 4 ? 32 : 64) * 1024)
+            reg.lds = 2;
+        return reg;
     }
     if (mt == 2)
         return {strips >= 1024 ? 2 : 1, 8, 2, 0};

@@ -75,11 +75,12 @@ struct StreamStage
 //       the all-ones MFMA out of the K loop
 // ACT   the epilogue applies p.activation; a gated activation (value column j, gate column j + n/2) pairs
 //       the strips of a wavefront (even slot: value half, odd slot: gate half), output [m, n/2]
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
     bool ACT = false>
 __device__ __forceinline__ void stream_body(StreamParams const& p)
 {
-    static_assert(!ALDS || MT == 1, "LDS-staged activations are for M <= 16");
+    constexpr bool ALDS = LDS == 1;
+    static_assert(LDS == 0 || MT == 1, "LDS-staged operands are for M <= 16");
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
@@ -88,7 +89,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     constexpr int SEGS = TK / SEG;
     constexpr float OFF = Offset<DT, BITS>::value;
     using Stage = StreamStage<NS, SLABS, SEGS, MT, PQS, ALDS>;
-    constexpr bool SLDS = ALDS && GROUP != 0; // group scales / zeros live in LDS as well
+    constexpr bool SCLDS = LDS != 0 && GROUP != 0; // group scales / zeros live in LDS
+    constexpr bool SUMLDS = ALDS && GROUP != 0;    // and so do the activation row sums
     constexpr int THREADS = WAVES * 64;
     extern __shared__ u32x4 act_lds[]; // ALDS: rows x (KT*TK*2 + 16) bytes, then scales, then zeros
 
@@ -158,8 +160,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
     // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
     // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
-    int const act_rows = p.m < 16 ? p.m : 16;
-    int const sc_rows = SLDS ? (KT * TK + (GROUP ? GROUP : 1) - 1) / (GROUP ? GROUP : 1) : 0;
+    int const act_rows = ALDS ? (p.m < 16 ? p.m : 16) : 0;
+    int const sc_rows = SCLDS ? (KT * TK + (GROUP ? GROUP : 1) - 1) / (GROUP ? GROUP : 1) : 0;
     constexpr uint32_t SC_ROW = NS * 32u;
     char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
     char* const zr_lds = sc_lds + (uint32_t) sc_rows * SC_ROW;
@@ -190,7 +192,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 }
             }
         }
-        if constexpr (GROUP != 0 && !SLDS)
+        if constexpr (GROUP != 0 && !SCLDS)
         {
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
@@ -233,7 +235,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                                 a[mt][r] = E::mul2(a[mt][r], st.sm[j][r]);
                         }
                     }
-                    if constexpr (!SLDS)
+                    if constexpr (!SUMLDS)
                         acc_s[mt] = E::mma(a[mt], ones, acc_s[mt]);
                 }
 #pragma unroll
@@ -254,7 +256,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 // a segment past the end of K carries zero activations, scale 0 and zero 0.
                 // Lane (kg, c) register r is output row kg*4 + r: with a single row (decode,
                 // m == 1) only r == 0 is ever stored, so the other three are not scaled.
-                if constexpr (SLDS) // rows kg*4 .. kg*4+3 of this segment's sums
+                if constexpr (SUMLDS) // rows kg*4 .. kg*4+3 of this segment's sums
                     acc_s[0] = *reinterpret_cast<f32x4 const*>(sum_lds + (uint32_t) (kt * SEGS + seg) * 64u + kg * 16u);
                 auto scale_rows = [&](auto rows_tag)
                 {
@@ -263,7 +265,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                     for (int s = 0; s < NS; ++s)
                     {
                         uint16_t s_raw, z_raw = 0;
-                        if constexpr (SLDS)
+                        if constexpr (SCLDS)
                         {
                             uint32_t const at
                                 = (uint32_t) ((kt * TK + seg * SEG) / (GROUP ? GROUP : 1)) * SC_ROW + (s * 16 + c) * 2u;
@@ -308,12 +310,68 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // compiler from sinking the prefetch below the compute (it would, to save registers).
     int const n_my = (KT - wave + WAVES - 1) / WAVES;
     auto kt_of = [&](int it) { return wave + it * WAVES; };
+    // staging of the group scales / zeros: 16-byte chunks of 8 columns, NS * 2 per group of K
+    int const sc_chunks = sc_rows * NS * 2;
+    auto sc_offset = [&](int idx, uint32_t& lds_at)
+    {
+        int const row = idx / (NS * 2), piece = idx - row * (NS * 2); // piece = strip slot * 2 + half
+        int strip = strip0 + (piece >> 1);
+        if (gated)
+        {
+            int const pair = strip0 / 2 + (piece >> 2);
+            strip = (pair < half_strips ? pair : half_strips - 1) + ((piece >> 1) & 1) * half_strips;
+        }
+        else if (strip >= p.strips)
+            strip = p.strips - 1;
+        lds_at = (uint32_t) row * SC_ROW + (uint32_t) piece * 16u;
+        return idx < sc_chunks ? ((uint32_t) row * (uint32_t) p.n + (uint32_t) (strip * 16 + (piece & 1) * 8)) * 2u
+                               : kOob;
+    };
+    // chunks past the first THREADS (long K): a plain loop after the weight prefetch is under way
+    auto stage_scales_tail = [&]()
+    {
+        for (int idx = threadIdx.x + THREADS; idx < sc_chunks; idx += THREADS)
+        {
+            uint32_t at;
+            uint32_t const off = sc_offset(idx, at);
+            *reinterpret_cast<u32x4*>(sc_lds + at) = buffer_load_x4(sc_rsrc, off);
+            if constexpr (ZERO)
+                *reinterpret_cast<u32x4*>(zr_lds + at) = buffer_load_x4(zr_rsrc, off);
+        }
+    };
     Stage st[PF];
     if constexpr (!ALDS)
     {
+        if constexpr (SCLDS)
+        {
+            // the staged scales are requested first, the weight and activation prefetch right
+            // behind them: loads complete in order, so the barrier waits for the scales only
+            uint32_t s_at;
+            uint32_t const off = sc_offset(threadIdx.x, s_at);
+            u32x4 const sv = buffer_load_x4(sc_rsrc, off);
+            u32x4 zv;
+            if constexpr (ZERO)
+                zv = buffer_load_x4(zr_rsrc, off);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < PF; ++i)
-            fetch(st[i], kt_of(i));
+            for (int i = 0; i < PF; ++i)
+                fetch(st[i], kt_of(i));
+            __builtin_amdgcn_sched_barrier(0);
+            if ((int) threadIdx.x < sc_chunks)
+            {
+                *reinterpret_cast<u32x4*>(sc_lds + s_at) = sv;
+                if constexpr (ZERO)
+                    *reinterpret_cast<u32x4*>(zr_lds + s_at) = zv;
+            }
+            stage_scales_tail();
+            __syncthreads();
+        }
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < PF; ++i)
+                fetch(st[i], kt_of(i));
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     else
@@ -327,7 +385,6 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         constexpr int UA = 2;
         int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
         int const act_chunks = act_rows * chunks_per_row;
-        int const sc_chunks = sc_rows * NS * 2; // 8 columns each
         auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
         {
             int const row = act_rows == 1 ? 0 : idx / chunks_per_row;
@@ -336,21 +393,6 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;
             bool const ok = idx < act_chunks && (int) ch * 8 < K;
             return ok ? ((uint32_t) row * (uint32_t) K + ch * 8u) * 2u : kOob;
-        };
-        auto sc_offset = [&](int idx, uint32_t& lds_at)
-        {
-            int const row = idx / (NS * 2), piece = idx - row * (NS * 2); // piece = strip slot * 2 + half
-            int strip = strip0 + (piece >> 1);
-            if (gated)
-            {
-                int const pair = strip0 / 2 + (piece >> 2);
-                strip = (pair < half_strips ? pair : half_strips - 1) + ((piece >> 1) & 1) * half_strips;
-            }
-            else if (strip >= p.strips)
-                strip = p.strips - 1;
-            lds_at = (uint32_t) row * SC_ROW + (uint32_t) piece * 16u;
-            return idx < sc_chunks ? ((uint32_t) row * (uint32_t) p.n + (uint32_t) (strip * 16 + (piece & 1) * 8)) * 2u
-                                   : kOob;
         };
         auto smooth = [&](u32x4 v, u32x4 sm)
         {
@@ -387,7 +429,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             if constexpr (PQS)
                 pv[u] = buffer_load_x4(pqs_rsrc, ch * 16u);
         }
-        if constexpr (SLDS)
+        if constexpr (SCLDS)
         {
             uint32_t const off = sc_offset(threadIdx.x, s_at);
             sv = buffer_load_x4(sc_rsrc, off);
@@ -405,10 +447,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             u32x4 const v = PQS ? smooth(av[u], pv[u]) : av[u];
             if ((int) threadIdx.x + u * THREADS < act_chunks)
                 *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = v;
-            if constexpr (SLDS)
+            if constexpr (SUMLDS)
                 stage_sum(v, threadIdx.x + u * THREADS, sum_at[u]);
         }
-        if constexpr (SLDS)
+        if constexpr (SCLDS)
         {
             if ((int) threadIdx.x < sc_chunks)
             {
@@ -424,20 +466,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             if constexpr (PQS)
                 v = smooth(v, buffer_load_x4(pqs_rsrc, ch * 16u));
             *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + at) = v;
-            if constexpr (SLDS)
+            if constexpr (SUMLDS)
                 stage_sum(v, idx, sum_at);
         }
-        if constexpr (SLDS)
-        {
-            for (int idx = threadIdx.x + THREADS; idx < sc_chunks; idx += THREADS)
-            {
-                uint32_t at;
-                uint32_t const off = sc_offset(idx, at);
-                *reinterpret_cast<u32x4*>(sc_lds + at) = buffer_load_x4(sc_rsrc, off);
-                if constexpr (ZERO)
-                    *reinterpret_cast<u32x4*>(zr_lds + at) = buffer_load_x4(zr_rsrc, off);
-            }
-        }
+        if constexpr (SCLDS)
+            stage_scales_tail();
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -546,16 +579,16 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     }
 }
 
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS>
 __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 {
-    stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>(p);
+    stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS>(p);
 }
 
 // Grouped problems: workgroup (x, e) is workgroup x of expert e's own matmul.  The parameters are
 // narrowed to that expert's operands and rows; an expert with more than 16 rows streams its
 // weights once per 16 rows (this kernel is chosen when that is rare).
-template <int DT, int BITS, int GROUP, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
+template <int DT, int BITS, int GROUP, bool ZERO, int NS, int WAVES, int PF, int LDS>
 __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams p)
 {
     int const e = (int) blockIdx.y;
@@ -580,7 +613,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams
     for (; rows_left > 0; rows_left -= 16)
     {
         p.m = rows_left;
-        stream_body<DT, BITS, GROUP, false, ZERO, 1, NS, WAVES, PF, ALDS, true>(p);
+        stream_body<DT, BITS, GROUP, false, ZERO, 1, NS, WAVES, PF, LDS, true>(p);
         __syncthreads(); // this pass is done with the LDS areas
         p.act = static_cast<char const*>(p.act) + (size_t) 16 * (size_t) p.k * 2;
         p.out = static_cast<char*>(p.out) + (size_t) 16 * (size_t) n_out * 2;
@@ -590,7 +623,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_grouped_kernel(StreamParams
 }
 
 // launch shape: NS strips per wavefront, WAVES wavefronts per workgroup, PF tile rows in flight,
-// lds != 0: activations staged in LDS
+// lds = 1: activations, group scales / zeros and activation row sums staged in LDS; lds = 2: only
+// the group scales / zeros (activations in registers); lds = 0: nothing staged
 struct StreamShape
 {
     int ns, waves, pf, lds;
@@ -603,41 +637,42 @@ inline size_t stream_act_lds_bytes(int m, int k, int tile_k)
     return (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
 }
 
-// bytes of LDS the staged group scales (and zeros) of ns strips and the activation row sums take
-inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool zeros)
+// bytes of LDS the staged group scales (and zeros) of ns strips and, with sums, the activation row
+// sums take
+inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool zeros, bool sums)
 {
     if (group == 0)
         return 0;
     size_t const k_padded = (size_t) ((k + tile_k - 1) / tile_k) * tile_k;
     size_t const seg = group > tile_k ? tile_k : group; // rows of K per activation row sum
-    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1) + k_padded / seg * 64;
+    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1) + (sums ? k_padded / seg * 64 : 0);
 }
 
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k);
 
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, bool ALDS,
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
     bool GROUPED = false>
 int launch_stream_variant(StreamParams sp, hipStream_t stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
     auto kernel = [] {
         if constexpr (GROUPED)
-            return stream_grouped_kernel<DT, BITS, GROUP, ZERO, NS, WAVES, PF, ALDS>;
+            return stream_grouped_kernel<DT, BITS, GROUP, ZERO, NS, WAVES, PF, LDS>;
         else
-            return stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, ALDS>;
+            return stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS>;
     }();
     size_t lds = 0;
-    if constexpr (ALDS)
+    if constexpr (LDS != 0)
     {
-        lds = stream_act_lds_bytes(sp.m, sp.k, TK) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO);
+        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO, LDS == 1);
         // the reduction buffer of the epilogue is static LDS of this variant and shares the CU's 160 KiB
         constexpr size_t kStaticLds = (size_t) WAVES * NS * MT * 4 * 64 * sizeof(float);
         constexpr size_t kMaxDynamic = stream_max_staged_lds(NS * MT, WAVES);
         static_assert(kStaticLds + kMaxDynamic <= 160 * 1024, "LDS of one CU");
         if (lds > kMaxDynamic)
-            return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
+            return fail(WOQ_ERR_UNSUPPORTED, "staged operands of %zu bytes do not fit the LDS staging area", lds);
         static bool raised = false; // benign race: the attribute call is idempotent
         if (lds > 32 * 1024 && !raised)
         {
@@ -665,31 +700,40 @@ template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    StreamShape const sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK);
+    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK);
+    if (GROUP == 0 && sh.lds == 2)
+        sh.lds = 0; // per-channel scales are applied once, in the epilogue: nothing to stage
 #define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
-    if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                      \
+    if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                             \
         return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, MT_, NS_, WAVES_, PF_, LDS_>(sp, s);
     // decode (M <= 16), activations in LDS
-    WOQ_SHAPE(1, 1, 8, 4, true)
-    WOQ_SHAPE(1, 1, 8, 6, true)
-    WOQ_SHAPE(1, 1, 16, 4, true)
-    WOQ_SHAPE(1, 2, 8, 4, true)
-    WOQ_SHAPE(1, 2, 4, 4, true)
-    WOQ_SHAPE(1, 4, 4, 2, true)
-    WOQ_SHAPE(1, 4, 4, 4, true)
-    WOQ_SHAPE(1, 4, 8, 2, true)
-    WOQ_SHAPE(1, 4, 8, 4, true)
+    WOQ_SHAPE(1, 1, 8, 4, 1)
+    WOQ_SHAPE(1, 1, 8, 6, 1)
+    WOQ_SHAPE(1, 1, 16, 4, 1)
+    WOQ_SHAPE(1, 2, 8, 4, 1)
+    WOQ_SHAPE(1, 2, 4, 4, 1)
+    WOQ_SHAPE(1, 4, 4, 2, 1)
+    WOQ_SHAPE(1, 4, 4, 4, 1)
+    WOQ_SHAPE(1, 4, 8, 2, 1)
+    WOQ_SHAPE(1, 4, 8, 4, 1)
     // decode, activations in registers (M x K too large for LDS)
-    WOQ_SHAPE(1, 1, 8, 4, false)
-    WOQ_SHAPE(1, 2, 8, 2, false)
-    WOQ_SHAPE(1, 4, 4, 2, false)
+    WOQ_SHAPE(1, 1, 8, 4, 0)
+    WOQ_SHAPE(1, 2, 8, 2, 0)
+    WOQ_SHAPE(1, 4, 4, 2, 0)
+    if constexpr (GROUP != 0)
+    {
+        // decode, activations in registers, group scales / zeros in LDS
+        WOQ_SHAPE(1, 1, 8, 4, 2)
+        WOQ_SHAPE(1, 2, 8, 2, 2)
+        WOQ_SHAPE(1, 4, 4, 2, 2)
+    }
     // skinny M
-    WOQ_SHAPE(2, 2, 8, 2, false)
-    WOQ_SHAPE(2, 1, 8, 2, false)
-    WOQ_SHAPE(4, 1, 8, 1, false)
-    WOQ_SHAPE(4, 2, 8, 1, false)
-    WOQ_SHAPE(8, 1, 4, 1, false)
-    WOQ_SHAPE(8, 1, 8, 1, false)
+    WOQ_SHAPE(2, 2, 8, 2, 0)
+    WOQ_SHAPE(2, 1, 8, 2, 0)
+    WOQ_SHAPE(4, 1, 8, 1, 0)
+    WOQ_SHAPE(4, 2, 8, 1, 0)
+    WOQ_SHAPE(8, 1, 4, 1, 0)
+    WOQ_SHAPE(8, 1, 8, 1, 0)
 #undef WOQ_SHAPE
     return fail(WOQ_ERR_UNSUPPORTED, "stream shape mt=%d ns=%d waves=%d pf=%d lds=%d is not instantiated", mt, sh.ns,
         sh.waves, sh.pf, sh.lds);
@@ -703,16 +747,24 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
     // every expert's column groups run side by side: the grid is num_experts times taller
     StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK);
     if (act_is_gated(sp.activation) && sh.ns == 1) // value and gate strips pair up inside a wavefront
-        sh = sh.lds ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, 0};
+        sh = sh.lds == 1 ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, sh.lds};
+    if (GROUP == 0 && sh.lds == 2)
+        sh.lds = 0;
 #define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
-    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                                   \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                                          \
         return launch_stream_variant<DT, BITS, GROUP, false, ZERO, 1, NS_, WAVES_, PF_, LDS_, true>(sp, s);
-    WOQ_SHAPE(1, 8, 4, true)
-    WOQ_SHAPE(2, 8, 4, true)
-    WOQ_SHAPE(4, 8, 2, true)
-    WOQ_SHAPE(1, 8, 4, false)
-    WOQ_SHAPE(2, 8, 2, false)
-    WOQ_SHAPE(4, 4, 2, false)
+    WOQ_SHAPE(1, 8, 4, 1)
+    WOQ_SHAPE(2, 8, 4, 1)
+    WOQ_SHAPE(4, 8, 2, 1)
+    WOQ_SHAPE(1, 8, 4, 0)
+    WOQ_SHAPE(2, 8, 2, 0)
+    WOQ_SHAPE(4, 4, 2, 0)
+    if constexpr (GROUP != 0)
+    {
+        WOQ_SHAPE(1, 8, 4, 2)
+        WOQ_SHAPE(2, 8, 2, 2)
+        WOQ_SHAPE(4, 4, 2, 2)
+    }
 #undef WOQ_SHAPE
     return fail(WOQ_ERR_UNSUPPORTED, "grouped stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated", sh.ns,
         sh.waves, sh.pf, sh.lds);

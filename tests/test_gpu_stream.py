@@ -131,7 +131,7 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
 
 
 STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,1", "4,4,4,1", "4,8,2,1", "4,8,4,1",
-                 "1,8,4,0", "2,8,2,0", "4,4,2,0"]
+                 "1,8,4,0", "2,8,2,0", "4,4,2,0", "1,8,4,2", "2,8,2,2", "4,4,2,2"]
 
 
 @pytest.mark.parametrize("shape", STREAM_SHAPES)
@@ -179,5 +179,14 @@ def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, M):
 def test_stream_activations_too_large_for_lds(pkg, oracle, dev):
     """M x K beyond the LDS staging area falls back to register-held activation fragments."""
     p = random_problem(oracle, 16, 4096, 64, 4, 128, "bf16", zero=True, seed=77)
+    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    assert err < TOL, err
+
+
+@pytest.mark.parametrize("K,group", [(28672, 64), (66048, 128)])
+def test_stream_register_activations_long_k(pkg, oracle, dev, K, group):
+    """More rows than the LDS holds and a long K: the group scales / zeros are staged in more than
+    one pass (28672 / 64 groups), or not at all when even they are too many (K = 66048)."""
+    p = random_problem(oracle, 9, K, 48, 4, group, "bf16", zero=True, seed=K % 1000)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
     assert err < TOL, err
