@@ -87,20 +87,22 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         int const rows = m < 16 ? m : 16;
         size_t const act_lds = (size_t) rows * ((size_t) ((k + tile_k - 1) / tile_k) * tile_k * 2 + 16);
         // the group scales and zeros are staged next to the activations (at most k * ns bytes, and k more
-        // for the activation row sums).  Staging pays as long as it does not cost resident workgroups:
-        // always up to ~48 KiB of activations; beyond that only when one workgroup per CU covers the
-        // whole problem anyway and the rows are few (few column groups, long K: the down projections
-        // at M = 2..4; with more rows the staging traffic itself outweighs the gain)
+        // for the activation row sums).  Staging the activations pays for a single row (the kernel
+        // then scales one output row only) up to ~48 KiB, for more rows up to ~20 KiB (M = 2 at
+        // K = 4096; beyond that register-held fragments with staged scales measure faster: the
+        // staging pass and the resident workgroups it costs outweigh the shared reads), and with
+        // few column groups and at most 3 rows, where one workgroup per CU covers the whole problem
+        // anyway (the down projections: long K, N <= 4096)
         StreamShape const sh = strips >= 1024 ? StreamShape{4, 8, 2, 1}
                                               : (strips >= 384 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
-        if (act_lds <= 48 * 1024)
+        if (act_lds <= (size_t) (rows == 1 ? 48 : 20) * 1024)
         {
             if (act_lds + (size_t) k * (sh.ns + 1) <= stream_max_staged_lds(sh.ns, sh.waves))
                 return sh;
             if (act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
                 return {1, 8, 4, 1};
         }
-        else if (strips <= 256 && rows <= 4 && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
+        else if (strips <= 256 && rows <= 3 && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
             return {1, 8, 4, 1};
         // activations stay in registers; the group scales / zeros (at most k * ns bytes) are still
         // staged while that leaves room for the resident workgroups the shape counts on

@@ -156,21 +156,26 @@ def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
 
 
 @pytest.mark.parametrize("M,K,group,bits", [(1, 8192, 64, 4), (3, 8192, 64, 4), (2, 4160, 64, 4), (5, 4096, 128, 8)])
-def test_stream_long_k_staged_operands(pkg, oracle, dev, M, K, group, bits):
-    """Long K with four strips per wavefront: the activations, the group scales / zeros and the
+def test_stream_long_k_staged_operands(pkg, oracle, dev, monkeypatch, M, K, group, bits):
+    """Long K with four strips per wavefront (launch shape forced): the activations, the group scales / zeros and the
     activation row sums staged in LDS exceed what a thread keeps in registers across the weight
     prefetch (the staging tail loops run), take more than 64 KiB of LDS, and K = 4160 ends in half
     a weight tile whose scales, zeros and row sums must read as zero."""
     N = 16384
+    monkeypatch.setenv("WOQ_STREAM_SHAPE", "4,8,2,1")
     p = random_problem(oracle, M, K, N, bits, group, "bf16", zero=True, pqs=True, seed=K + M)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
     assert err < TOL, err
 
 
 @pytest.mark.parametrize("M", [2, 4])
-def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, M):
+@pytest.mark.parametrize("forced", [False, True])
+def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, monkeypatch, M, forced):
     """Few column groups and a long K (a down projection at M = 2..4): the activations are staged in
-    LDS although they take 57 / 115 KiB, since one workgroup per CU covers the problem anyway."""
+    LDS although they take 57 / 115 KiB (by the heuristic up to 3 rows, since one workgroup per CU
+    covers the problem anyway; forced for 4)."""
+    if forced:
+        monkeypatch.setenv("WOQ_STREAM_SHAPE", "1,8,4,1")
     p = random_problem(oracle, M, 14336, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
     assert err < TOL, err
