@@ -201,6 +201,40 @@ int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 
+/* ---- tactic profiler ------------------------------------------------------------------------ */
+
+/* Times, on `stream`, every candidate way this library has of running the 16-bit problem `args`
+ * describes (streaming launch shapes; deferred-scale / exact-dequantize GEMM kernels, tile heights
+ * and K splits) for every m in [min_m, 15], the powers of two from 16 below max_m, and max_m, and
+ * records the fastest per row count in a process-wide table.  Later woq_matmul calls with
+ * regime AUTO on the same (n, k, quant_algo, group_size, out_dtype) use the entry of their m, else
+ * of the next profiled row count above it, else the built-in heuristics (also when the workspace
+ * they are given is too small for the tuned choice).  Replaces
+ * GemmPluginProfiler::profileTactics (plugins/common/gemmPluginProfiler.cpp:118-216, timing loop
+ * :329-367, lookup :221-250) as called from the plugins' configGemm / initialize
+ * (weightOnlyQuantMatmulPlugin.cpp:255-275).  A set-up call: the buffers of `args` must hold
+ * max_m rows (workspace: woq_workspace_bytes for max_m; candidates that need more are skipped),
+ * `out` is overwritten, the stream is synchronised, 512 MiB of device memory are allocated and
+ * freed (the last-level cache is evicted between timed runs), and it must not run under stream
+ * capture.  W4A8 problems have one kernel per regime: accepted, nothing recorded. */
+int woq_profile_tactics(const woq_matmul_args* args, int32_t min_m, int32_t max_m, void* stream);
+
+/* Entries in the table; emptying it (back to the heuristics). */
+int woq_tactic_count(void);
+void woq_clear_tactics(void);
+
+/* Writes what a woq_matmul call with these arguments would go by: "heuristic", or the tuned entry
+ * ("stream mt=.. ns=.. waves=.. pf=.. lds=..", "gemm exact|skinny rt=.. splits=.."). */
+int woq_describe_tactic(const woq_matmul_args* args, char* buf, size_t len);
+
+/* The table as text (one line per entry), so that it can be stored next to a model and loaded
+ * instead of profiling again: the reference serialises its tactic map into the engine
+ * (weightOnlyQuantMatmulPlugin.cpp:374-391, gemmPluginProfiler.cpp:69-116).  Export returns the
+ * bytes needed including the terminator and writes only if len suffices; import adds the entries
+ * of `text` to the table (all or none) and rejects text this library did not write. */
+size_t woq_export_tactics(char* buf, size_t len);
+int woq_import_tactics(const char* text);
+
 /* ---- host-side weight preparation (CPU buffers) ------------------------------------------- */
 
 /* Bytes of the preprocessed weight of one [k, n] matrix.  Equals k*n*bits/8 whenever k is a

@@ -76,6 +76,12 @@ def _load():
         "woq_apply_per_channel_scale": (ctypes.c_int, [vp, vp, vp, i32, i32, i32, i32, vp]),
         "woq_rmsnorm_prequant": (ctypes.c_int, [vp, vp, vp, vp, vp, ctypes.c_float, i32, i32, i32, i32, vp]),
         "woq_dequantize": (ctypes.c_int, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
+        "woq_profile_tactics": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), i32, i32, vp]),
+        "woq_tactic_count": (ctypes.c_int, []),
+        "woq_clear_tactics": (None, []),
+        "woq_describe_tactic": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_char_p, sz]),
+        "woq_export_tactics": (sz, [ctypes.c_char_p, sz]),
+        "woq_import_tactics": (ctypes.c_int, [ctypes.c_char_p]),
         "woq_last_error": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),
         "woq_layout_version": (ctypes.c_int, []),

@@ -32,11 +32,28 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream);
 
 int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream);
 
+// plan of a plain (not grouped) 16-bit GEMM-regime call: the tactic in force, else the cost model's
+GemmPlan planned_gemm(int m, int n, int k, int bits)
+{
+    Tactic const* t = current_tactic();
+    if (t && t->regime == WOQ_REGIME_GEMM && t->rt != 0 && (t->rt != 2 || (t->skinny && bits == 4)))
+    {
+        GemmPlan pl{};
+        pl.skinny = t->skinny != 0;
+        pl.rt = t->rt;
+        int const k_tiles = (k + tile_k_of_bits(bits) - 1) / tile_k_of_bits(bits);
+        pl.k_splits = t->k_splits < 1 ? 1 : (t->k_splits > k_tiles ? k_tiles : t->k_splits);
+        pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+        return pl;
+    }
+    return plan_gemm(m, n, k, bits);
+}
+
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_gemm_w4a8(p, stream);
-    return launch_gemm_planned(p, plan_gemm(p.m, p.n, p.k, p.bits), stream);
+    return launch_gemm_planned(p, planned_gemm(p.m, p.n, p.k, p.bits), stream);
 }
 
 int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream)
@@ -82,6 +99,11 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
             return sh;
     }
     (void) k_tiles;
+    if (Tactic const* t = current_tactic())
+    {
+        if (t->regime == WOQ_REGIME_STREAM && t->ns != 0 && t->mt == mt)
+            return {t->ns, t->waves, t->pf, t->lds};
+    }
     if (mt == 1)
     {
         int const rows = m < 16 ? m : 16;
@@ -224,6 +246,8 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
 int pick_regime(woq_matmul_args const* a)
 {
     int r = a->regime != WOQ_REGIME_AUTO ? a->regime : env_regime();
+    if (r == WOQ_REGIME_AUTO && current_tactic())
+        r = current_tactic()->regime;
     if (r == WOQ_REGIME_AUTO)
         r = woq_select_regime(a->m, a->n, a->k, a->quant_algo);
     return r;
@@ -274,7 +298,7 @@ static size_t split_bytes(int m, int n, int k, int quant_algo)
 {
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
         return plan_gemm_w4a8(m, n, k).ws_bytes;
-    return plan_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
+    return planned_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
 }
 
 // what one GEMM-regime call with exactly m rows uses
@@ -301,7 +325,8 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
         size_t const b = split_bytes(mm, n, k, quant_algo);
         split = b > split ? b : split;
     }
-    bytes += split;
+    size_t const tuned = tuned_split_bytes(m, n, k, quant_algo);
+    bytes += split > tuned ? split : tuned;
     return bytes;
 }
 
@@ -328,7 +353,30 @@ extern "C" int woq_matmul_check(const woq_matmul_args* args)
     return WOQ_OK;
 }
 
+static int run_matmul(const woq_matmul_args* args, void* stream);
+
 extern "C" int woq_matmul(const woq_matmul_args* args, void* stream)
+{
+    // a tuned tactic for this problem, unless the caller, the environment or a profiling run
+    // already fixed the choice, or the workspace given is too small for it
+    Tactic tuned;
+    if (args && args->regime == WOQ_REGIME_AUTO && !current_tactic() && env_regime() == WOQ_REGIME_AUTO
+        && find_tactic(*args, tuned))
+    {
+        TacticScope scope(&tuned);
+        if (woq_matmul_check(args) == WOQ_OK)
+        {
+            // an imported entry may name a launch shape this build does not have: nothing has been
+            // launched then, and the heuristics take over
+            int const rc = run_matmul(args, stream);
+            if (rc != WOQ_ERR_UNSUPPORTED)
+                return rc;
+        }
+    }
+    return run_matmul(args, stream);
+}
+
+static int run_matmul(const woq_matmul_args* args, void* stream)
 {
     if (int rc = woq_matmul_check(args))
         return rc;

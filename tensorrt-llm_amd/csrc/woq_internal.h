@@ -219,6 +219,32 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
     return pl;
 }
 
+// One way to run a 16-bit problem: the regime and, inside it, the streaming kernel's launch shape
+// (for problems of `mt` 16-row tiles) or the GEMM kernel, tile height and K split.  Counterpart of
+// the reference's CutlassGemmConfig with its enableCudaKernel pseudo-tactic
+// (cutlass_heuristic.cpp:393-441).
+struct Tactic
+{
+    int regime;               // WOQ_REGIME_STREAM or WOQ_REGIME_GEMM
+    int mt, ns, waves, pf, lds; // streaming launch shape
+    int skinny, rt, k_splits; // GEMM plan
+};
+
+// The tactic in force for the call running on this thread (set while profiling, or from the tuned
+// table by woq_matmul); nullptr: every choice is the heuristics'.
+Tactic const* current_tactic();
+struct TacticScope
+{
+    explicit TacticScope(Tactic const* t);
+    ~TacticScope();
+    Tactic const* prev;
+};
+// Tuned table (filled by woq_profile_tactics / woq_import_tactics): the entry of exactly m rows,
+// else of the smallest profiled row count above m.
+bool find_tactic(woq_matmul_args const& a, Tactic& out);
+// float32 split-K bytes the tuned entries of this n, k, quant_algo may use for at most m rows
+size_t tuned_split_bytes(int m, int n, int k, int quant_algo);
+
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;
 constexpr int kStreamW4a8MaxM = 16;

@@ -67,6 +67,59 @@ def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int,
     return out
 
 
+def profile_tactics(pre_quant_scale, weight, scales, zeros, bias, *, n: int, k: int, group_size: int,
+                    quant_algo: int, dtype: torch.dtype, min_m: int = 1, max_m: int = 4096, alpha: float = 1.0) -> int:
+    """Times this library's candidate kernels for the layer on the current stream and records the
+    fastest per row count (woq_profile_tactics; the reference does this in the plugins' initialize
+    through GemmPluginProfiler::profileTactics, gemmPluginProfiler.cpp:118-216).  Allocates the
+    activations, output and workspace of max_m rows itself, as the reference's profiler allocates its
+    temporary buffers (gemmPluginProfiler.cpp:252-270).  Returns the number of table entries."""
+    _require_gpu(pre_quant_scale, weight, scales, zeros, bias)
+    dev = weight.device
+    act = torch.randn((max_m, k), device=dev).to(dtype)
+    out = torch.empty((max_m, n), dtype=dtype, device=dev)
+    need = lib.woq_workspace_bytes(max_m, n, k, quant_algo, _WOQ_DT[dtype])
+    # room for every split-K candidate, not only the heuristics' own
+    need = max(need, max_m * k * 2 + 256 + min(max_m, 1024) * n * 4)
+    workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+    args = MatmulArgs(
+        act=_ptr(act), pre_quant_scale=_ptr(pre_quant_scale), weight=_ptr(weight), scales=_ptr(scales),
+        zeros=_ptr(zeros), bias=_ptr(bias), out=_ptr(out), alpha=float(alpha), m=max_m, n=n, k=k,
+        group_size=group_size, quant_algo=quant_algo, act_dtype=_WOQ_DT[dtype], out_dtype=_WOQ_DT[dtype],
+        regime=0, workspace=_ptr(workspace), workspace_bytes=workspace.numel())
+    check(lib.woq_profile_tactics(ctypes.byref(args), min_m, max_m, _stream_handle(dev)))
+    return lib.woq_tactic_count()
+
+
+def describe_tactic(m: int, n: int, k: int, group_size: int, quant_algo: int, dtype: torch.dtype) -> str:
+    """What a matmul call of this shape goes by: "heuristic" or the tuned table's entry."""
+    args = MatmulArgs(m=m, n=n, k=k, group_size=group_size, quant_algo=quant_algo, act_dtype=_WOQ_DT[dtype],
+                      out_dtype=_WOQ_DT[dtype], regime=0)
+    buf = ctypes.create_string_buffer(128)
+    check(lib.woq_describe_tactic(ctypes.byref(args), buf, len(buf)))
+    return buf.value.decode()
+
+
+def export_tactics() -> str:
+    """The tuned table as text (store it next to the model; import_tactics loads it again)."""
+    need = lib.woq_export_tactics(None, 0)
+    buf = ctypes.create_string_buffer(need)
+    lib.woq_export_tactics(buf, need)
+    return buf.value.decode()
+
+
+def import_tactics(text: str) -> None:
+    check(lib.woq_import_tactics(text.encode()))
+
+
+def clear_tactics() -> None:
+    lib.woq_clear_tactics()
+
+
+def tactic_count() -> int:
+    return lib.woq_tactic_count()
+
+
 def woq_grouped_matmul_raw(act, weight, scales, zeros, bias, total_rows_before_expert, *, n: int, k: int,
                            group_size: int, quant_algo: int, activation: str = "identity", residual=None,
                            regime: int = 0, out=None) -> torch.Tensor:
