@@ -342,10 +342,13 @@ SWEEPS = {
 }
 
 
-def run_sweep(pkg, dev, which):
+def run_sweep(pkg, dev, which, tuned=False):
     """The benchmark's other configurations: one JSON line per (kind, shape, M) with the launch time,
     algorithmic GB/s and TFLOP/s.  Launches rotate over weight copies exceeding the last-level cache
-    while M <= 256 (weight traffic matters there); all launches of a case replay from one HIP graph."""
+    while M <= 256 (weight traffic matters there); all launches of a case replay from one HIP graph.
+    With `tuned`, each layer is then profiled (woq_profile_tactics over the sweep's row counts) and
+    timed again, and the line also carries the tuned tactic and its time."""
+    F = pkg.functional
     shapes, kinds, ms = SWEEPS[which]
     for kind, group in kinds:
         for name, k, n in shapes:
@@ -355,28 +358,43 @@ def run_sweep(pkg, dev, which):
                 layers = rotated_copies(make_layer_int8(pkg, dev, k, n, 5000), copies)
             else:
                 layers = rotated_copies(make_layer(pkg, dev, k, n, 5000, group), copies)
-            for m in ms:
+
+            def time_case(m):
                 reps = 40 if m <= 256 else 5
                 if kind == "w4a8":
                     runner = w4a8_setup(pkg, dev, m, k, n, 5000, copies, layers)
                     body = lambda: [runner(r) for r in range(reps)]
                     runner(0)
-                    act_bytes = 1
                 else:
                     act = torch.randn((m, k), device=dev).to(torch.bfloat16)
                     out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
                     body = lambda: [launch(pkg, act, layers[r % copies], out) for r in range(reps)]
                     launch(pkg, act, layers[0], out)
-                    act_bytes = 2
                 torch.cuda.synchronize()
                 _, sec, launches = time_graph(body, reps, repeats=3)
-                us = sec / launches * 1e6
+                return sec / launches * 1e6
+
+            F.clear_tactics()
+            base = {m: time_case(m) for m in ms}
+            best, tactic = {}, {}
+            if tuned and kind != "w4a8":
+                lay = layers[0]
+                F.profile_tactics(None, lay["weight"], lay["scales"], lay["zeros"], None, n=n, k=k, group_size=group,
+                                  quant_algo=lay["algo"], dtype=torch.bfloat16, min_m=min(ms), max_m=max(ms))
+                for m in ms:
+                    tactic[m] = F.describe_tactic(m, n, k, group, lay["algo"], torch.bfloat16)
+                    best[m] = time_case(m)
+                F.clear_tactics()
+            for m in ms:
+                us = base[m]
                 n_sz = 1 if kind != "w4a16" else 2  # scales only, or scales + zeros
-                by = algorithmic_bytes(m, k, n, bits, group, n_sz, act_bytes)
-                print(json.dumps({"sweep": which, "kind": kind, "group": group, "shape": name, "k": k, "n": n, "m": m,
-                                  "us": round(us, 2), "gbs": round(by / us / 1e3, 1),
-                                  "tflops": round(2.0 * m * n * k / us / 1e6, 1), "weight_copies": copies}),
-                      flush=True)
+                by = algorithmic_bytes(m, k, n, bits, group, n_sz, 1 if kind == "w4a8" else 2)
+                line = {"sweep": which, "kind": kind, "group": group, "shape": name, "k": k, "n": n, "m": m,
+                        "us": round(us, 2), "gbs": round(by / us / 1e3, 1),
+                        "tflops": round(2.0 * m * n * k / us / 1e6, 1), "weight_copies": copies}
+                if m in best:
+                    line.update({"tuned_us": round(best[m], 2), "tuned": tactic[m]})
+                print(json.dumps(line), flush=True)
             layers = None
             torch.cuda.empty_cache()
 
@@ -436,6 +454,8 @@ def main():
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
+    ap.add_argument("--tuned", action="store_true",
+                    help="sweep: also profile each layer's tactics and time the tuned choices")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1): the op contains no communication, a "
@@ -450,7 +470,7 @@ def main():
         if args.sweep == "moe":
             run_moe_sweep(pkg, dev)
         else:
-            run_sweep(pkg, dev, args.sweep)
+            run_sweep(pkg, dev, args.sweep, args.tuned)
         return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode)

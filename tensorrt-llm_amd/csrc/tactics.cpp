@@ -42,6 +42,8 @@ bool same_problem(Key const& a, Key const& b)
 
 bool valid_tactic(Tactic const& t)
 {
+    if (t.regime == WOQ_REGIME_AUTO) // "as the heuristics choose": profiled, and nothing was clearly faster
+        return true;
     if (t.regime == WOQ_REGIME_STREAM)
         return t.ns >= 1 && t.waves >= 1 && t.pf >= 1 && t.lds >= 0 && t.lds <= 2
             && (t.mt == 1 || t.mt == 2 || t.mt == 4 || t.mt == 8);
@@ -59,6 +61,8 @@ void store(Key const& key, Tactic const& t)
 
 int describe(Tactic const& t, char* buf, size_t len)
 {
+    if (t.regime == WOQ_REGIME_AUTO)
+        return std::snprintf(buf, len, "heuristic");
     if (t.regime == WOQ_REGIME_STREAM)
         return std::snprintf(buf, len, "stream mt=%d ns=%d waves=%d pf=%d lds=%d", t.mt, t.ns, t.waves, t.pf, t.lds);
     return std::snprintf(buf, len, "gemm %s rt=%d splits=%d", t.skinny ? "skinny" : "exact", t.rt, t.k_splits);
@@ -99,11 +103,12 @@ std::vector<Tactic> candidates(woq_matmul_args const& a, bool stream_allowed)
         int const tk = tile_k_of_bits(bits);
         int const k_tiles = (a.k + tk - 1) / tk;
         auto add = [&](bool skinny, int rt) {
-            int const s = auto_k_splits(gemm_tiles(m, a.n, rt), k_tiles);
+            long const tiles = gemm_tiles(m, a.n, rt);
+            int s = 1;
+            (void) gemm_best_split(skinny, rt, tiles, m, a.n, a.k, bits, true, s);
             int const cap = k_tiles / 4 > 1 ? k_tiles / 4 : 1;
-            std::vector<int> splits{1, s, s / 2, s * 2};
-            if (s == 1 && gemm_tiles(m, a.n, rt) < 256)
-                splits.push_back(2), splits.push_back(4);
+            // around the cost model's split, and the largest that still runs as one round of workgroups
+            std::vector<int> splits{1, s - 1, s, s + 1, s * 3 / 4, (int) (256 / tiles), (int) (224 / tiles)};
             std::sort(splits.begin(), splits.end());
             splits.erase(std::unique(splits.begin(), splits.end()), splits.end());
             for (int v : splits)
@@ -213,39 +218,54 @@ extern "C" int woq_profile_tactics(const woq_matmul_args* args, int32_t min_m, i
     if (max_m > 15)
         rows.push_back(max_m);
 
-    constexpr int kWarmup = 1, kRuns = 3;
+    // Time of one candidate: the three fastest of five runs after a warm-up, each after an eviction
+    // of the last-level cache.  Negative: the candidate does not run on this problem.
+    constexpr int kWarmup = 1, kRuns = 5, kKept = 3;
+    auto time_tactic = [&](Tactic const& t) -> float {
+        TacticScope scope(&t);
+        if (woq_matmul_check(&a) != WOQ_OK)
+            return -1.f; // e.g. the workspace given does not cover this split
+        float ms[kRuns];
+        for (int r = 0; r < kWarmup + kRuns; ++r)
+        {
+            float v = 0.f;
+            bool const ok = hipMemsetAsync(flush, r, flush_bytes, s) == hipSuccess && hipEventRecord(t0, s) == hipSuccess
+                && woq_matmul(&a, stream) == WOQ_OK && hipEventRecord(t1, s) == hipSuccess
+                && hipEventSynchronize(t1) == hipSuccess && hipEventElapsedTime(&v, t0, t1) == hipSuccess;
+            if (!ok)
+            {
+                (void) hipGetLastError();
+                return -1.f;
+            }
+            if (r >= kWarmup)
+                ms[r - kWarmup] = v;
+        }
+        std::sort(ms, ms + kRuns);
+        float total = 0.f;
+        for (int r = 0; r < kKept; ++r)
+            total += ms[r];
+        return total;
+    };
+    // A candidate replaces the heuristics' own choice only when it is clearly faster: differences
+    // of a few percent are within what the same launch varies by from run to run.
+    constexpr float kClearlyFaster = 0.96f;
+    Tactic const heuristic{WOQ_REGIME_AUTO, 0, 0, 0, 0, 0, 0, 0, 0};
     bool gemm_won = false;
     int rc_out = WOQ_OK;
     for (int m : rows)
     {
         a.m = m;
-        Tactic best{};
-        float best_ms = -1.f;
+        float const heuristic_ms = time_tactic(heuristic);
+        Tactic best = heuristic;
+        float best_ms = heuristic_ms;
         for (Tactic const& t : candidates(a, !(gemm_won && m > 16)))
         {
-            TacticScope scope(&t);
-            if (woq_matmul_check(&a) != WOQ_OK)
-                continue; // e.g. the workspace given does not cover this split
-            float total = 0.f;
-            bool ok = true;
-            for (int r = 0; r < kWarmup + kRuns && ok; ++r)
-            {
-                ok = hipMemsetAsync(flush, r, flush_bytes, s) == hipSuccess && hipEventRecord(t0, s) == hipSuccess
-                    && woq_matmul(&a, stream) == WOQ_OK && hipEventRecord(t1, s) == hipSuccess
-                    && hipEventSynchronize(t1) == hipSuccess;
-                float ms = 0.f;
-                ok = ok && hipEventElapsedTime(&ms, t0, t1) == hipSuccess;
-                if (r >= kWarmup)
-                    total += ms;
-            }
-            if (!ok)
-            {
-                (void) hipGetLastError(); // a tactic that does not run is not a candidate
+            float const ms = time_tactic(t);
+            if (ms < 0.f)
                 continue;
-            }
-            if (best_ms < 0.f || total < best_ms)
+            if (best_ms < 0.f || (ms < best_ms && (heuristic_ms < 0.f || ms < kClearlyFaster * heuristic_ms)))
             {
-                best_ms = total;
+                best_ms = ms;
                 best = t;
             }
         }
@@ -254,7 +274,8 @@ extern "C" int woq_profile_tactics(const woq_matmul_args* args, int32_t min_m, i
             rc_out = fail(WOQ_ERR_RUNTIME, "no tactic ran for m = %d", m);
             break;
         }
-        if (best.regime == WOQ_REGIME_GEMM && m >= 16)
+        if (m >= 16 && (best.regime == WOQ_REGIME_GEMM
+                || (best.regime == WOQ_REGIME_AUTO && woq_select_regime(m, a.n, a.k, a.quant_algo) == WOQ_REGIME_GEMM)))
             gemm_won = true;
         store(key_of(a, m), best);
     }

@@ -98,32 +98,57 @@ inline int auto_k_splits(long tiles, int k_tiles)
     return splits > 1 ? (int) splits : 1;
 }
 
-// Estimated time (microseconds) of a 16-bit GEMM-regime problem on one kernel and tile height, from
-// a model fitted to sweeps over the Llama-3-8B / 70B layer shapes (M = 32 .. 1024, int4 g64 / g128
-// and int8 per-channel; picking by it stays within 1 % of the best measured choice on average):
-//   * a workgroup spends c microseconds per tile row of K: c = a + b * rows for the exact-dequantize
-//     kernel (the dequantize is paid once per workgroup, the MFMAs per row), a constant for the
-//     deferred-scale kernel's 64-row (or 32-row) tile;
-//   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another;
-//   * splitting K costs two more launches and the float32 partial traffic.
+// Estimated time (microseconds) of a 16-bit GEMM-regime problem on one kernel, tile height and K
+// split, from a model fitted to sweeps over the Llama-3-8B / 70B layer shapes (M = 32 .. 1024, int4
+// g128 and int8 per-channel, every kernel / tile height / split count from 1 to 20: picking by it
+// stays within 1 % of the best measured choice on average, 10 % at worst):
+//   * a workgroup spends c microseconds per tile row of K (c = a + b * rt for the exact-dequantize
+//     kernel: the dequantize is paid once per workgroup, the MFMAs per row; a constant for the
+//     deferred-scale kernel's 64- or 32-row tile) plus a prologue / epilogue of ~2 us per tile;
+//   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another, and a last
+//     round of more than 224 workgroups runs ~10 % longer (measured: 256 workgroups are no faster
+//     than 192, and 257 take two rounds);
+//   * splitting K costs the reduction launch and the float32 partial traffic.
 // `tiles` is the output tile count of that tile height (for a grouped problem: over all experts).
-inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, bool allow_split, int& splits)
+inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, int splits)
 {
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
-    double const per_k = bits == 4 ? 1.0 : 0.5; // a tile row of int8 covers half the K of an int4 one
     double c;
     if (skinny)
-        c = (bits == 4 ? 1.5 : 1.2) * per_k * (rt == 2 ? 0.72 : 1.0);
+        c = bits == 4 ? (rt == 2 ? 0.878 : 1.344) : 0.596;
     else
-        c = (0.8 + 0.007 * 16 * rt) * per_k;
-    splits = allow_split ? auto_k_splits(tiles, k_tiles) : 1;
-    long const rounds = (tiles * splits + 255) / 256;
+        c = bits == 4 ? 0.803 + 0.105 * rt : 0.640 + 0.0387 * rt;
+    long const wgs = tiles * splits;
+    long const rounds = (wgs + 255) / 256;
     int const steps = (k_tiles + splits - 1) / splits;
-    double t = (double) rounds * steps * c + 4.0;
+    double const last_round = wgs - (rounds - 1) * 256 > 224 ? 0.10 : 0.0;
+    double t = ((double) rounds + last_round) * (steps * c + 1.98 + 0.02 * rt) + 1.6;
     if (splits > 1)
-        t += 5.0 + (double) m * n * 4.0 * (2 + 2 * splits) / (bits == 4 ? 1.5e6 : 2.5e6);
+        t += 2.5 + (double) m * n * 4.0 * (2 + 2 * splits) * 3.5e-7;
     return t;
+}
+
+// The K split (1 = none) that gemm_cost_us estimates cheapest for this kernel and tile height, and
+// its cost.  A split leaves every workgroup at least four tile rows of K.
+inline double gemm_best_split(bool skinny, int rt, long tiles, int m, int n, int k, int bits, bool allow_split, int& splits)
+{
+    int const tk = tile_k_of_bits(bits);
+    int const k_tiles = (k + tk - 1) / tk;
+    splits = 1;
+    double best = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, 1);
+    if (!allow_split || k_tiles < 8)
+        return best;
+    for (int s = 2; s <= k_tiles / 4 && tiles * s <= 512; ++s)
+    {
+        double const t = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, s);
+        if (t < best)
+        {
+            best = t;
+            splits = s;
+        }
+    }
+    return best;
 }
 
 // Kernel, tile height and K split of a 16-bit GEMM-regime problem: the cheapest by gemm_cost_us of
@@ -156,8 +181,8 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
         if (!skinny && forced_rt && rt != forced_rt)
             continue;
         int splits;
-        double const cost
-            = gemm_cost_us(skinny, rt, (long) num_experts * gemm_tiles(rows, n, rt), m, n, k, bits, allow_split, splits);
+        double const cost = gemm_best_split(
+            skinny, rt, (long) num_experts * gemm_tiles(rows, n, rt), m, n, k, bits, allow_split, splits);
         if (!have || cost < best)
         {
             have = true;

@@ -19,6 +19,23 @@ PLUGIN_NAMESPACE = "tensorrt_llm"
 PLUGIN_VERSION = "1"
 
 
+def _profile_layer(n: int, k: int, group_size: int, quant_algo: int, dtype: torch.dtype, min_m: int, max_m: int,
+                   alpha: float, device) -> int:
+    """Tactic profiling of one layer shape on stand-in operands, as the reference's profiler does on
+    its own temporary buffers (gemmPluginProfiler.cpp:252-270, called from the plugins' initialize
+    through configGemm, weightOnlyQuantMatmulPlugin.cpp:255-275): kernel times do not depend on the
+    values, so random packed weights and unit scales stand in for the layer's."""
+    nbytes = int(lib.woq_preprocessed_bytes(k, n, _lib.W8_A16 if quant_algo & F.INT8_WEIGHT else _lib.W4_A16))
+    weight = torch.randint(0, 256, (nbytes,), dtype=torch.uint8, device=device)
+    groups = (k // group_size, n) if group_size else (n,)
+    scales = torch.full(groups, 0.01, dtype=dtype, device=device)
+    zeros = torch.zeros(groups, dtype=dtype, device=device) if quant_algo & F.ZERO else None
+    bias = torch.zeros((n,), dtype=dtype, device=device) if quant_algo & F.BIAS else None
+    pqs = torch.ones((k,), dtype=dtype, device=device) if quant_algo & F.PRE_QUANT_SCALE else None
+    return F.profile_tactics(pqs, weight, scales, zeros, bias, n=n, k=k, group_size=group_size,
+                             quant_algo=quant_algo, dtype=dtype, min_m=min_m, max_m=max_m, alpha=alpha)
+
+
 class WeightOnlyQuantMatmulPlugin:
     name = "WeightOnlyQuantMatmul"
 
@@ -31,7 +48,17 @@ class WeightOnlyQuantMatmulPlugin:
         self.weight_type_id = weight_type_id
 
     def get_workspace_size(self, max_m: int, n: int, k: int) -> int:
-        return 0
+        dt = _lib.BF16 if self.type_id == torch.bfloat16 else _lib.FP16
+        algo = F.INT8_WEIGHT if self.weight_type_id == F.INT8 else 0
+        return int(lib.woq_workspace_bytes(max_m, n, k, algo, dt))
+
+    def initialize(self, min_m: int, max_m: int, n: int, k: int, device="cuda") -> int:
+        """configurePlugin's dimensions + initialize's profiling in one call
+        (weightOnlyQuantMatmulPlugin.cpp:233-275).  Returns the number of tuned entries; the table
+        travels as text (functional.export_tactics / import_tactics), the counterpart of the tactic
+        map the reference serialises with the plugin (:374-391)."""
+        algo = F.INT8_WEIGHT if self.weight_type_id == F.INT8 else 0
+        return _profile_layer(n, k, 0, algo, self.type_id, min_m, max_m, 1.0, device)
 
     def enqueue(self, inputs, outputs, workspace=None) -> int:
         """inputs: [act [.., K], weight [K, N or N/2], scales [N]]; outputs: [out [.., N]]."""
@@ -55,6 +82,12 @@ class WeightOnlyGroupwiseQuantMatmulPlugin:
     def get_workspace_size(self, max_m: int, n: int, k: int) -> int:
         dt = _lib.BF16 if self.type_id == torch.bfloat16 else _lib.FP16
         return int(lib.woq_workspace_bytes(max_m, n, k, self.quant_algo, dt))
+
+    def initialize(self, min_m: int, max_m: int, n: int, k: int, device="cuda") -> int:
+        """Profiles the layer shape for row counts min_m..max_m
+        (weightOnlyGroupwiseQuantMatmulPlugin.cpp: configurePlugin + initialize → configGemm →
+        profileTactics).  Returns the number of tuned entries."""
+        return _profile_layer(n, k, self.group_size, self.quant_algo, self.type_id, min_m, max_m, self.alpha, device)
 
     def enqueue(self, inputs, outputs, workspace=None) -> int:
         """inputs in plugin order: act, [pre_quant_scale], weight, scales, [zeros], [bias]."""

@@ -1,4 +1,5 @@
-"""Tactic profiler on the GPU: after profiling a layer the tuned choices are in force for regime
+"""Tactic profiler on the GPU: after profiling a layer the tuned choices (a kernel and launch shape,
+or "heuristic" where nothing was clearly faster than the built-in choice) are in force for regime
 AUTO and the results still match the oracle (same tolerance as the kernels' own parity tests);
 an imported entry this build has no kernel for falls back to the heuristics."""
 import pytest
@@ -32,7 +33,7 @@ def test_profile_then_matmul(pkg, oracle, dev, bits, group, dtype):
     assert n == 15 + 4 + 1
     text = F.export_tactics()
     for m in (1, 5, 16, 40, 100, max_m):
-        assert F.describe_tactic(m, N, K, group, algo, tdt) != "heuristic"
+        assert F.describe_tactic(m, N, K, group, algo, tdt).split()[0] in ("heuristic", "stream", "gemm")
         q = dict(p, act=p["act"][:m], M=m)
         err = oracle.max_rel_err(run_product(pkg, oracle, dev, q, 0, w_dev=w), reference(oracle, q))
         assert err < TOL, (m, F.describe_tactic(m, N, K, group, algo, tdt), err)
@@ -53,3 +54,20 @@ def test_unknown_shape_falls_back(pkg, oracle, dev):
     assert F.describe_tactic(m, N, K, 128, F.ZERO, torch.bfloat16).startswith("stream")
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
     assert err < TOL, err
+
+
+def test_plugin_initialize_profiles_the_layer(pkg, oracle, dev):
+    """The plugin mirrors' initialize (configurePlugin dimensions + profiling on stand-in buffers):
+    afterwards the real layer's calls go by the tuned table and match the oracle."""
+    F, P = pkg.functional, pkg.plugin
+    K, N, max_m = 512, 1024, 48
+    plug = P.WeightOnlyGroupwiseQuantMatmulPlugin(torch.bfloat16, F.ZERO, 64)
+    assert plug.initialize(1, max_m, N, K, device=dev) == 15 + 2 + 1
+    assert "woq-tactics 1" in F.export_tactics()
+    for m in (2, 20, max_m):
+        p = random_problem(oracle, m, K, N, 4, 64, "bf16", zero=True, seed=m)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+        assert err < TOL, (m, err)
+    per_channel = P.WeightOnlyQuantMatmulPlugin(torch.float16, F.INT8)
+    assert per_channel.initialize(4, 4, N, K, device=dev) == 18 + 1
+    assert per_channel.get_workspace_size(4, N, K) >= 0
