@@ -115,8 +115,11 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         // staging pass and the resident workgroups it costs outweigh the shared reads), and with
         // few column groups and at most 3 rows, where one workgroup per CU covers the whole problem
         // anyway (the down projections: long K, N <= 4096)
-        StreamShape const sh = strips >= 1024 ? StreamShape{4, 8, 2, 1}
-                                              : (strips >= 384 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
+        // strips per workgroup: one up to 256 column strips, two up to 512, else four, so that no launch
+        // has between 256 and 512 workgroups (a partly filled second round over the 256 CUs measured
+        // 10-70 % slower than half as many workgroups of twice the width)
+        StreamShape const sh = strips > 512 ? StreamShape{4, 8, 2, 1}
+                                            : (strips > 256 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
         if (act_lds <= (size_t) (rows == 1 ? 48 : 20) * 1024)
         {
             if (act_lds + (size_t) k * (sh.ns + 1) <= stream_max_staged_lds(sh.ns, sh.waves))
@@ -128,16 +131,16 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
             return {1, 8, 4, 1};
         // activations stay in registers; the group scales / zeros (at most k * ns bytes) are still
         // staged while that leaves room for the resident workgroups the shape counts on
-        StreamShape reg = strips >= 1024 ? StreamShape{4, 4, 2, 0}
-                                         : (strips >= 384 ? StreamShape{2, 8, 2, 0} : StreamShape{1, 8, 4, 0});
+        StreamShape reg = strips > 512 ? StreamShape{4, 4, 2, 0}
+                                       : (strips > 256 ? StreamShape{2, 8, 2, 0} : StreamShape{1, 8, 4, 0});
         if ((size_t) k * reg.ns <= (size_t) (reg.waves == 4 ? 32 : 64) * 1024)
             reg.lds = 2;
         return reg;
     }
     if (mt == 2)
-        return {strips >= 1024 ? 2 : 1, 8, 2, 0};
+        return {stream_mid_ns(strips), 8, 2, 0};
     if (mt == 4)
-        return {strips >= 1024 ? 2 : 1, 8, 1, 0};
+        return {stream_mid_ns(strips), 8, 1, 0};
     return {1, 8, 1, 0};
 }
 
@@ -264,18 +267,17 @@ extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_
     // memory speed for one 16-row tile; beyond that the fp8 GEMM kernel
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
         return m <= kStreamW4a8MaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
-    // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed; with two row
-    // tiles the streaming kernel still wins on small matrices (it needs no split-K passes): up to
-    // 2^24 int4 weights and up to 2^26 int8 weights (up to 64 rows on int8 matrices of 2^24).
-    // Beyond that the MFMA GEMM kernels are faster.
+    // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed.  With 17..64 rows
+    // the streaming kernel (no split-K passes) still wins on small matrices with short K: whichever
+    // the two fitted cost models estimate cheaper.  Beyond that the MFMA GEMM kernels are faster.
     if (m <= 16)
         return WOQ_REGIME_STREAM;
-    int64_t const weights = (int64_t) n * k;
-    bool const int8 = quant_algo & WOQ_ALGO_INT8_WEIGHT;
-    if (m <= 32 && weights <= ((int64_t) 1 << (int8 ? 26 : 24)))
-        return WOQ_REGIME_STREAM;
-    if (m <= 64 && int8 && weights <= ((int64_t) 1 << 24))
-        return WOQ_REGIME_STREAM;
+    if (m <= 64)
+    {
+        int const bits = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
+        if (stream_cost_us(m, n, k) < plan_gemm(m, n, k, bits).cost_us)
+            return WOQ_REGIME_STREAM;
+    }
     return WOQ_REGIME_GEMM;
 }
 

@@ -77,6 +77,7 @@ struct GemmPlan
     int rt;       // row tiles per wavefront (tile rows = 16 * rt)
     int k_splits;
     size_t ws_bytes;
+    double cost_us; // the cost model's estimate (plan_gemm only)
 };
 
 // Output tiles (of 16*rt rows x 256 columns) a problem has.
@@ -105,9 +106,9 @@ inline int auto_k_splits(long tiles, int k_tiles)
 //   * a workgroup spends c microseconds per tile row of K (c = a + b * rt for the exact-dequantize
 //     kernel: the dequantize is paid once per workgroup, the MFMAs per row; a constant for the
 //     deferred-scale kernel's 64- or 32-row tile) plus a prologue / epilogue of ~2 us per tile;
-//   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another, and a last
-//     round of more than 224 workgroups runs ~10 % longer (measured: 256 workgroups are no faster
-//     than 192, and 257 take two rounds);
+//   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another (counted on the
+//     fullest XCD), and a last round of more than 224 workgroups runs ~10 % longer (measured: 256
+//     workgroups are no faster than 192, and 257 take two rounds);
 //   * splitting K costs the reduction launch and the float32 partial traffic.
 // `tiles` is the output tile count of that tile height (for a grouped problem: over all experts).
 inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, int splits)
@@ -119,10 +120,12 @@ inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k,
         c = bits == 4 ? (rt == 2 ? 0.878 : 1.344) : 0.596;
     else
         c = bits == 4 ? 0.803 + 0.105 * rt : 0.640 + 0.0387 * rt;
-    long const wgs = tiles * splits;
-    long const rounds = (wgs + 255) / 256;
+    // the tiles are dealt to the 8 XCDs (32 CUs each) in equal contiguous runs: the fullest XCD
+    // sets the number of rounds
+    long const wgs = (tiles + 7) / 8 * splits;
+    long const rounds = (wgs + 31) / 32;
     int const steps = (k_tiles + splits - 1) / splits;
-    double const last_round = wgs - (rounds - 1) * 256 > 224 ? 0.10 : 0.0;
+    double const last_round = wgs - (rounds - 1) * 32 > 28 ? 0.10 : 0.0;
     double t = ((double) rounds + last_round) * (steps * c + 1.98 + 0.02 * rt) + 1.6;
     if (splits > 1)
         t += 2.5 + (double) m * n * 4.0 * (2 + 2 * splits) * 3.5e-7;
@@ -201,7 +204,30 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
             pl.k_splits = v;
     }
     pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+    pl.cost_us = best;
     return pl;
+}
+
+// Strips (16 output columns) per workgroup of the streaming kernel for 17..64 rows: one up to 256
+// column strips, else two (257..511 workgroups, a partly filled second round over the 256 CUs,
+// measured 40-60 % slower than half as many workgroups of twice the width).
+inline int stream_mid_ns(int strips)
+{
+    return strips > 256 ? 2 : 1;
+}
+
+// Estimated time (microseconds) of the streaming kernel on 17..64 rows, fitted to the Llama-3-8B / 70B
+// layer shapes and N = 2048 / 5120 (int4 and int8 read at the same rate here): every workgroup walks
+// all of K, at a rate that falls with the rows it carries, in ceil(workgroups / 256) rounds.
+inline double stream_cost_us(int m, int n, int k)
+{
+    int const strips = (n + 15) / 16;
+    int const ns = stream_mid_ns(strips);
+    long const groups = (strips + ns - 1) / ns;
+    long const rounds = (groups + 255) / 256;
+    int const rows = m > 32 ? m + 6 : m; // the step from two to four row tiles per wavefront
+    double const per_1024 = ns == 1 ? 0.7 + 0.045 * rows : 0.6 + 0.06 * rows;
+    return 3.0 + (double) rounds * k / 1024.0 * per_1024;
 }
 
 // W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K).
@@ -223,7 +249,7 @@ inline int w4a8_rt(int m, int n, int k)
 
 inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
 {
-    GemmPlan pl;
+    GemmPlan pl{};
     pl.skinny = false;
     pl.rt = w4a8_rt(m, n, k);
     if (char const* r = std::getenv("WOQ_GEMM_RT"))

@@ -109,18 +109,21 @@ def test_regime_table(pkg):
     sel = L.lib.woq_select_regime
     for m in (1, 2, 4, 15, 16, 17, 32):
         assert sel(m, 4096, 4096, 0) == L.REGIME_STREAM
-    for m in (33, 64, 128, 129, 256, 4096, 8192):
+    for m in (65, 128, 129, 256, 4096, 8192):
         assert sel(m, 4096, 4096, 0) == L.REGIME_GEMM
-    # two row tiles: streaming on small matrices only
-    assert sel(32, 28672, 4096, 0) == L.REGIME_GEMM
-    assert sel(16, 28672, 4096, 0) == L.REGIME_STREAM
-    assert sel(32, 6144, 4096, 0) == L.REGIME_GEMM  # int4: 32-row MFMA tiles win above 2^24 weights
-    assert sel(32, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM
-    assert sel(32, 8192, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM  # 2^26 int8 weights: still streaming
-    assert sel(32, 10240, 8192, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
-    assert sel(64, 4096, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_STREAM  # small int8 matrices stream up to 64 rows
-    assert sel(65, 4096, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
-    assert sel(64, 6144, 4096, L.ALGO_INT8_WEIGHT) == L.REGIME_GEMM
+    # 17..64 rows: streaming where its cost estimate beats the GEMM plan's (small N, short K)
+    for algo in (0, L.ALGO_INT8_WEIGHT):
+        assert sel(16, 28672, 4096, algo) == L.REGIME_STREAM
+        assert sel(32, 28672, 4096, algo) == L.REGIME_GEMM
+        assert sel(32, 6144, 4096, algo) == L.REGIME_STREAM   # 384 strips, two per workgroup: one round of 192
+        assert sel(20, 8192, 8192, algo) == L.REGIME_STREAM
+        assert sel(20, 10240, 8192, algo) == L.REGIME_GEMM    # 320 workgroups: two rounds
+        assert sel(20, 4096, 14336, algo) == L.REGIME_GEMM    # long K: split-K GEMM
+        assert sel(48, 8192, 8192, algo) == L.REGIME_GEMM
+        # the choice never goes back to streaming as the rows grow
+        for n, k in ((4096, 4096), (6144, 4096), (8192, 8192), (2048, 4096), (5120, 8192)):
+            picks = [sel(m, n, k, algo) for m in range(17, 130)]
+            assert picks == sorted(picks, key=lambda r: r != L.REGIME_STREAM), (n, k, algo)
     # W4A8: streaming kernel for one 16-row tile, the fp8 GEMM above
     assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
     assert sel(16, 57344, 8192, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
