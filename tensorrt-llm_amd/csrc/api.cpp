@@ -90,7 +90,7 @@ struct StreamShape
     int ns, waves, pf, lds;
 };
 
-StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k)
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group)
 {
     if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
     {
@@ -118,8 +118,17 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         // strips per workgroup: one up to 256 column strips, two up to 512, else four, so that no launch
         // has between 256 and 512 workgroups (a partly filled second round over the 256 CUs measured
         // 10-70 % slower than half as many workgroups of twice the width)
-        StreamShape const sh = strips > 512 ? StreamShape{4, 8, 2, 1}
-                                            : (strips > 256 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
+        StreamShape sh = strips > 512 ? StreamShape{4, 8, 2, 1}
+                                      : (strips > 256 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
+        // LDS of one workgroup of the staged variants: activations, group scales + zeros and row sums
+        // (at most k * ns + k bytes, group 64 with zeros), the epilogue's reduction buffer
+        size_t const scale_unit = group == 0 ? 0 : (size_t) k * 64 / group;
+        auto footprint = [&](StreamShape const& v) {
+            return act_lds + scale_unit * (v.ns + 1) + (size_t) v.waves * v.ns * 1024;
+        };
+        // a launch of more workgroups than CUs wants two of them resident per CU
+        if (sh.ns == 4 && strips > 4 * 256 && 2 * footprint(sh) > (size_t) 160 * 1024)
+            sh = StreamShape{2, 8, 4, 1};
         if (act_lds <= (size_t) (rows == 1 ? 48 : 20) * 1024)
         {
             if (act_lds + (size_t) k * (sh.ns + 1) <= stream_max_staged_lds(sh.ns, sh.waves))
@@ -129,6 +138,12 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         }
         else if (strips <= 256 && rows <= 3 && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
             return {1, 8, 4, 1};
+        // 513..1024 strips run as at most 256 workgroups of four strips: with one workgroup per CU the
+        // eight wavefronts of the staged variant keep more loads in flight than the four of the
+        // register variant, for up to four rows
+        else if (strips > 512 && strips <= 1024 && rows <= 4
+            && act_lds + (size_t) k * 5 <= stream_max_staged_lds(4, 8))
+            return {4, 8, 2, 1};
         // activations stay in registers; the group scales / zeros (at most k * ns bytes) are still
         // staged while that leaves room for the resident workgroups the shape counts on
         StreamShape reg = strips > 512 ? StreamShape{4, 4, 2, 0}

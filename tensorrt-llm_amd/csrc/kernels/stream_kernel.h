@@ -650,7 +650,7 @@ inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool 
 
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
-StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k);
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group);
 
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
     bool GROUPED = false>
@@ -700,7 +700,7 @@ template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK);
+    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK, GROUP);
     if (GROUP == 0 && sh.lds == 2)
         sh.lds = 0; // per-channel scales are applied once, in the epilogue: nothing to stage
 #define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
@@ -745,7 +745,7 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
     // every expert's column groups run side by side: the grid is num_experts times taller
-    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK);
+    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK, GROUP);
     if (act_is_gated(sp.activation) && sh.ns == 1) // value and gate strips pair up inside a wavefront
         sh = sh.lds == 1 ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, sh.lds};
     if (GROUP == 0 && sh.lds == 2)
