@@ -334,14 +334,14 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     // the split-K region does not (large m does not split), so take its maximum over the row
     // counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
-    // kEnoughTiles or more tiles never split, which even one column of the tallest (256-row) tiles
-    // reaches at 256 * kEnoughTiles rows; below that the plan may change at any row count
+    // A plan splits K only while tiles * splits <= 512, which even the tallest (256-row) tiles exceed
+    // beyond 256 * (256 / column tiles) rows; below that the plan may change at any row count.  The
+    // partial buffer grows with the rows, so the largest row count that splits sets the maximum.
     size_t split = split_bytes(m, n, k, quant_algo);
-    for (int mm = 1; mm < m && mm <= 256 * (int) kEnoughTiles; ++mm)
-    {
-        size_t const b = split_bytes(mm, n, k, quant_algo);
-        split = b > split ? b : split;
-    }
+    int const col_tiles = (n + 255) / 256;
+    int const cap = 256 * (col_tiles >= 256 ? 1 : 256 / col_tiles);
+    for (int mm = m - 1 < cap ? m - 1 : cap; mm >= 1 && split == 0; --mm)
+        split = split_bytes(mm, n, k, quant_algo);
     size_t const tuned = tuned_split_bytes(m, n, k, quant_algo);
     bytes += split > tuned ? split : tuned;
     return bytes;

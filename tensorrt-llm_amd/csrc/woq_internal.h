@@ -86,19 +86,6 @@ inline long gemm_tiles(int m, int n, int rt)
     return (long) ((m + rt * 16 - 1) / (rt * 16)) * ((n + 255) / 256);
 }
 
-// A launch fills the 256 CUs from about this many workgroups on; below it K is split.
-constexpr long kEnoughTiles = 160;
-
-inline int auto_k_splits(long tiles, int k_tiles)
-{
-    if (tiles >= kEnoughTiles || k_tiles < 8)
-        return 1;
-    long splits = 2 * kEnoughTiles / tiles;
-    if (splits > k_tiles / 4)
-        splits = k_tiles / 4;
-    return splits > 1 ? (int) splits : 1;
-}
-
 // Estimated time (microseconds) of a 16-bit GEMM-regime problem on one kernel, tile height and K
 // split, from a model fitted to sweeps over the Llama-3-8B / 70B layer shapes (M = 32 .. 1024, int4
 // g128 and int8 per-channel, every kernel / tile height / split count from 1 to 20: picking by it
@@ -231,40 +218,58 @@ inline double stream_cost_us(int m, int n, int k)
 }
 
 // W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K).
-// Tile height above 128 rows, from measured crossovers (per-CU rates 1 : 0.65 : 0.37 for
-// 256 : 128 : 64 rows): 256 rows when those tiles fill the chip or K is very long (splitting K is
-// then cheap); else 128 rows when they fill it, or nearly do and K is long; else 64 rows.
-inline int w4a8_rt(int m, int n, int k)
+// Estimated time (microseconds) of one tile height and K split: the same model as gemm_cost_us,
+// fitted to a sweep of the fp8 kernel over the Llama-3-8B / 70B shapes (M = 32 .. 4096, every tile
+// height, splits 1 .. 20): picking by it stays within 0.6 % of the best measured choice on average.
+inline double w4a8_cost_us(int rt, long tiles, int m, int n, int k, int splits)
 {
-    if (m <= 64)
-        return 4;
-    if (m <= 128)
-        return 8;
-    if (gemm_tiles(m, n, 16) >= kEnoughTiles || k >= 16384)
-        return 16;
-    if (gemm_tiles(m, n, 8) >= kEnoughTiles || (gemm_tiles(m, n, 8) >= 96 && k >= 8192))
-        return 8;
-    return 4;
+    int const k_tiles = (k + 127) / 128;
+    long const wgs = (tiles + 7) / 8 * splits; // on the fullest XCD
+    long const rounds = (wgs + 31) / 32;
+    int const steps = (k_tiles + splits - 1) / splits;
+    double const last_round = wgs - (rounds - 1) * 32 > 28 ? 0.07 : 0.0;
+    double t = ((double) rounds + last_round) * (steps * (1.18 + 0.0405 * rt) + 1.42) + 4.1;
+    if (splits > 1)
+        t += 1.7 + (double) m * n * 4.0 * (2 + 2 * splits) * 3.44e-7;
+    return t;
 }
 
 inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
 {
     GemmPlan pl{};
     pl.skinny = false;
-    pl.rt = w4a8_rt(m, n, k);
+    int const k_tiles = (k + 127) / 128;
+    int forced_rt = 0, forced_splits = 0;
     if (char const* r = std::getenv("WOQ_GEMM_RT"))
     {
         int const v = std::atoi(r);
         if (v == 4 || v == 8 || v == 16)
-            pl.rt = v;
+            forced_rt = v;
     }
-    int const k_tiles = (k + 127) / 128;
-    pl.k_splits = auto_k_splits(gemm_tiles(m, n, pl.rt), k_tiles);
     if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
     {
         int const v = std::atoi(f);
         if (v >= 1 && v <= k_tiles)
-            pl.k_splits = v;
+            forced_splits = v;
+    }
+    bool have = false;
+    for (int rt = 4; rt <= 16; rt *= 2)
+    {
+        if (forced_rt ? rt != forced_rt : ((rt == 8 && m <= 64) || (rt == 16 && m <= 128)))
+            continue;
+        long const tiles = gemm_tiles(m, n, rt);
+        int const max_s = forced_splits ? forced_splits : (k_tiles >= 8 ? k_tiles / 4 : 1);
+        for (int s = forced_splits ? forced_splits : 1; s <= max_s && (s == 1 || forced_splits || tiles * s <= 512); ++s)
+        {
+            double const t = w4a8_cost_us(rt, tiles, m, n, k, s);
+            if (!have || t < pl.cost_us)
+            {
+                have = true;
+                pl.cost_us = t;
+                pl.rt = rt;
+                pl.k_splits = s;
+            }
+        }
     }
     pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
     return pl;
