@@ -196,20 +196,23 @@ int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* stream);
 /* Validation only (no launch): what woq_grouped_matmul would return for these arguments. */
 int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);
 
-/* The regime AUTO picks: STREAM for m <= 16 (m <= 32 when n*k <= 2^24 for int4, <= 2^26 for int8
- * weights, m <= 64 for int8 when n*k <= 2^24; m <= 16 for W4A8), GEMM otherwise - crossovers measured on MI355X.  Counterpart of the tactic choice
+/* The regime the built-in rule picks for AUTO: STREAM for m <= 16; for 17 <= m <= 64 (16-bit
+ * activations) STREAM where the streaming kernel's estimated time is below the GEMM plan's (small n
+ * with short k, e.g. 4096 x 4096 up to 64 rows, 8192 x 8192 up to ~20), GEMM otherwise; m <= 16 for
+ * W4A8 - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 
 /* ---- tactic profiler ------------------------------------------------------------------------ */
 
-/* Times, on `stream`, every candidate way this library has of running the 16-bit problem `args`
- * describes (streaming launch shapes; deferred-scale / exact-dequantize GEMM kernels, tile heights
- * and K splits) for every m in [min_m, 15], the powers of two from 16 below max_m, and max_m, and
- * records the fastest per row count in a process-wide table.  Later woq_matmul calls with
- * regime AUTO on the same (n, k, quant_algo, group_size, out_dtype) use the entry of their m, else
- * of the next profiled row count above it, else the built-in heuristics (also when the workspace
- * they are given is too small for the tuned choice).  Replaces
+/* Times, on `stream`, the built-in choice and every candidate way this library has of running the
+ * 16-bit problem `args` describes (streaming launch shapes; deferred-scale / exact-dequantize GEMM
+ * kernels, tile heights and K splits) for every m in [min_m, 15], the powers of two from 16 below
+ * max_m, and max_m, and records per row count the fastest candidate if it beats the built-in choice
+ * by more than 4 % (else "heuristic") in a process-wide table.  Later woq_matmul calls with regime
+ * AUTO on the same (n, k, quant_algo, group_size, out_dtype) use the entry of their m, else of the
+ * next profiled row count above it, else the built-in heuristics (also when the workspace they are
+ * given is too small for the tuned choice, or the entry names a kernel this build lacks).  Replaces
  * GemmPluginProfiler::profileTactics (plugins/common/gemmPluginProfiler.cpp:118-216, timing loop
  * :329-367, lookup :221-250) as called from the plugins' configGemm / initialize
  * (weightOnlyQuantMatmulPlugin.cpp:255-275).  A set-up call: the buffers of `args` must hold
@@ -224,7 +227,8 @@ int woq_tactic_count(void);
 void woq_clear_tactics(void);
 
 /* Writes what a woq_matmul call with these arguments would go by: "heuristic", or the tuned entry
- * ("stream mt=.. ns=.. waves=.. pf=.. lds=..", "gemm exact|skinny rt=.. splits=.."). */
+ * ("stream mt=.. ns=.. waves=.. pf=.. lds=..", "gemm exact|skinny rt=.. splits=.."; "heuristic"
+ * also for an entry that recorded the built-in choice as the fastest). */
 int woq_describe_tactic(const woq_matmul_args* args, char* buf, size_t len);
 
 /* The table as text (one line per entry), so that it can be stored next to a model and loaded
