@@ -139,7 +139,8 @@ int woq_matmul_check(const woq_matmul_args* args);
 /* Device scratch that is enough for every woq_matmul call of this n, k, quant_algo with AT MOST m
  * rows (pass the largest m, as the reference passes its profile's maxM): a region for smoothed
  * activations (PRE_QUANT_SCALE, GEMM regime) followed by the float32 partial sums of the
- * split-K GEMM that skinny problems use (the reference's split-K workspace).  Replaces
+ * split-K GEMM that skinny problems use (one [m, n] slab per slice of K, summed in slice order, so
+ * results are bit-reproducible from run to run; the reference's split-K workspace).  Replaces
  * CutlassFpAIntBGemmRunner::getWorkspaceSize (fpA_intB_gemm_template.h:549-582) plus the
  * plugin's own m*k*sizeof(half) smoothing buffer (weightOnlyGroupwiseQuantMatmulPlugin.cpp:377-379). */
 size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype);

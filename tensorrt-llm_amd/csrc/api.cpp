@@ -43,7 +43,7 @@ GemmPlan planned_gemm(int m, int n, int k, int bits)
         pl.rt = t->rt;
         int const k_tiles = (k + tile_k_of_bits(bits) - 1) / tile_k_of_bits(bits);
         pl.k_splits = t->k_splits < 1 ? 1 : (t->k_splits > k_tiles ? k_tiles : t->k_splits);
-        pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+        pl.ws_bytes = split_partial_bytes(m, n, pl.k_splits);
         return pl;
     }
     return plan_gemm(m, n, k, bits);
@@ -331,17 +331,24 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
         return 0;
     // Enough for every call with at most m rows (the reference sizes its workspace for the
     // profile's largest M the same way), in either regime.  The smoothing region grows with m;
-    // the split-K region does not (large m does not split), so take its maximum over the row
-    // counts up to m.
+    // the split-K region does not (large m does not split, small m splits most), so take its
+    // maximum over the row counts up to m.
     size_t bytes = smooth_bytes(m, k, quant_algo);
     // A plan splits K only while tiles * splits <= 512, which even the tallest (256-row) tiles exceed
-    // beyond 256 * (256 / column tiles) rows; below that the plan may change at any row count.  The
-    // partial buffer grows with the rows, so the largest row count that splits sets the maximum.
+    // beyond 256 * (256 / column tiles) rows; below that the plan may change at any row count.
+    // Within a class of 16 rows every candidate has the same tiles, and the partial traffic, which
+    // grows with the rows, only ever favours fewer splits: the splits of the class's first row count
+    // times its last row count bound the class.
     size_t split = split_bytes(m, n, k, quant_algo);
     int const col_tiles = (n + 255) / 256;
     int const cap = 256 * (col_tiles >= 256 ? 1 : 256 / col_tiles);
-    for (int mm = m - 1 < cap ? m - 1 : cap; mm >= 1 && split == 0; --mm)
-        split = split_bytes(mm, n, k, quant_algo);
+    int const top = m - 1 < cap ? m - 1 : cap;
+    for (int lo = 1; lo <= top; lo += 16)
+    {
+        int const hi = lo + 15 < top ? lo + 15 : top;
+        size_t const per_row = split_bytes(lo, n, k, quant_algo) / (size_t) lo;
+        split = per_row * hi > split ? per_row * hi : split;
+    }
     size_t const tuned = tuned_split_bytes(m, n, k, quant_algo);
     bytes += split > tuned ? split : tuned;
     return bytes;

@@ -22,7 +22,7 @@ struct GemmParams
     int tiles_m, tiles_n;
     int k_splits;        // workgroups along K per output tile (blockIdx.y)
     int tiles_per_split; // tile rows of K each of them covers
-    float* partial;      // [m, n] float32, zeroed, when k_splits > 1
+    float* partial;      // [k_splits, m, n] float32 when k_splits > 1: slab y holds K slice y's sums
     // grouped problems (see MatmulProblem): m is the total row count, tiles_m an upper bound of
     // the row tiles of all experts together
     int64_t const* expert_rows = nullptr;
@@ -111,26 +111,36 @@ __device__ __forceinline__ bool xcd_tile(int total, int& t)
     return (int) (blockIdx.x >> 3) < per_xcd && t < total;
 }
 
-// split-K helpers: clear the float32 partial buffer, then out = T(alpha * partial + bias)
-template <int DT>
-__global__ void __launch_bounds__(256) gemm_zero_partial(float* partial, size_t count)
-{
-    size_t const i = ((size_t) blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i < count)
-        *reinterpret_cast<f32x4*>(partial + i) = f32x4{0.f, 0.f, 0.f, 0.f}; // count is a multiple of 16
-}
-
+// split-K finish: the workgroups of K slice y store their float32 partial sums in slab y of the
+// workspace ([splits][m][n], every element of every slab written exactly once per call, so nothing
+// needs clearing); out = T(alpha * (slab 0 + slab 1 + ...) + bias), summed in slab order: the result
+// does not depend on which workgroup finished first.  Four consecutive columns per thread
+// (n is a multiple of 16).
 template <int DT>
 __global__ void __launch_bounds__(256) gemm_finish_partial(
-    void* out, float const* partial, void const* bias, float alpha, int m, int n)
+    void* out, float const* partial, void const* bias, float alpha, int m, int n, int splits)
 {
     using E = Elem<DT>;
-    size_t const i = (size_t) blockIdx.x * 256 + threadIdx.x;
-    if (i >= (size_t) m * n)
+    size_t const count = (size_t) m * n;
+    size_t const i = ((size_t) blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= count)
         return;
+    f32x4 sum = *reinterpret_cast<f32x4 const*>(partial + i);
+    for (int y = 1; y < splits; ++y)
+    {
+        f32x4 const v = *reinterpret_cast<f32x4 const*>(partial + (size_t) y * count + i);
+        sum[0] += v[0], sum[1] += v[1], sum[2] += v[2], sum[3] += v[3];
+    }
     int const col = (int) (i % n);
-    float const b = bias ? E::load(bias, col) : 0.f;
-    static_cast<uint16_t*>(out)[i] = E::store(__builtin_fmaf(alpha, partial[i], b));
+    f32x4 b = {0.f, 0.f, 0.f, 0.f};
+    if (bias)
+    {
+        u32x2 const v = *reinterpret_cast<u32x2 const*>(static_cast<uint16_t const*>(bias) + col);
+        b = f32x4{E::lo(v[0]), E::hi(v[0]), E::lo(v[1]), E::hi(v[1])};
+    }
+    u32x2 const o = {E::pack(__builtin_fmaf(alpha, sum[0], b[0]), __builtin_fmaf(alpha, sum[1], b[1])),
+        E::pack(__builtin_fmaf(alpha, sum[2], b[2]), __builtin_fmaf(alpha, sum[3], b[3]))};
+    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + i) = o;
 }
 
 } // namespace woq

@@ -346,8 +346,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block,
                     // lane (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c, so the
                     // epilogue moves 8 bytes per lane and block instead of 2
-                    // (the split-K variant keeps the plain orientation: its float atomics coalesce
-                    // better with 16 consecutive columns per row and instruction)
+                    // (the split-K variant keeps the plain orientation: its float32 stores cover
+                    // 64 consecutive bytes per row and instruction)
                     if constexpr (SPLITK)
                         E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
                     else
@@ -392,7 +392,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     mma_drain();
     if constexpr (SPLITK)
     {
-        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c)
+        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c);
+        // this K slice's own slab of the partial buffer (a slice past the end of K stores zeros)
+        float* const slab = p.partial + (size_t) blockIdx.y * ((size_t) p.m * p.n);
 #pragma unroll
         for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -402,7 +404,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 {
                     int const row = m0 + rt * 16 + kg * 4 + r;
                     if (strip_ok[s] && row < p.m)
-                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + strip_of[s] * 16 + c, acc[rt][s][r]);
+                        slab[(size_t) row * p.n + strip_of[s] * 16 + c] = acc[rt][s][r];
                 }
         return;
     }
@@ -530,11 +532,9 @@ int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;
-        hipLaunchKernelGGL((gemm_zero_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream, gp.partial,
-            count);
         hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, true>), grid, block, 0, stream, gp);
-        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count + 255) / 256)), block, 0, stream, gp.out,
-            gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
+        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream,
+            gp.out, gp.partial, gp.bias, gp.alpha, gp.m, gp.n, gp.k_splits);
     }
     else
         hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);

@@ -193,8 +193,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             {
                 // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block, lane
                 // (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c (8-byte epilogue accesses)
-                // (the split-K variant keeps the plain orientation: its float atomics coalesce better
-                // with 16 consecutive columns per row and instruction)
+                // (the split-K variant keeps the plain orientation: its float32 stores cover 64 consecutive
+                // bytes per row and instruction)
                 if constexpr (SPLITK)
                     mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
                 else
@@ -248,7 +248,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     fp8_saturation_off();
     if constexpr (SPLITK)
     {
-        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c)
+        // plain orientation: acc[rt][s][r] = (row m0 + rt*16 + kg*4 + r, column strip*16 + c);
+        // this K slice's own slab of the partial buffer (a slice past the end of K stores zeros)
+        float* const slab = p.partial + (size_t) blockIdx.y * ((size_t) p.m * p.n);
 #pragma unroll
         for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -258,7 +260,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 {
                     int const row = m0 + rt * 16 + kg * 4 + r;
                     if (strip0 + s < p.strips && row < p.m)
-                        unsafeAtomicAdd(p.partial + (size_t) row * p.n + (strip0 + s) * 16 + c, acc[rt][s][r]);
+                        slab[(size_t) row * p.n + (strip0 + s) * 16 + c] = acc[rt][s][r];
                 }
         return;
     }
@@ -303,11 +305,9 @@ int launch_w4a8_variant(GemmParams const& gp, hipStream_t stream)
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;
-        hipLaunchKernelGGL((gemm_zero_partial<ODT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream,
-            gp.partial, count);
         hipLaunchKernelGGL((gemm_w4a8_kernel<ODT, ZERO, RT, true>), grid, block, 0, stream, gp);
-        hipLaunchKernelGGL((gemm_finish_partial<ODT>), dim3((unsigned) ((count + 255) / 256)), block, 0, stream, gp.out,
-            gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
+        hipLaunchKernelGGL((gemm_finish_partial<ODT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream,
+            gp.out, gp.partial, gp.bias, gp.alpha, gp.m, gp.n, gp.k_splits);
     }
     else
         hipLaunchKernelGGL((gemm_w4a8_kernel<ODT, ZERO, RT, false>), grid, block, 0, stream, gp);

@@ -533,7 +533,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 if (strip_ok[s] && row0 + r < p.m)
                 {
                     if constexpr (SPLITK)
-                        unsafeAtomicAdd(p.partial + (size_t) (row0 + r) * p.n + col[s], v);
+                        (p.partial + (size_t) blockIdx.y * ((size_t) p.m * p.n))[(size_t) (row0 + r) * p.n + col[s]] = v;
                     else
                         out16[(size_t) (row0 + r) * p.n + col[s]] = E::store(__builtin_fmaf(p.alpha, v, bias[s]) + res[s][r]);
                 }
@@ -549,11 +549,9 @@ int launch_skinny_rt(GemmParams const& gp, hipStream_t stream)
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;
-        hipLaunchKernelGGL((gemm_zero_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block256, 0, stream,
-            gp.partial, count);
         hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, RT, true>), grid, block, 0, stream, gp);
-        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count + 255) / 256)), block256, 0, stream, gp.out,
-            gp.partial, gp.bias, gp.alpha, gp.m, gp.n);
+        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block256, 0, stream,
+            gp.out, gp.partial, gp.bias, gp.alpha, gp.m, gp.n, gp.k_splits);
     }
     else
         hipLaunchKernelGGL((skinny_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);

@@ -164,14 +164,19 @@ size_t tuned_split_bytes(int m, int n, int k, int quant_algo)
         return 0;
     std::shared_lock<std::shared_timed_mutex> lock(g_mutex);
     // an entry serves every row count from the previous profiled one up to its own
+    size_t bytes = 0;
     for (auto const& e : g_table)
     {
         Key const& key = e.first;
         if (std::get<0>(key) == n && std::get<1>(key) == k && std::get<2>(key) == quant_algo
             && e.second.regime == WOQ_REGIME_GEMM && e.second.k_splits > 1)
-            return (size_t) m * (size_t) n * 4; // some call of at most m rows may split K
+        {
+            int const rows = std::get<5>(key) < m ? std::get<5>(key) : m;
+            size_t const b = split_partial_bytes(rows, n, e.second.k_splits);
+            bytes = b > bytes ? b : bytes;
+        }
     }
-    return 0;
+    return bytes;
 }
 
 } // namespace woq

@@ -70,7 +70,7 @@ int launch_dequant(void* out, void const* weight, void const* scales, void const
     int bits, int dtype, void* stream);
 
 // How the GEMM regime runs a problem: which kernel, rows per output tile and the number of
-// workgroups that split K for one tile (with a float32 partial buffer of ws_bytes when > 1).
+// workgroups that split K for one tile (each with its own float32 slab of the ws_bytes when > 1).
 struct GemmPlan
 {
     bool skinny;  // deferred-scale 64-row kernel instead of the exact-dequantize prefill kernel
@@ -79,6 +79,12 @@ struct GemmPlan
     size_t ws_bytes;
     double cost_us; // the cost model's estimate (plan_gemm only)
 };
+
+// float32 partial sums of a K split: one [m, n] slab per slice of K
+inline size_t split_partial_bytes(int m, int n, int k_splits)
+{
+    return k_splits > 1 ? (size_t) m * (size_t) n * 4 * (size_t) k_splits : 0;
+}
 
 // Output tiles (of 16*rt rows x 256 columns) a problem has.
 inline long gemm_tiles(int m, int n, int rt)
@@ -89,14 +95,14 @@ inline long gemm_tiles(int m, int n, int rt)
 // Estimated time (microseconds) of a 16-bit GEMM-regime problem on one kernel, tile height and K
 // split, from a model fitted to sweeps over the Llama-3-8B / 70B layer shapes (M = 32 .. 1024, int4
 // g128 and int8 per-channel, every kernel / tile height / split count from 1 to 20: picking by it
-// stays within 1 % of the best measured choice on average, 10 % at worst):
+// stays within 1.6 % of the best measured choice on average, 15 % at worst):
 //   * a workgroup spends c microseconds per tile row of K (c = a + b * rt for the exact-dequantize
 //     kernel: the dequantize is paid once per workgroup, the MFMAs per row; a constant for the
-//     deferred-scale kernel's 64- or 32-row tile) plus a prologue / epilogue of ~2 us per tile;
+//     deferred-scale kernel's 64- or 32-row tile) plus a prologue / epilogue of 1.7 - 3 us per tile;
 //   * one workgroup per CU: ceil(workgroups / 256) rounds of tiles one after another (counted on the
 //     fullest XCD), and a last round of more than 224 workgroups runs ~10 % longer (measured: 256
 //     workgroups are no faster than 192, and 257 take two rounds);
-//   * splitting K costs the reduction launch and the float32 partial traffic.
+//   * splitting K costs the reduction launch and the float32 partial slabs (written once, read once).
 // `tiles` is the output tile count of that tile height (for a grouped problem: over all experts).
 inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, int splits)
 {
@@ -104,18 +110,19 @@ inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k,
     int const k_tiles = (k + tk - 1) / tk;
     double c;
     if (skinny)
-        c = bits == 4 ? (rt == 2 ? 0.878 : 1.344) : 0.596;
+        c = bits == 4 ? (rt == 2 ? 0.79 : 1.29) : 0.565;
     else
-        c = bits == 4 ? 0.803 + 0.105 * rt : 0.640 + 0.0387 * rt;
+        c = bits == 4 ? 0.807 + 0.108 * rt : 0.642 + 0.0404 * rt;
     // the tiles are dealt to the 8 XCDs (32 CUs each) in equal contiguous runs: the fullest XCD
     // sets the number of rounds
     long const wgs = (tiles + 7) / 8 * splits;
     long const rounds = (wgs + 31) / 32;
     int const steps = (k_tiles + splits - 1) / splits;
     double const last_round = wgs - (rounds - 1) * 32 > 28 ? 0.10 : 0.0;
-    double t = ((double) rounds + last_round) * (steps * c + 1.98 + 0.02 * rt) + 1.6;
+    double const per_tile = skinny ? 3.15 : 1.34 + 0.081 * rt; // prologue and epilogue
+    double t = ((double) rounds + last_round) * (steps * c + per_tile) + 2.25;
     if (splits > 1)
-        t += 2.5 + (double) m * n * 4.0 * (2 + 2 * splits) * 3.5e-7;
+        t += 2.9 + (double) m * n * 4.0 * splits * 3.3e-7;
     return t;
 }
 
@@ -190,7 +197,7 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
         if (allow_split && v >= 1 && v <= k_tiles)
             pl.k_splits = v;
     }
-    pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+    pl.ws_bytes = split_partial_bytes(m, n, pl.k_splits);
     pl.cost_us = best;
     return pl;
 }
@@ -220,17 +227,17 @@ inline double stream_cost_us(int m, int n, int k)
 // W4A8 runs on one kernel (exact dequantize to e4m3, 64/128/256-row tiles, optional split-K).
 // Estimated time (microseconds) of one tile height and K split: the same model as gemm_cost_us,
 // fitted to a sweep of the fp8 kernel over the Llama-3-8B / 70B shapes (M = 32 .. 4096, every tile
-// height, splits 1 .. 20): picking by it stays within 0.6 % of the best measured choice on average.
+// height, splits 1 .. 20): picking by it stays within 0.4 % of the best measured choice on average.
 inline double w4a8_cost_us(int rt, long tiles, int m, int n, int k, int splits)
 {
     int const k_tiles = (k + 127) / 128;
     long const wgs = (tiles + 7) / 8 * splits; // on the fullest XCD
     long const rounds = (wgs + 31) / 32;
     int const steps = (k_tiles + splits - 1) / splits;
-    double const last_round = wgs - (rounds - 1) * 32 > 28 ? 0.07 : 0.0;
-    double t = ((double) rounds + last_round) * (steps * (1.18 + 0.0405 * rt) + 1.42) + 4.1;
+    double const last_round = wgs - (rounds - 1) * 32 > 28 ? 0.04 : 0.0;
+    double t = ((double) rounds + last_round) * (steps * (1.13 + 0.044 * rt) + 2.09) + 4.6;
     if (splits > 1)
-        t += 1.7 + (double) m * n * 4.0 * (2 + 2 * splits) * 3.44e-7;
+        t += 2.5 + (double) m * n * 4.0 * (2 + 2 * splits) * 1.29e-7;
     return t;
 }
 
@@ -271,7 +278,7 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
             }
         }
     }
-    pl.ws_bytes = pl.k_splits > 1 ? (size_t) m * (size_t) n * 4 : 0;
+    pl.ws_bytes = split_partial_bytes(m, n, pl.k_splits);
     return pl;
 }
 

@@ -80,7 +80,7 @@ def profile_tactics(pre_quant_scale, weight, scales, zeros, bias, *, n: int, k: 
     out = torch.empty((max_m, n), dtype=dtype, device=dev)
     need = lib.woq_workspace_bytes(max_m, n, k, quant_algo, _WOQ_DT[dtype])
     # room for every split-K candidate, not only the heuristics' own
-    need = max(need, max_m * k * 2 + 256 + min(max_m, 1024) * n * 4)
+    need = max(need, max_m * k * 2 + 256 + min(max_m * n * 4 * 20, 160 << 20))
     workspace = torch.empty(need, dtype=torch.uint8, device=dev)
     args = MatmulArgs(
         act=_ptr(act), pre_quant_scale=_ptr(pre_quant_scale), weight=_ptr(weight), scales=_ptr(scales),
