@@ -112,7 +112,8 @@ def test_gemm_skinny_m_splits_k(pkg, oracle, dev, M, K, N):
 
 
 def test_gemm_split_k_reuses_a_dirty_workspace(pkg, oracle, dev):
-    """The partial buffer is cleared by the call itself: a workspace full of garbage, used twice."""
+    """Every element of the partial slabs is written by the call before the finish pass reads it: a
+    workspace full of garbage, used twice."""
     F = pkg.functional
     p = random_problem(oracle, 48, 4096, 256, 4, 128, "bf16", zero=True, pqs=True, seed=77)
     need = pkg._lib.lib.woq_workspace_bytes(48, 256, 4096, F.ZERO | F.PRE_QUANT_SCALE, pkg._lib.BF16)
@@ -128,3 +129,17 @@ def test_gemm_split_k_reuses_a_dirty_workspace(pkg, oracle, dev):
                                workspace=ws)
         torch.cuda.synchronize()
         assert oracle.max_rel_err(out.float().cpu().numpy(), ref) < TOL
+
+
+@pytest.mark.parametrize("bits,group,dtype", [(4, 128, "bf16"), (8, 0, "fp16")])
+def test_gemm_split_k_is_bit_reproducible(pkg, oracle, dev, monkeypatch, bits, group, dtype):
+    """The K slices are summed in slice order, whichever workgroup finishes first: repeated calls
+    return the same bits, on either GEMM kernel (the fixture's) and for several split counts."""
+    p = random_problem(oracle, 96, 4096, 512, bits, group, dtype, zero=group != 0, bias=True, seed=13)
+    for splits in (2, 5, 8):
+        monkeypatch.setenv("WOQ_GEMM_SPLITS", str(splits))
+        first = run_product(pkg, oracle, dev, p, GEMM)
+        assert oracle.max_rel_err(first, reference(oracle, p)) < TOL, splits
+        for _ in range(3):
+            again = run_product(pkg, oracle, dev, p, GEMM)
+            assert (again.view(np.uint32) == first.view(np.uint32)).all(), splits
