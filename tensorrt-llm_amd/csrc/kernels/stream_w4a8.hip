@@ -22,15 +22,18 @@
 namespace woq
 {
 
-// ALDS: the workgroup stages the activation rows in LDS once (small M x K) and the lanes read
+// LDSM 1: the workgroup stages the activation rows in LDS once (small M x K) and the lanes read
 // their A pieces from there; a pipeline stage then holds packed weights and scales only.
-template <int ODT, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
+// LDSM 2: the group scales and zeros of the workgroup's columns are staged as well.
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
 __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 {
     using EO = Elem<ODT>;
     using EH = Elem<WOQ_FP16>;
     constexpr int TK = 128, SLABS = 4;
-    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (K + 16) bytes
+    constexpr bool ALDS = LDSM != 0; // activation rows staged in LDS
+    constexpr bool SCLDS = LDSM == 2; // and the group scales / zeros of the workgroup's columns
+    extern __shared__ u32x4 act_lds[]; // ALDS: rows x (K + 16) bytes, then the staged scales, then zeros
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
     if (group >= p.groups)
@@ -72,6 +75,12 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     uint32_t const lds_row = (uint32_t) K + 16u;
     int const a_row = c < p.m ? c : p.m - 1;
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 8u;
+    // SCLDS variants stage the group scales (and zeros) of the workgroup's columns behind the
+    // activations (it pays on long K, where the staging pass is a small part of the workgroup's time): one row of NS * 16 values per tile row of K (group 128 = one tile row), strip
+    // slot s at columns s * 16 ..; a pipeline stage then holds packed weights only
+    constexpr uint32_t SC_ROW = NS * 32u;
+    char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) (p.m < 16 ? p.m : 16) * lds_row;
+    char* const zr_lds = sc_lds + (uint32_t) KT * SC_ROW;
 
     struct Stage
     {
@@ -93,27 +102,45 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             for (int j = 0; j < SLABS; ++j)
                 st.a[j] = buffer_load_x2(act_rsrc, (a_lane + (uint32_t) (kt * TK + j * 32)) | past);
         }
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
+        if constexpr (!SCLDS)
         {
-            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + sc_lane[s]) | past;
-            st.s[s] = buffer_load_u16(sc_rsrc, off);
-            if constexpr (ZERO)
-                st.z[s] = buffer_load_u16(zr_rsrc, off);
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+            {
+                uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + sc_lane[s]) | past;
+                st.s[s] = buffer_load_u16(sc_rsrc, off);
+                if constexpr (ZERO)
+                    st.z[s] = buffer_load_u16(zr_rsrc, off);
+            }
         }
+    };
+    // raw scale / zero of strip slot s for tile row kt: from the stage, or from the staged copy
+    auto scale_bits = [&](Stage const& st, int kt, int s) -> uint16_t
+    {
+        if constexpr (SCLDS)
+            return *reinterpret_cast<uint16_t const*>(sc_lds + (uint32_t) kt * SC_ROW + (uint32_t) (s * 16 + c) * 2u);
+        else
+            return st.s[s];
+    };
+    auto zero_bits = [&](Stage const& st, int kt, int s) -> uint16_t
+    {
+        if constexpr (SCLDS)
+            return *reinterpret_cast<uint16_t const*>(zr_lds + (uint32_t) kt * SC_ROW + (uint32_t) (s * 16 + c) * 2u);
+        else
+            return st.z[s];
     };
 
     // Saturation to +-448 is part of the conversion, but a weight cannot reach it while
     // 8|s| + |z| stays below: one wavefront-wide test per tile row takes the clamp (a quarter of
     // the conversion's instructions) out of the common case.
-    auto convert_and_multiply = [&](Stage const& st, i32x8 a, auto clamp_tag)
+    auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 a, auto clamp_tag)
     {
         constexpr bool CLAMP = decltype(clamp_tag)::value;
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
-            float const sc = EH::from_bits(st.s[s]);
-            float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
+            float const sc = EH::from_bits(scale_bits(st, kt, s));
+            float const zr = ZERO ? EH::from_bits(zero_bits(st, kt, s)) : 0.f;
             i32x8 b;
 #pragma unroll
             for (int j = 0; j < SLABS; ++j)
@@ -137,14 +164,14 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
-            float const bound = __builtin_fmaf(8.f, __builtin_fabsf(EH::from_bits(st.s[s])),
-                ZERO ? __builtin_fabsf(EH::from_bits(st.z[s])) : 0.f);
+            float const bound = __builtin_fmaf(8.f, __builtin_fabsf(EH::from_bits(scale_bits(st, kt, s))),
+                ZERO ? __builtin_fabsf(EH::from_bits(zero_bits(st, kt, s))) : 0.f);
             may_saturate |= !(bound <= 440.f); // also true for NaN scales
         }
         if (__builtin_amdgcn_ballot_w64(may_saturate) != 0)
-            convert_and_multiply(st, a, std::true_type{});
+            convert_and_multiply(st, kt, a, std::true_type{});
         else
-            convert_and_multiply(st, a, std::false_type{});
+            convert_and_multiply(st, kt, a, std::false_type{});
     };
 
     // tile rows of this wavefront: kt = wave + it * WAVES.  Every load tolerates kt >= KT, so
@@ -166,6 +193,18 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
             u32x4 const v = buffer_load_x4(act_rsrc, (uint32_t) row * (uint32_t) K + (uint32_t) ch * 16u);
             *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + (uint32_t) row * lds_row + (uint32_t) ch * 16u) = v;
+        }
+        // group scales / zeros: 16-byte chunks of 8 columns, NS * 2 per tile row of K; strips past
+        // the end of N are clamped as for the weights
+        for (int idx = threadIdx.x; SCLDS && idx < KT * NS * 2; idx += WAVES * 64)
+        {
+            int const kt = idx / (NS * 2), ch = idx - kt * (NS * 2);
+            int const strip = strip0 + (ch >> 1) < p.strips ? strip0 + (ch >> 1) : p.strips - 1;
+            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n + (uint32_t) (strip * 16 + (ch & 1) * 8)) * 2u;
+            *reinterpret_cast<u32x4*>(sc_lds + (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u) = buffer_load_x4(sc_rsrc, off);
+            if constexpr (ZERO)
+                *reinterpret_cast<u32x4*>(zr_lds + (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u)
+                    = buffer_load_x4(zr_rsrc, off);
         }
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
@@ -222,6 +261,14 @@ struct W4a8Shape
 };
 
 constexpr size_t kMaxActLds = 48 * 1024;
+// most dynamic LDS of a staged variant: activations plus the group scales and zeros of its columns
+// (k / 128 rows of ns * 32 bytes each); the static reduction buffer takes up to 32 KiB more
+constexpr size_t kMaxStagedLds = 96 * 1024;
+
+size_t scale_lds_bytes(int k_tiles, int ns, bool zeros)
+{
+    return (size_t) k_tiles * (size_t) ns * 32 * (zeros ? 2 : 1);
+}
 
 size_t act_lds_bytes(int m, int k)
 {
@@ -241,9 +288,12 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
     // and 8-way split K (two strips on very wide matrices, deeper prefetch on long K).
     if (act_lds_bytes(m, k) <= kMaxActLds)
     {
+        // the group scales join the activations in LDS from K = 8192 on (2-4 % there; on K = 4096 the
+        // staging pass costs more than the loads it saves)
+        int const lds = k_tiles >= 64 && act_lds_bytes(m, k) + scale_lds_bytes(k_tiles, 2, true) <= kMaxStagedLds ? 2 : 1;
         if (strips >= 2048)
-            return {2, 8, 2, 1};
-        return k_tiles >= 112 ? W4a8Shape{1, 8, 4, 1} : W4a8Shape{1, 8, 2, 1};
+            return {2, 8, 2, lds};
+        return k_tiles >= 112 ? W4a8Shape{1, 8, 4, lds} : W4a8Shape{1, 8, 2, lds};
     }
     // otherwise two strips per wavefront share the activation loads once there are enough
     // column groups to fill the chip; narrow matrices keep one strip
@@ -256,21 +306,24 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
     return {1, 8, 2, 0};
 }
 
-template <int ODT, bool ZERO, int NS, int WAVES, int PF, bool ALDS>
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
 int launch_variant(StreamParams sp, hipStream_t stream)
 {
-    auto kernel = stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF, ALDS>;
+    auto kernel = stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF, LDSM>;
     size_t lds = 0;
-    if constexpr (ALDS)
+    if constexpr (LDSM != 0)
     {
         lds = act_lds_bytes(sp.m, sp.k);
         if (lds > kMaxActLds)
             return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
+        lds += LDSM == 2 ? scale_lds_bytes(sp.k_tiles, NS, ZERO) : 0;
+        if (lds > kMaxStagedLds)
+            return fail(WOQ_ERR_UNSUPPORTED, "staged operands of %zu bytes do not fit the LDS staging area", lds);
         static bool raised = false; // benign race: the attribute call is idempotent
         if (lds > 32 * 1024 && !raised)
         {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxActLds);
+                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxStagedLds);
             if (e != hipSuccess)
                 return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             raised = true;
@@ -291,19 +344,22 @@ int launch_shaped(StreamParams const& sp, hipStream_t s)
 {
     W4a8Shape const sh = pick_shape(sp.m, sp.k, sp.strips, sp.k_tiles);
 #define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
-    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && (sh.lds != 0) == LDS_)                                   \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                                   \
         return launch_variant<ODT, ZERO, NS_, WAVES_, PF_, LDS_>(sp, s);
-    WOQ_SHAPE(1, 8, 2, false)
-    WOQ_SHAPE(1, 16, 2, false)
-    WOQ_SHAPE(2, 8, 2, false)
-    WOQ_SHAPE(2, 8, 3, false)
-    WOQ_SHAPE(2, 4, 4, false)
-    WOQ_SHAPE(4, 8, 2, false)
-    WOQ_SHAPE(1, 8, 2, true)
-    WOQ_SHAPE(1, 8, 4, true)
-    WOQ_SHAPE(2, 8, 2, true)
-    WOQ_SHAPE(2, 4, 4, true)
-    WOQ_SHAPE(4, 8, 2, true)
+    WOQ_SHAPE(1, 8, 2, 0)
+    WOQ_SHAPE(1, 16, 2, 0)
+    WOQ_SHAPE(2, 8, 2, 0)
+    WOQ_SHAPE(2, 8, 3, 0)
+    WOQ_SHAPE(2, 4, 4, 0)
+    WOQ_SHAPE(4, 8, 2, 0)
+    WOQ_SHAPE(1, 8, 2, 1)
+    WOQ_SHAPE(1, 8, 4, 1)
+    WOQ_SHAPE(2, 8, 2, 1)
+    WOQ_SHAPE(2, 4, 4, 1)
+    WOQ_SHAPE(4, 8, 2, 1)
+    WOQ_SHAPE(1, 8, 2, 2)
+    WOQ_SHAPE(1, 8, 4, 2)
+    WOQ_SHAPE(2, 8, 2, 2)
 #undef WOQ_SHAPE
     return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated", sh.ns,
         sh.waves, sh.pf, sh.lds);
