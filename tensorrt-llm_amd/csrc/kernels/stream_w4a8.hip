@@ -25,14 +25,15 @@ namespace woq
 // LDSM 1: the workgroup stages the activation rows in LDS once (small M x K) and the lanes read
 // their A pieces from there; a pipeline stage then holds packed weights and scales only.
 // LDSM 2: the group scales and zeros of the workgroup's columns are staged as well.
+// LDSM 3: only those (activations too large for the LDS come from registers).
 template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
 __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 {
     using EO = Elem<ODT>;
     using EH = Elem<WOQ_FP16>;
     constexpr int TK = 128, SLABS = 4;
-    constexpr bool ALDS = LDSM != 0; // activation rows staged in LDS
-    constexpr bool SCLDS = LDSM == 2; // and the group scales / zeros of the workgroup's columns
+    constexpr bool ALDS = LDSM == 1 || LDSM == 2; // activation rows staged in LDS
+    constexpr bool SCLDS = LDSM >= 2;             // the group scales / zeros of the workgroup's columns staged
     extern __shared__ u32x4 act_lds[]; // ALDS: rows x (K + 16) bytes, then the staged scales, then zeros
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
@@ -79,7 +80,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     // activations (it pays on long K, where the staging pass is a small part of the workgroup's time): one row of NS * 16 values per tile row of K (group 128 = one tile row), strip
     // slot s at columns s * 16 ..; a pipeline stage then holds packed weights only
     constexpr uint32_t SC_ROW = NS * 32u;
-    char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) (p.m < 16 ? p.m : 16) * lds_row;
+    char* const sc_lds = reinterpret_cast<char*>(act_lds) + (ALDS ? (uint32_t) (p.m < 16 ? p.m : 16) * lds_row : 0u);
     char* const zr_lds = sc_lds + (uint32_t) KT * SC_ROW;
 
     struct Stage
@@ -183,12 +184,12 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     for (int i = 0; i < PF; ++i)
         fetch(st[i], wave + i * WAVES);
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (ALDS)
+    if constexpr (ALDS || SCLDS)
     {
         // behind the first weight prefetches: the activations come from L2 and land first
         int const rows = p.m < 16 ? p.m : 16;
         int const chunks_per_row = K / 16;
-        for (int idx = threadIdx.x; idx < rows * chunks_per_row; idx += WAVES * 64)
+        for (int idx = threadIdx.x; ALDS && idx < rows * chunks_per_row; idx += WAVES * 64)
         {
             int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
             u32x4 const v = buffer_load_x4(act_rsrc, (uint32_t) row * (uint32_t) K + (uint32_t) ch * 16u);
@@ -295,15 +296,16 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
             return {2, 8, 2, lds};
         return k_tiles >= 112 ? W4a8Shape{1, 8, 4, lds} : W4a8Shape{1, 8, 2, lds};
     }
-    // otherwise two strips per wavefront share the activation loads once there are enough
-    // column groups to fill the chip; narrow matrices keep one strip
-    if (strips >= 2048)
-        return {2, 4, 4, 0};
-    if (strips >= 512)
-        return k_tiles >= 128 ? W4a8Shape{2, 8, 3, 0} : W4a8Shape{2, 8, 2, 0};
-    if (strips >= 384 && m > 4)
-        return {2, 8, 2, 0};
-    return {1, 8, 2, 0};
+    // otherwise (activations in registers) the group scales alone are staged, and two strips per
+    // wavefront share the activation loads once there are enough column groups to fill the chip, four
+    // on very wide matrices with more than 8 rows; narrow matrices keep one strip (swept over every
+    // instantiated shape on the Llama-3-8B / 70B layer shapes, M = 8 and 16)
+    int const lds = scale_lds_bytes(k_tiles, 4, true) <= kMaxStagedLds ? 3 : 0;
+    if (strips > 1024)
+        return m > 8 ? W4a8Shape{4, 8, 2, lds} : W4a8Shape{2, 8, 2, lds};
+    if (strips >= 512 || (strips >= 384 && m > 4))
+        return {2, 8, 2, lds};
+    return {1, 8, 2, lds};
 }
 
 template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
@@ -313,10 +315,10 @@ int launch_variant(StreamParams sp, hipStream_t stream)
     size_t lds = 0;
     if constexpr (LDSM != 0)
     {
-        lds = act_lds_bytes(sp.m, sp.k);
+        lds = LDSM == 3 ? 0 : act_lds_bytes(sp.m, sp.k);
         if (lds > kMaxActLds)
             return fail(WOQ_ERR_UNSUPPORTED, "activations of %zu bytes do not fit the LDS staging area", lds);
-        lds += LDSM == 2 ? scale_lds_bytes(sp.k_tiles, NS, ZERO) : 0;
+        lds += LDSM >= 2 ? scale_lds_bytes(sp.k_tiles, NS, ZERO) : 0;
         if (lds > kMaxStagedLds)
             return fail(WOQ_ERR_UNSUPPORTED, "staged operands of %zu bytes do not fit the LDS staging area", lds);
         static bool raised = false; // benign race: the attribute call is idempotent
@@ -360,6 +362,11 @@ int launch_shaped(StreamParams const& sp, hipStream_t s)
     WOQ_SHAPE(1, 8, 2, 2)
     WOQ_SHAPE(1, 8, 4, 2)
     WOQ_SHAPE(2, 8, 2, 2)
+    WOQ_SHAPE(1, 8, 2, 3)
+    WOQ_SHAPE(2, 8, 2, 3)
+    WOQ_SHAPE(2, 8, 3, 3)
+    WOQ_SHAPE(2, 4, 4, 3)
+    WOQ_SHAPE(4, 8, 2, 3)
 #undef WOQ_SHAPE
     return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated", sh.ns,
         sh.waves, sh.pf, sh.lds);
