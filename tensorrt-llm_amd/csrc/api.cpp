@@ -152,10 +152,13 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
             reg.lds = 2;
         return reg;
     }
-    if (mt == 2)
-        return {stream_mid_ns(strips), 8, 2, 0};
-    if (mt == 4)
-        return {stream_mid_ns(strips), 8, 1, 0};
+    if (mt == 2 || mt == 4)
+    {
+        // the group scales / zeros (at most k * ns bytes) are staged in LDS while they are small
+        int const ns = stream_mid_ns(strips);
+        int const lds = group != 0 && (size_t) k * ns <= (size_t) 48 * 1024 ? 2 : 0;
+        return {ns, 8, mt == 2 ? 2 : 1, lds};
+    }
     return {1, 8, 1, 0};
 }
 

@@ -80,7 +80,7 @@ template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int 
 __device__ __forceinline__ void stream_body(StreamParams const& p)
 {
     constexpr bool ALDS = LDS == 1;
-    static_assert(LDS == 0 || MT == 1, "LDS-staged operands are for M <= 16");
+    static_assert(LDS != 1 || MT == 1, "LDS-staged activations are for M <= 16");
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
@@ -734,6 +734,14 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
     WOQ_SHAPE(4, 2, 8, 1, 0)
     WOQ_SHAPE(8, 1, 4, 1, 0)
     WOQ_SHAPE(8, 1, 8, 1, 0)
+    if constexpr (GROUP != 0)
+    {
+        // skinny M, group scales / zeros in LDS
+        WOQ_SHAPE(2, 2, 8, 2, 2)
+        WOQ_SHAPE(2, 1, 8, 2, 2)
+        WOQ_SHAPE(4, 1, 8, 1, 2)
+        WOQ_SHAPE(4, 2, 8, 1, 2)
+    }
 #undef WOQ_SHAPE
     return fail(WOQ_ERR_UNSUPPORTED, "stream shape mt=%d ns=%d waves=%d pf=%d lds=%d is not instantiated", mt, sh.ns,
         sh.waves, sh.pf, sh.lds);

@@ -92,9 +92,9 @@ std::vector<Tactic> candidates(woq_matmul_args const& a, bool stream_allowed)
             add(1, 8, 4, l), add(2, 8, 2, l), add(4, 4, 2, l);
         }
         else if (mt == 2)
-            add(2, 8, 2, 0), add(1, 8, 2, 0);
+            add(2, 8, 2, 0), add(1, 8, 2, 0), add(2, 8, 2, l), add(1, 8, 2, l);
         else if (mt == 4)
-            add(1, 8, 1, 0), add(2, 8, 1, 0);
+            add(1, 8, 1, 0), add(2, 8, 1, 0), add(1, 8, 1, l), add(2, 8, 1, l);
         else
             add(1, 4, 1, 0), add(1, 8, 1, 0);
     }

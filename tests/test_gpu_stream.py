@@ -195,3 +195,16 @@ def test_stream_register_activations_long_k(pkg, oracle, dev, K, group):
     p = random_problem(oracle, 9, K, 48, 4, group, "bf16", zero=True, seed=K % 1000)
     err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
     assert err < TOL, err
+
+
+@pytest.mark.parametrize("shape,M", [("2,8,2,2", 17), ("1,8,2,2", 32), ("2,8,2,0", 25), ("1,8,1,2", 33), ("2,8,1,2", 64),
+                                     ("1,8,1,0", 50), ("1,4,1,0", 100), ("1,8,1,0", 128)])
+def test_stream_skinny_m_launch_shapes(pkg, oracle, dev, monkeypatch, shape, M):
+    """The launch shapes of 17..128 rows (two, four and eight row tiles per wavefront), with and
+    without the group scales staged in LDS: a tile-row count no wavefront count divides, N that ends
+    inside a workgroup's strips."""
+    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    for bits, group, dtype in [(4, 128, "bf16"), (4, 64, "fp16"), (8, 128, "bf16")]:
+        p = random_problem(oracle, M, 1408, 272, bits, group, dtype, zero=True, bias=True, pqs=True, seed=M)
+        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        assert err < TOL, (shape, bits, group, dtype, err)
