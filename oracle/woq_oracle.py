@@ -525,6 +525,28 @@ def max_rel_err(out, ref) -> float:
     return float(np.abs(np.asarray(out, np.float64) - ref).max() / (denom if denom > 0 else 1.0))
 
 
+def column_magnitude(act, w, alpha: float = 1.0) -> np.ndarray:
+    """Expected magnitude of one output of column n when the signs of its K products are random:
+    sqrt(mean_m sum_k (alpha * a[m, k] * w[k, n])^2).  The floor of the per-column norm below."""
+    a2 = np.asarray(act, np.float64) ** 2
+    w2 = np.asarray(w, np.float64) ** 2
+    return abs(float(alpha)) * np.sqrt((a2 @ w2).mean(axis=0))
+
+
+def max_col_rel_err(out, ref, col_floor=None) -> float:
+    """Per-output-column parity norm: max_n ( max_m |out - ref|[m, n] / max(max_m |ref|[m, n], floor[n]) ).
+    A wrong strip or column shows here whatever the magnitude of the other columns.  `col_floor`
+    (column_magnitude of the same operands) keeps the norm meaningful when a column's few outputs all
+    happen to lie near zero (M = 1: the elementwise relative error is ill-defined there)."""
+    ref = np.asarray(ref, np.float64)
+    ref = ref.reshape(-1, ref.shape[-1])
+    err = np.abs(np.asarray(out, np.float64).reshape(ref.shape) - ref).max(axis=0)
+    denom = np.abs(ref).max(axis=0)
+    if col_floor is not None:
+        denom = np.maximum(denom, np.asarray(col_floor, np.float64))
+    return float((err / np.where(denom > 0, denom, 1.0)).max())
+
+
 # --------------------------------------------------------------------------------------
 # checkpoint-side folding rules (callers of the op)
 # --------------------------------------------------------------------------------------

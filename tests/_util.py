@@ -35,6 +35,17 @@ def reference(oracle, p, alpha=1.0):
                                  p["group"], p["dtype"])
 
 
+def parity_err(oracle, out, p, alpha=1.0, w4a8=False):
+    """The larger of the two parity norms of `out` against the float64 oracle: the global one,
+    max|out - ref| / max|ref|, and the per-output-column one (oracle.max_col_rel_err, floored by the
+    column's expected output magnitude)."""
+    ref = reference(oracle, p, alpha)
+    a = p["act"] if p["pqs"] is None else oracle.apply_per_channel_scale(p["act"], p["pqs"], p["dtype"])
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], p["group"], p["dtype"])
+    floor = oracle.column_magnitude(a, w, alpha)
+    return max(oracle.max_rel_err(out, ref), oracle.max_col_rel_err(out, ref, floor))
+
+
 def preprocess(pkg, oracle, q, bits, act_dtype=torch.bfloat16):
     src = torch.from_numpy(q if bits == 8 else oracle.pack_int8_tensor_to_packed_int4(q))
     qt = torch.int8 if bits == 8 else torch.quint4x2

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import random_problem, reference, run_product
+from _util import parity_err, random_problem, reference, run_product
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -27,7 +27,7 @@ def test_gemm_variants(pkg, oracle, dev, dtype, bits, group, zero):
     if group == 0 and zero:
         pytest.skip("per-channel has no zeros")
     p = random_problem(oracle, 300, 512, 512, bits, group, dtype, zero=zero, seed=bits + group)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
 
 
@@ -38,7 +38,7 @@ def test_gemm_at_most_32_rows(pkg, oracle, dev, dtype, group, zero, M):
     """M <= 32 with int4 weights: the deferred-scale kernel switches to 32-row tiles; K long enough
     that it also splits K, N ragged."""
     p = random_problem(oracle, M, 2048, 784, 4, group, dtype, zero=zero, bias=True, seed=M + group)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
 
 
@@ -46,7 +46,7 @@ def test_gemm_at_most_32_rows(pkg, oracle, dev, dtype, group, zero, M):
 def test_gemm_m_edges(pkg, oracle, dev, M):
     """Row counts around the 256-row tile, including the decode sizes forced onto this kernel."""
     p = random_problem(oracle, M, 256, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
 
 
@@ -55,7 +55,7 @@ def test_gemm_ragged_shapes(pkg, oracle, dev, K, N):
     """K with a padded last weight tile row, N that is not a multiple of the 256-column tile."""
     for bits, group in [(4, 64), (8, 64), (4, 0)]:
         p = random_problem(oracle, 260, K, N, bits, group, "bf16", zero=group != 0, seed=K + N)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
         assert err < TOL, (bits, group, err)
 
 
@@ -63,7 +63,7 @@ def test_gemm_ragged_shapes(pkg, oracle, dev, K, N):
 def test_gemm_prequant_scale_goes_through_workspace(pkg, oracle, dev, dtype):
     """AWQ smoothing in the GEMM regime: the smoothing pass writes the workspace, the GEMM reads it."""
     p = random_problem(oracle, 384, 512, 256, 4, 128, dtype, zero=True, bias=True, pqs=True, seed=5)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
 
 
@@ -93,10 +93,10 @@ def test_auto_regime_and_kernel_choice(pkg, oracle, dev, monkeypatch):
     monkeypatch.delenv("WOQ_GEMM_KERNEL")
     for m in (200, 640):
         p = random_problem(oracle, m, 512, 256, 4, 128, "bf16", zero=True, seed=40 + m)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p)
         assert err < TOL, (m, err)
     p = random_problem(oracle, 640, 256, 256, 8, 0, "fp16", seed=41)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p)
     assert err < TOL, err
 
 
@@ -107,7 +107,7 @@ def test_gemm_skinny_m_splits_k(pkg, oracle, dev, M, K, N):
     partial buffer (ragged K slices, a last slice shorter than the others, bias in the finish pass)."""
     for bits, group, dtype in [(4, 128, "bf16"), (8, 64, "fp16"), (4, 0, "fp16")]:
         p = random_problem(oracle, M, K, N, bits, group, dtype, zero=group != 0, bias=True, seed=M + K)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, GEMM), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
         assert err < TOL, (bits, group, dtype, err)
 
 
@@ -139,7 +139,7 @@ def test_gemm_split_k_is_bit_reproducible(pkg, oracle, dev, monkeypatch, bits, g
     for splits in (2, 5, 8):
         monkeypatch.setenv("WOQ_GEMM_SPLITS", str(splits))
         first = run_product(pkg, oracle, dev, p, GEMM)
-        assert oracle.max_rel_err(first, reference(oracle, p)) < TOL, splits
+        assert parity_err(oracle, first, p) < TOL, splits
         for _ in range(3):
             again = run_product(pkg, oracle, dev, p, GEMM)
             assert (again.view(np.uint32) == first.view(np.uint32)).all(), splits

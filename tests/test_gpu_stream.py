@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import random_problem, reference, run_product, preprocess, to_dev
+from _util import parity_err, random_problem, reference, run_product, preprocess, to_dev
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -19,7 +19,7 @@ STREAM = 1
 @pytest.mark.parametrize("M", [1, 3, 16])
 def test_stream_basic(pkg, oracle, dev, dtype, bits, group, M):
     p = random_problem(oracle, M, 512, 128, bits, group, dtype, seed=M + bits + group)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -29,14 +29,14 @@ def test_stream_basic(pkg, oracle, dev, dtype, bits, group, M):
 def test_stream_optional_inputs(pkg, oracle, dev, dtype, zero, bias, pqs, bits, group):
     """The eight (act_scale, zero, bias) variants of the reference dispatcher (kernelDispatcher.h:101-143)."""
     p = random_problem(oracle, 5, 1024, 256, bits, group, dtype, zero, bias, pqs, seed=zero * 4 + bias * 2 + pqs)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
 @pytest.mark.parametrize("M", [1, 2, 4, 7, 8, 15, 16, 17, 32, 33, 64, 100, 128])
 def test_stream_m_sweep(pkg, oracle, dev, M):
     p = random_problem(oracle, M, 1024, 1024, 4, 128, "bf16", zero=True, seed=M)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -46,7 +46,7 @@ def test_stream_ragged_shapes(pkg, oracle, dev, K, N):
     (partly empty XCD chunks), and the reference's own small test shapes."""
     for bits, group in [(4, 64), (8, 64), (4, 0)]:
         p = random_problem(oracle, 3, K, N, bits, group, "bf16", zero=group != 0, seed=K + N)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
         assert err < TOL, (bits, group, err)
 
 
@@ -87,7 +87,7 @@ def test_stream_large_activations_offset_cancellation(pkg, oracle, dev):
         for bits, group in [(4, 128), (8, 0)]:
             p = random_problem(oracle, 2, 4096, 64, bits, group, dtype, seed=5)
             p["act"] = oracle.round_to(p["act"] + 3.0, dtype)
-            err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+            err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
             assert err < TOL, (dtype, bits, err)
 
 
@@ -107,7 +107,7 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
     w = preprocess(pkg, oracle, p["q"], 8, torch.float16).to(dev)
     act, s = to_dev(p["act"], "fp16", dev), to_dev(p["scales"], "fp16", dev)
     out = F.weight_only_quant_matmul(act, w, s, F.INT8, "float16")
-    assert oracle.max_rel_err(out.float().cpu().numpy(), reference(oracle, p)) < TOL
+    assert parity_err(oracle, out.float().cpu().numpy(), p) < TOL
     out2 = torch.empty_like(out)
     assert P.WeightOnlyQuantMatmulPlugin(torch.float16, F.INT8).enqueue([act, w, s], [out2]) == 0
     assert (out2 == out).all()
@@ -116,7 +116,7 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
     w4 = preprocess(pkg, oracle, p4["q"], 4, torch.float16).to(dev)
     out4 = F.weight_only_quant_matmul(to_dev(p4["act"], "fp16", dev), w4, to_dev(p4["scales"], "fp16", dev), F.INT4)
     assert out4.shape == (4, 256)
-    assert oracle.max_rel_err(out4.float().cpu().numpy(), reference(oracle, p4)) < TOL
+    assert parity_err(oracle, out4.float().cpu().numpy(), p4) < TOL
     # groupwise plugin: inputs in plugin order, weight typed as the activation dtype ([K, N/4] halfs)
     pg = random_problem(oracle, 3, 512, 256, 4, 128, "bf16", zero=True, bias=True, pqs=True, seed=23)
     wg = preprocess(pkg, oracle, pg["q"], 4).to(dev).view(torch.bfloat16)
@@ -127,7 +127,7 @@ def test_functional_and_plugin_mirrors(pkg, oracle, dev):
                                                                          ("scales", "zeros", "bias")]
     assert plug.enqueue(ins, [outg]) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err(outg.float().cpu().numpy(), reference(oracle, pg)) < TOL
+    assert parity_err(oracle, outg.float().cpu().numpy(), pg) < TOL
 
 
 STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,1", "4,4,4,1", "4,8,2,1", "4,8,4,1",
@@ -143,7 +143,7 @@ def test_stream_every_launch_shape(pkg, oracle, dev, monkeypatch, shape, M):
     monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
     for bits, group, N in [(4, 128, 272), (8, 64, 64), (4, 0, 48)]:
         p = random_problem(oracle, M, 1280, N, bits, group, "bf16", zero=group != 0, pqs=True, seed=M + N)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
         assert err < TOL, (shape, bits, group, err)
 
 
@@ -151,7 +151,7 @@ def test_stream_every_launch_shape(pkg, oracle, dev, monkeypatch, shape, M):
 def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
     """Wide outputs take the multi-strip launch shapes of the heuristic."""
     p = random_problem(oracle, 1, 512, N, 4, 128, "bf16", zero=True, seed=N)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -164,7 +164,7 @@ def test_stream_long_k_staged_operands(pkg, oracle, dev, monkeypatch, M, K, grou
     N = 16384
     monkeypatch.setenv("WOQ_STREAM_SHAPE", "4,8,2,1")
     p = random_problem(oracle, M, K, N, bits, group, "bf16", zero=True, pqs=True, seed=K + M)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -177,14 +177,14 @@ def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, monkeypatch,
     if forced:
         monkeypatch.setenv("WOQ_STREAM_SHAPE", "1,8,4,1")
     p = random_problem(oracle, M, 14336, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
 def test_stream_activations_too_large_for_lds(pkg, oracle, dev):
     """M x K beyond the LDS staging area falls back to register-held activation fragments."""
     p = random_problem(oracle, 16, 4096, 64, 4, 128, "bf16", zero=True, seed=77)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -193,7 +193,7 @@ def test_stream_register_activations_long_k(pkg, oracle, dev, K, group):
     """More rows than the LDS holds and a long K: the group scales / zeros are staged in more than
     one pass (28672 / 64 groups), or not at all when even they are too many (K = 66048)."""
     p = random_problem(oracle, 9, K, 48, 4, group, "bf16", zero=True, seed=K % 1000)
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
 
 
@@ -206,5 +206,5 @@ def test_stream_skinny_m_launch_shapes(pkg, oracle, dev, monkeypatch, shape, M):
     monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
     for bits, group, dtype in [(4, 128, "bf16"), (4, 64, "fp16"), (8, 128, "bf16")]:
         p = random_problem(oracle, M, 1408, 272, bits, group, dtype, zero=True, bias=True, pqs=True, seed=M)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, STREAM), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
         assert err < TOL, (shape, bits, group, dtype, err)

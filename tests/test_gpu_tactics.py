@@ -5,7 +5,7 @@ an imported entry this build has no kernel for falls back to the heuristics."""
 import pytest
 import torch
 
-from _util import random_problem, reference, run_product, preprocess, to_dev
+from _util import parity_err, random_problem, reference, run_product, preprocess, to_dev
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -35,7 +35,7 @@ def test_profile_then_matmul(pkg, oracle, dev, bits, group, dtype):
     for m in (1, 5, 16, 40, 100, max_m):
         assert F.describe_tactic(m, N, K, group, algo, tdt).split()[0] in ("heuristic", "stream", "gemm")
         q = dict(p, act=p["act"][:m], M=m)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, q, 0, w_dev=w), reference(oracle, q))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, q, 0, w_dev=w), q)
         assert err < TOL, (m, F.describe_tactic(m, N, K, group, algo, tdt), err)
     assert F.describe_tactic(max_m + 1, N, K, group, algo, tdt) == "heuristic"
     # the exported text brings the same table back
@@ -52,7 +52,7 @@ def test_unknown_shape_falls_back(pkg, oracle, dev):
     # a streaming launch shape that passes the range checks but is not instantiated
     F.import_tactics("woq-tactics 1\n%d %d %d 128 %d %d 1 1 3 5 7 0 0 0 0\n" % (N, K, F.ZERO, dt, m))
     assert F.describe_tactic(m, N, K, 128, F.ZERO, torch.bfloat16).startswith("stream")
-    err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p)
     assert err < TOL, err
 
 
@@ -66,7 +66,7 @@ def test_plugin_initialize_profiles_the_layer(pkg, oracle, dev):
     assert "woq-tactics 1" in F.export_tactics()
     for m in (2, 20, max_m):
         p = random_problem(oracle, m, K, N, 4, 64, "bf16", zero=True, seed=m)
-        err = oracle.max_rel_err(run_product(pkg, oracle, dev, p, 0), reference(oracle, p))
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p)
         assert err < TOL, (m, err)
     per_channel = P.WeightOnlyQuantMatmulPlugin(torch.float16, F.INT8)
     assert per_channel.initialize(4, 4, N, K, device=dev) == 18 + 1
