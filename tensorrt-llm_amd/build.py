@@ -39,9 +39,25 @@ def sources():
     return sorted(out)
 
 
+def _headers_mtime() -> float:
+    newest = 0.0
+    for root, _, files in os.walk(os.path.dirname(HERE)):
+        if os.sep + "build" in root or os.sep + "." in root:
+            continue
+        for f in files:
+            if f.endswith(".h"):
+                newest = max(newest, os.path.getmtime(os.path.join(root, f)))
+    return newest
+
+
+_ONLY_CHANGED = False  # --changed: skip a translation unit whose object is newer than it and every header
+
+
 def _compile(src: str) -> str:
     rel = os.path.relpath(src, CSRC).replace(os.sep, "_")
     obj = os.path.join(OBJ, rel + ".o")
+    if _ONLY_CHANGED and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _headers_mtime()):
+        return obj
     extra = os.environ.get("WOQ_EXTRA_FLAGS", "").split()
     for prefix, flags in PER_FILE.items():
         if os.path.basename(src).startswith(prefix):
@@ -75,4 +91,7 @@ def build_lib(jobs: int | None = None, verbose: bool = True) -> str:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=None)
-    build_lib(ap.parse_args().jobs)
+    ap.add_argument("--changed", action="store_true", help="recompile only what changed (development)")
+    a = ap.parse_args()
+    _ONLY_CHANGED = a.changed
+    build_lib(a.jobs)
