@@ -136,6 +136,20 @@ int woq_matmul(const woq_matmul_args* args, void* stream);
 /* Validates exactly like woq_matmul but launches nothing (usable without a GPU). */
 int woq_matmul_check(const woq_matmul_args* args);
 
+/* woq_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose plugins
+ * always receive a workspace from TensorRT.  Same arguments and results, bit for bit, as
+ * woq_matmul; `workspace` / `workspace_bytes` are ignored: the split-K partial sums and the
+ * smoothed activations go to a device array of WOQ_STATIC_SCRATCH_BYTES that the library itself
+ * holds on every GPU it runs on until the process ends.  The call allocates and frees nothing.  A
+ * call that would need more scratch than that returns WOQ_ERR_WORKSPACE and launches nothing.
+ * All calls on one GPU share that GPU's array: calls that may overlap there (different streams)
+ * race; order them, or use woq_matmul with separate workspaces.  Every element of the scratch a
+ * call reads was written by that call, so nothing is cleared between calls. */
+#define WOQ_STATIC_SCRATCH_BYTES (32u << 20)
+int woq_matmul_static(const woq_matmul_args* args, void* stream);
+size_t woq_static_scratch_bytes(void);
+
 /* Device scratch that is enough for every woq_matmul call of this n, k, quant_algo with AT MOST m
  * rows (pass the largest m, as the reference passes its profile's maxM): a region for smoothed
  * activations (PRE_QUANT_SCALE, GEMM regime) followed by the float32 partial sums of the

@@ -62,6 +62,8 @@ def _load():
     sig = {
         "woq_matmul": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), vp]),
         "woq_matmul_check": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
+        "woq_matmul_static": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), vp]),
+        "woq_static_scratch_bytes": (sz, []),
         "woq_grouped_matmul": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs), vp]),
         "woq_grouped_matmul_check": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs)]),
         "woq_workspace_bytes": (sz, [i32, i32, i32, i32, i32]),

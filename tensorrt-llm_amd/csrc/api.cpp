@@ -5,10 +5,13 @@
 // of the small-M dispatcher (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernelDispatcher.h:30-166)
 // and of the runner's argument checks
 // (cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h:129-196).
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <initializer_list>
+
+#include <hip/hip_runtime.h>
 
 #include "woq_internal.h"
 
@@ -429,6 +432,88 @@ static int run_matmul(const woq_matmul_args* args, void* stream)
         p.workspace_bytes -= used;
     }
     return streaming ? launch_stream(p, stream) : launch_gemm(p, stream);
+}
+
+// ---- woq_matmul_static: the matmul for callers that cannot allocate ----------------------------
+// The split-K partial sums and the smoothed activations of the GEMM regime live in a file-scope
+// device array instead of a caller workspace.  In host code the array's NAME is only a stand-in
+// for the symbol: its device address is looked up once per device (every GPU holds its own copy
+// at its own address) and that pointer is what the kernels, through the workspace fields, receive.
+static __device__ __align__(256) unsigned char scratch[WOQ_STATIC_SCRATCH_BYTES];
+
+namespace
+{
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// device address of `scratch` on the current device (looked up on the first call there)
+int static_scratch_ptr(void** out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess)
+    {
+        (void) hipGetLastError();
+        return fail(WOQ_ERR_RUNTIME, "hipGetDevice failed: %s", hipGetErrorString(e));
+    }
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(WOQ_ERR_RUNTIME, "device ordinal %d is beyond the %d this library keeps scratch pointers for", dev,
+            kMaxDevices);
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr)
+    {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+        {
+            (void) hipGetLastError();
+            return fail(WOQ_ERR_RUNTIME, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+        }
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release); // racing first calls store the same address
+    }
+    *out = ptr;
+    return WOQ_OK;
+}
+} // namespace
+
+extern "C" size_t woq_static_scratch_bytes(void)
+{
+    return WOQ_STATIC_SCRATCH_BYTES;
+}
+
+extern "C" int woq_matmul_static(const woq_matmul_args* args, void* stream)
+{
+    if (!args)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "args is NULL");
+    woq_matmul_args a = *args;
+    a.workspace = nullptr;
+    a.workspace_bytes = 0;
+    // what this very call needs (the regime and plan woq_matmul would take without a tuned table
+    // entry that wants more room: with too little workspace it falls back to the built-in choice)
+    MatmulProblem p;
+    if (int rc = validate(&a, p))
+        return rc;
+    if (p.m == 0)
+        return WOQ_OK;
+    int const regime = pick_regime(&a);
+    size_t need = 0;
+    if (regime == WOQ_REGIME_GEMM)
+        need = gemm_workspace_bytes(p.m, p.n, p.k, a.quant_algo);
+    else if (p.w4a8)
+        need = smooth_bytes(p.m, p.k, a.quant_algo);
+    if (need > (size_t) WOQ_STATIC_SCRATCH_BYTES)
+        return fail(WOQ_ERR_WORKSPACE,
+            "woq_matmul_static: this call needs %zu bytes of scratch, the static scratch holds %zu; use woq_matmul "
+            "with a caller workspace",
+            need, (size_t) WOQ_STATIC_SCRATCH_BYTES);
+    if (need)
+    {
+        void* ptr = nullptr;
+        if (int rc = static_scratch_ptr(&ptr))
+            return rc;
+        a.workspace = ptr;
+        a.workspace_bytes = WOQ_STATIC_SCRATCH_BYTES;
+    }
+    return woq_matmul(&a, stream);
 }
 
 namespace

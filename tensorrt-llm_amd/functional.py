@@ -45,8 +45,10 @@ def _require_gpu(*tensors):
 
 def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int, k: int, group_size: int,
                    quant_algo: int, alpha: float = 1.0, out_dtype=None, regime: int = 0, workspace=None,
-                   out=None) -> torch.Tensor:
-    """One call of woq_matmul.  `act` is [..., k]; returns [..., n]."""
+                   out=None, static_scratch: bool = False) -> torch.Tensor:
+    """One call of woq_matmul.  `act` is [..., k]; returns [..., n].  With `static_scratch` the call goes
+    through woq_matmul_static: no workspace is allocated or passed, the library's own device array is
+    used (pass `out` as well and the call allocates nothing at all)."""
     _require_gpu(act, pre_quant_scale, weight, scales, zeros, bias, workspace, out)
     out_dtype = out_dtype or (act.dtype if act.dtype != torch.float8_e4m3fn else scales.dtype)
     if act.shape[-1] != k:
@@ -54,7 +56,7 @@ def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int,
     m = act.numel() // k if k else 0
     if out is None:
         out = torch.empty(act.shape[:-1] + (n,), dtype=out_dtype, device=act.device)
-    need = lib.woq_workspace_bytes(m, n, k, quant_algo, _WOQ_DT[act.dtype])
+    need = 0 if static_scratch else lib.woq_workspace_bytes(m, n, k, quant_algo, _WOQ_DT[act.dtype])
     if need and workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=act.device)
     args = MatmulArgs(
@@ -63,7 +65,8 @@ def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int,
         group_size=group_size, quant_algo=quant_algo, act_dtype=_WOQ_DT[act.dtype], out_dtype=_WOQ_DT[out_dtype],
         regime=regime, workspace=_ptr(workspace),
         workspace_bytes=0 if workspace is None else workspace.numel() * workspace.element_size())
-    check(lib.woq_matmul(ctypes.byref(args), _stream_handle(act.device)))
+    entry = lib.woq_matmul_static if static_scratch else lib.woq_matmul
+    check(entry(ctypes.byref(args), _stream_handle(act.device)))
     return out
 
 
