@@ -318,6 +318,11 @@ int woq_dequantize(void* out, const void* weight, const void* scales, const void
 
 /* ---- misc ------------------------------------------------------------------------------------ */
 
+/* The WOQ_* environment variables (experiment overrides of the built-in kernel choices) are read
+ * once, at the first call that consults them; this reads them again.  For tests and tuning scripts;
+ * no counterpart in the reference. */
+void woq_reload_env(void);
+
 const char* woq_last_error(void);
 int woq_abi_version(void);
 int woq_layout_version(void);

@@ -84,6 +84,7 @@ def _load():
         "woq_describe_tactic": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_char_p, sz]),
         "woq_export_tactics": (sz, [ctypes.c_char_p, sz]),
         "woq_import_tactics": (ctypes.c_int, [ctypes.c_char_p]),
+        "woq_reload_env": (None, []),
         "woq_last_error": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),
         "woq_layout_version": (ctypes.c_int, []),

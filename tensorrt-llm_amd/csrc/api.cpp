@@ -95,12 +95,9 @@ struct StreamShape
 
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group)
 {
-    if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
-    {
-        StreamShape sh{0, 0, 0, 0};
-        if (std::sscanf(e, "%d,%d,%d,%d", &sh.ns, &sh.waves, &sh.pf, &sh.lds) == 4)
-            return sh;
-    }
+    EnvOverrides const& env = env_overrides();
+    if (env.has_stream_shape)
+        return {env.stream_shape[0], env.stream_shape[1], env.stream_shape[2], env.stream_shape[3]};
     (void) k_tiles;
     if (Tactic const* t = current_tactic())
     {
@@ -165,20 +162,117 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
     return {1, 8, 1, 0};
 }
 
+int raise_lds_once(std::atomic<uint64_t>& raised, void const* kernel, int bytes)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess)
+    {
+        uint64_t const bit = (uint64_t) 1 << (dev & 63);
+        if (raised.load(std::memory_order_relaxed) & bit)
+            return WOQ_OK;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess)
+        {
+            raised.fetch_or(bit, std::memory_order_relaxed);
+            return WOQ_OK;
+        }
+    }
+    (void) hipGetLastError(); // do not leave the error for the caller's next runtime call
+    return fail(WOQ_ERR_RUNTIME, "raising the dynamic LDS limit failed: %s", hipGetErrorString(e));
+}
+
+struct WideShape
+{
+    int ns, waves, pf;
+};
+
+// The wide streaming kernel (a wavefront per NS strips over all of K) for this problem, and its launch
+// shape.  WOQ_WIDE_SHAPE="ns,waves,pf" forces it, "0" switches it off.
+bool pick_wide_shape(int m, int n, int k, int group, int bits, WideShape& out)
+{
+    (void) group;
+    (void) bits;
+    if (Tactic const* t = current_tactic())
+        if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)
+            return false; // a tuned launch shape of the strip-group kernel
+    EnvOverrides const& env = env_overrides();
+    if (env.wide_mode == 0 || (env.has_stream_shape && env.wide_mode != 1))
+        return false; // switched off, or a launch shape of the strip-group kernel is forced
+    if (env.wide_mode == 1)
+    {
+        out = WideShape{env.wide_shape[0], env.wide_shape[1], env.wide_shape[2]};
+        return true;
+    }
+    // Measured on MI355X (one row, int4): with K up to 4096 and at least 1536 column strips (the
+    // Llama-3-8B gate_up, 4096 x 28672) two strips per wavefront, four wavefronts, four tile rows in
+    // flight run 5-7 % faster than the strip-group kernel (13.5 against 14.3 us); with longer K or
+    // fewer columns the strip-group kernel is as fast or faster.
+    if (m == 1 && k <= 4096 && n >= 1536 * 16)
+    {
+        out = WideShape{2, 4, 4};
+        return true;
+    }
+    return false;
+}
+
+bool stream_slots_disabled()
+{
+    return env_overrides().slots_off;
+}
+
+namespace
+{
+EnvOverrides read_env()
+{
+    EnvOverrides o;
+    if (char const* e = std::getenv("WOQ_FORCE_REGIME"))
+        o.regime = !std::strcmp(e, "stream") ? WOQ_REGIME_STREAM : (!std::strcmp(e, "gemm") ? WOQ_REGIME_GEMM : 0);
+    if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
+        o.has_stream_shape = std::sscanf(e, "%d,%d,%d,%d", &o.stream_shape[0], &o.stream_shape[1], &o.stream_shape[2],
+                                 &o.stream_shape[3])
+            == 4;
+    if (char const* e = std::getenv("WOQ_WIDE_SHAPE"))
+        o.wide_mode = std::sscanf(e, "%d,%d,%d", &o.wide_shape[0], &o.wide_shape[1], &o.wide_shape[2]) == 3 ? 1 : 0;
+    if (char const* e = std::getenv("WOQ_STREAM_SLOTS"))
+        o.slots_off = e[0] == '0';
+    if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
+        o.gemm_kernel = !std::strcmp(e, "skinny") ? 2 : 1;
+    if (char const* e = std::getenv("WOQ_GEMM_RT"))
+    {
+        int const v = std::atoi(e);
+        o.gemm_rt = (v == 4 || v == 8 || v == 16) ? v : 0;
+    }
+    if (char const* e = std::getenv("WOQ_GEMM_SPLITS"))
+        o.gemm_splits = std::atoi(e);
+    return o;
+}
+
+// the overrides in force: replaced as a whole by woq_reload_env (the old set is left in place for
+// calls that still read it; reloading is a test and tuning facility, not a hot path)
+std::atomic<EnvOverrides const*> g_env{nullptr};
+} // namespace
+
+EnvOverrides const& env_overrides()
+{
+    EnvOverrides const* e = g_env.load(std::memory_order_acquire);
+    if (!e)
+    {
+        EnvOverrides const* fresh = new EnvOverrides(read_env());
+        if (g_env.compare_exchange_strong(e, fresh, std::memory_order_acq_rel))
+            return *fresh;
+        delete fresh; // another thread was first
+    }
+    return *e;
+}
+
 namespace
 {
 
 // Environment override of the regime, for experiments: WOQ_FORCE_REGIME=stream|gemm
 int env_regime()
 {
-    char const* e = std::getenv("WOQ_FORCE_REGIME");
-    if (!e)
-        return WOQ_REGIME_AUTO;
-    if (!std::strcmp(e, "stream"))
-        return WOQ_REGIME_STREAM;
-    if (!std::strcmp(e, "gemm"))
-        return WOQ_REGIME_GEMM;
-    return WOQ_REGIME_AUTO;
+    return env_overrides().regime;
 }
 
 int validate(woq_matmul_args const* a, MatmulProblem& p)
@@ -281,6 +375,11 @@ int pick_regime(woq_matmul_args const* a)
 } // namespace woq
 
 using namespace woq;
+
+extern "C" void woq_reload_env(void)
+{
+    g_env.store(new EnvOverrides(read_env()), std::memory_order_release);
+}
 
 extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo)
 {

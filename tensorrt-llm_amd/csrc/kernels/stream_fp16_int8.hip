@@ -1,5 +1,6 @@
 // Instantiates the weight-streaming kernel for FP16 activations and int8 weights.
 #include "stream_kernel.h"
+#include "stream_wide_kernel.h"
 
 namespace woq
 {

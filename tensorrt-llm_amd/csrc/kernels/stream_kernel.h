@@ -75,12 +75,22 @@ struct StreamStage
 //       the all-ones MFMA out of the K loop
 // ACT   the epilogue applies p.activation; a gated activation (value column j, gate column j + n/2) pairs
 //       the strips of a wavefront (even slot: value half, odd slot: gate half), output [m, n/2]
+// SLOTS group slots of the 16 MFMA rows (staged activations with group scales only).  With R = 16 / SLOTS
+//       rows or fewer, the M-tile has room for SLOTS groups of K side by side: the wavefront's g-th
+//       group puts its activations in MFMA rows (g % SLOTS) * R .. + R - 1 and zeros in the others, so
+//       one accumulator collects the partial sums of SLOTS groups, each in its own rows, and the scales
+//       are applied once per SLOTS groups instead of once per group (M = 1: every 16th group, i.e. once
+//       at the end for K up to 16 * WAVES tile rows).  1 = every group is scaled on its own.
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
-    bool ACT = false>
+    bool ACT = false, int SLOTS = 1>
 __device__ __forceinline__ void stream_body(StreamParams const& p)
 {
     constexpr bool ALDS = LDS == 1;
     static_assert(LDS != 1 || MT == 1, "LDS-staged activations are for M <= 16");
+    constexpr bool SL = SLOTS > 1;
+    constexpr int R = 16 / SLOTS; // rows of the M-tile one group slot takes
+    static_assert(!SL || (ALDS && GROUP != 0 && !ACT), "group slots need staged activations and group scales");
+    static_assert(SLOTS == 1 || SLOTS == 2 || SLOTS == 4 || SLOTS == 8 || SLOTS == 16, "SLOTS");
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
@@ -156,7 +166,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // LDS-staged activations: row r of the M-tile at byte r * lds_row; rows >= m read row m-1
     // (their products land in output rows that are never stored)
     uint32_t const lds_row = (uint32_t) KT * TK * 2u + 16u; // +16: rows start in different banks
-    int const a_row = c < p.m ? c : p.m - 1;
+    int const c_row = SL ? (c & (R - 1)) : c; // row of the M-tile this lane's A fragment belongs to
+    int const a_row = c_row < p.m ? c_row : p.m - 1;
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
     // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
     // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
@@ -167,6 +178,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     char* const zr_lds = sc_lds + (uint32_t) sc_rows * SC_ROW;
     // activation row sums of segment i (SEG rows of K): 16 floats (one per row of the M-tile) at i * 64
     char* const sum_lds = zr_lds + (ZERO ? (uint32_t) sc_rows * SC_ROW : 0u);
+    // group slots: 256 bytes of zeros behind the sums - the A fragments of the lanes whose slot is not the
+    // current group's, and the scale / zero / sum of slots past the end of K
+    char* const zero_lds = sum_lds + (SUMLDS ? (uint32_t) KT * SEGS * 64u : 0u);
+    int const n_my = (KT - wave + WAVES - 1) / WAVES; // tile rows of this wavefront: kt = wave + it * WAVES
 
     auto fetch = [&](Stage& st, int kt)
     {
@@ -210,11 +225,55 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
     };
 
-    auto compute = [&](Stage const& st, int kt)
+    // Group slots: scales of the SLOTS groups collected in acc_p (window `wnd` of this wavefront's groups).
+    // Register r of lane (kg, c) is MFMA row kg*4 + r = slot * R + row: the slot names the group, hence
+    // the scale, zero and activation row sum that apply; slots the wavefront never filled read zeros.
+    auto flush_slots = [&](int wnd)
+    {
+        if constexpr (SL)
+        {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                int const i = kg * 4 + r;
+                int const gi = wnd * SLOTS + i / R;        // the wavefront's gi-th group
+                int const it_i = gi / SEGS, seg_i = gi % SEGS;
+                bool const ok = it_i < n_my;
+                int const kt_i = wave + it_i * WAVES;
+                uint32_t const grow = (uint32_t) ((kt_i * TK + seg_i * SEG) / GROUP);
+                char const* sp = ok ? sc_lds + grow * SC_ROW + (uint32_t) c * 2u : zero_lds;
+                char const* zp = ok ? zr_lds + grow * SC_ROW + (uint32_t) c * 2u : zero_lds;
+                float const S = *reinterpret_cast<float const*>(
+                    ok ? sum_lds + (uint32_t) (kt_i * SEGS + seg_i) * 64u + (uint32_t) (i & (R - 1)) * 4u : zero_lds);
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    float const sc = E::from_bits(*reinterpret_cast<uint16_t const*>(sp + (ok ? s * 32 : 0)));
+                    float const zz = ZERO ? E::from_bits(*reinterpret_cast<uint16_t const*>(zp + (ok ? s * 32 : 0))) : 0.f;
+                    float const cc = __builtin_fmaf(-OFF, sc, zz);
+                    acc_out[s][0][r] = __builtin_fmaf(sc, acc_p[s][0][r], __builtin_fmaf(cc, S, acc_out[s][0][r]));
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                acc_p[s][0] = zero4;
+        }
+    };
+
+    auto compute = [&](Stage const& st, int kt, int it)
     {
 #pragma unroll
         for (int seg = 0; seg < SEGS; ++seg)
         {
+            // group slots: only the lanes of this group's slot read activations, the others zeros
+            [[maybe_unused]] char const* a_seg = a_lds;
+            if constexpr (SL)
+            {
+                int const slot = (it * SEGS + seg) & (SLOTS - 1);
+                a_seg = (c >> (R == 1 ? 0 : (R == 2 ? 1 : (R == 4 ? 2 : 3)))) == slot
+                    ? a_lds + (uint32_t) (kt * TK + seg * SEG) * 2u
+                    : zero_lds + (uint32_t) kg * 16u;
+            }
 #pragma unroll
             for (int js = 0; js < SEG_SLABS; ++js)
             {
@@ -223,7 +282,9 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                 {
-                    if constexpr (ALDS)
+                    if constexpr (SL)
+                        a[mt] = *reinterpret_cast<u32x4 const*>(a_seg + (uint32_t) (js * 32) * 2u);
+                    else if constexpr (ALDS)
                         a[mt] = *reinterpret_cast<u32x4 const*>(a_lds + (uint32_t) (kt * TK + j * 32) * 2u);
                     else
                     {
@@ -251,7 +312,12 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                         acc_p[s][mt] = E::mma(a[mt], b, acc_p[s][mt]);
                 }
             }
-            if constexpr (GROUP != 0)
+            if constexpr (SL)
+            {
+                if (((it * SEGS + seg + 1) & (SLOTS - 1)) == 0) // the last slot has been filled
+                    flush_slots((it * SEGS + seg) / SLOTS);
+            }
+            else if constexpr (GROUP != 0)
             {
                 // a segment past the end of K carries zero activations, scale 0 and zero 0.
                 // Lane (kg, c) register r is output row kg*4 + r: with a single row (decode,
@@ -308,7 +374,6 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // the compiler's wait-count tracking stays exact: compute(st[i]) waits only for its own
     // stage while the PF-1 younger stages stay in flight.  The scheduling barriers keep the
     // compiler from sinking the prefetch below the compute (it would, to save registers).
-    int const n_my = (KT - wave + WAVES - 1) / WAVES;
     auto kt_of = [&](int it) { return wave + it * WAVES; };
     // staging of the group scales / zeros: 16-byte chunks of 8 columns, NS * 2 per group of K
     int const sc_chunks = sc_rows * NS * 2;
@@ -471,6 +536,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         if constexpr (SCLDS)
             stage_scales_tail();
+        if constexpr (SL)
+        {
+            if (threadIdx.x < 16)
+                *reinterpret_cast<u32x4*>(zero_lds + threadIdx.x * 16u) = u32x4{0u, 0u, 0u, 0u};
+        }
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -481,13 +551,18 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         for (int i = 0; i < PF; ++i)
         {
             if (it + i < n_my)
-                compute(st[i], kt_of(it + i));
+                compute(st[i], kt_of(it + i), it + i);
             __builtin_amdgcn_sched_barrier(0);
             fetch(st[i], kt_of(it + i + PF));
             __builtin_amdgcn_sched_barrier(0);
         }
     }
 
+    if constexpr (SL)
+    {
+        if ((n_my * SEGS) & (SLOTS - 1)) // a last, partly filled window
+            flush_slots(n_my * SEGS / SLOTS);
+    }
     if constexpr (GROUP == 0)
     {
 #pragma unroll
@@ -505,8 +580,62 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     }
 
     // ---- cross-wavefront reduction (fixed order) and epilogue -------------------------------
-    constexpr int SLOTS = NS * MT * 4;
-    __shared__ float red[WAVES][SLOTS][64];
+    uint16_t* out16 = static_cast<uint16_t*>(p.out);
+    if constexpr (SL)
+    {
+        // Row `row` of the M-tile is spread over the SLOTS MFMA rows slot * R + row, i.e. over the lane's
+        // registers (R < 4) and the lanes kg: folded here in a fixed order, then across wavefronts.
+        constexpr int RL = R < 4 ? R : 4; // distinct rows of the M-tile per lane
+        __shared__ float red_sl[WAVES][NS][R][16];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            float v[RL];
+            if constexpr (R == 1)
+                v[0] = (acc_out[s][0][0] + acc_out[s][0][1]) + (acc_out[s][0][2] + acc_out[s][0][3]);
+            else if constexpr (R == 2)
+            {
+                v[0] = acc_out[s][0][0] + acc_out[s][0][2];
+                v[1] = acc_out[s][0][1] + acc_out[s][0][3];
+            }
+            else
+            {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    v[r] = acc_out[s][0][r];
+            }
+#pragma unroll
+            for (int r = 0; r < RL; ++r)
+            {
+                if constexpr (R <= 4)
+                    v[r] += __shfl_xor(v[r], 16);
+                v[r] += __shfl_xor(v[r], 32);
+                int const row = R <= 4 ? r : (kg & 1) * 4 + r;
+                if ((R <= 4 ? kg == 0 : kg < 2) && row < p.m)
+                    red_sl[wave][s][row][c] = v[r];
+            }
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < NS * R * 16; e += WAVES * 64)
+        {
+            int const s = e / (R * 16), row = (e >> 4) & (R - 1), cc = e & 15;
+            if (row >= p.m || strip0 + s >= p.strips)
+                continue;
+            float sum = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < WAVES; ++w2)
+                sum += red_sl[w2][s][row][cc];
+            int const ocol = (strip0 + s) * 16 + cc;
+            float v = p.alpha * sum;
+            if (p.bias)
+                v += E::load(p.bias, ocol);
+            out16[(size_t) row * p.n + ocol] = E::store(v);
+        }
+    }
+    else
+    {
+    constexpr int SLOTS_ = NS * MT * 4;
+    __shared__ float red[WAVES][SLOTS_][64];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
@@ -517,14 +646,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                     red[wave][(s * MT + mt) * 4 + r][lane] = acc_out[s][mt][r];
     __syncthreads();
 
-    uint16_t* out16 = static_cast<uint16_t*>(p.out);
     if (gated)
     {
         // value and gate sums sit in neighbouring strip slots: out = (x + bias_x) * f(g + bias_g)
         if constexpr (ACT && NS % 2 == 0)
         {
             int const n_out = p.n / 2;
-            for (int e = threadIdx.x; e < SLOTS / 2 * 64; e += WAVES * 64)
+            for (int e = threadIdx.x; e < SLOTS_ / 2 * 64; e += WAVES * 64)
             {
                 int const pslot = e >> 6, ln = e & 63; // (pair, mt, r)
                 int const ps = pslot / (MT * 4), mt = (pslot >> 2) % MT, r = pslot & 3;
@@ -554,7 +682,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         return;
     }
-    for (int e = threadIdx.x; e < SLOTS * 64; e += WAVES * 64)
+    for (int e = threadIdx.x; e < SLOTS_ * 64; e += WAVES * 64)
     {
         int const slot = e >> 6, ln = e & 63;
         int const s = slot / (MT * 4), mt = (slot >> 2) % MT, r = slot & 3;
@@ -577,12 +705,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         out16[(size_t) row * p.n + ocol] = E::store(v);
     }
+    } // !SL
 }
 
-template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS, int SLOTS = 1>
 __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 {
-    stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS>(p);
+    stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS, false, SLOTS>(p);
 }
 
 // Grouped problems: workgroup (x, e) is workgroup x of expert e's own matmul.  The parameters are
@@ -651,9 +780,11 @@ inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool 
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group);
+// WOQ_STREAM_SLOTS=0 switches the group-slot variants off (for A/B timing)
+bool stream_slots_disabled();
 
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
-    bool GROUPED = false>
+    bool GROUPED = false, int SLOTS = 1>
 int launch_stream_variant(StreamParams sp, hipStream_t stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
@@ -661,30 +792,23 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
         if constexpr (GROUPED)
             return stream_grouped_kernel<DT, BITS, GROUP, ZERO, NS, WAVES, PF, LDS>;
         else
-            return stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS>;
+            return stream_kernel<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS, SLOTS>;
     }();
     size_t lds = 0;
     if constexpr (LDS != 0)
     {
-        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO, LDS == 1);
+        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO, LDS == 1)
+            + (SLOTS > 1 ? 256 : 0); // group slots: a block of zeros behind the staged operands
         // the reduction buffer of the epilogue is static LDS of this variant and shares the CU's 160 KiB
         constexpr size_t kStaticLds = (size_t) WAVES * NS * MT * 4 * 64 * sizeof(float);
         constexpr size_t kMaxDynamic = stream_max_staged_lds(NS * MT, WAVES);
         static_assert(kStaticLds + kMaxDynamic <= 160 * 1024, "LDS of one CU");
         if (lds > kMaxDynamic)
             return fail(WOQ_ERR_UNSUPPORTED, "staged operands of %zu bytes do not fit the LDS staging area", lds);
-        static bool raised = false; // benign race: the attribute call is idempotent
-        if (lds > 32 * 1024 && !raised)
-        {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxDynamic);
-            if (e != hipSuccess)
-            {
-                (void) hipGetLastError(); // do not leave the error for the caller's next runtime call
-                return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-            }
-            raised = true;
-        }
+        static std::atomic<uint64_t> raised{0}; // one bit per device
+        if (lds > 32 * 1024)
+            if (int rc = raise_lds_once(raised, reinterpret_cast<void const*>(kernel), (int) kMaxDynamic))
+                return rc;
     }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
@@ -706,6 +830,19 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 #define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
     if (mt == MT_ && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                             \
         return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, MT_, NS_, WAVES_, PF_, LDS_>(sp, s);
+    // decode of a single row with staged activations and group scales: 16 groups of K share the MFMA
+    // rows and the scales are applied once per 16 groups (the launch shapes the built-in rule picks)
+    if constexpr (GROUP != 0)
+    {
+#define WOQ_SLOT_SHAPE(NS_, WAVES_, PF_)                                                                               \
+    if (mt == 1 && sp.m == 1 && sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == 1 && slots_ok)          \
+        return launch_stream_variant<DT, BITS, GROUP, PQS, ZERO, 1, NS_, WAVES_, PF_, 1, false, 16>(sp, s);
+        bool const slots_ok = !stream_slots_disabled();
+        WOQ_SLOT_SHAPE(1, 8, 4)
+        WOQ_SLOT_SHAPE(2, 8, 4)
+        WOQ_SLOT_SHAPE(4, 8, 2)
+#undef WOQ_SLOT_SHAPE
+    }
     // decode (M <= 16), activations in LDS
     WOQ_SHAPE(1, 1, 8, 4, 1)
     WOQ_SHAPE(1, 1, 8, 6, 1)
@@ -779,6 +916,9 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 }
 
 template <int DT, int BITS>
+bool try_launch_stream_wide(MatmulProblem const& p, StreamParams const& sp, hipStream_t s, int& rc);
+
+template <int DT, int BITS>
 int launch_stream_typed(MatmulProblem const& p, void* stream)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
@@ -807,6 +947,13 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;
     bool const zero = p.zeros != nullptr;
+    if (mt == 1)
+    {
+        // wide matrices at decode: the kernel whose wavefronts own whole columns, where the rule picks it
+        int rc = WOQ_OK;
+        if (try_launch_stream_wide<DT, BITS>(p, sp, s, rc) && rc != WOQ_ERR_UNSUPPORTED)
+            return rc;
+    }
     if (p.num_experts)
     {
         switch (p.group_size)

@@ -279,12 +279,9 @@ size_t act_lds_bytes(int m, int k)
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
 {
-    if (char const* e = std::getenv("WOQ_STREAM_SHAPE"))
-    {
-        W4a8Shape sh{0, 0, 0, 0};
-        if (std::sscanf(e, "%d,%d,%d,%d", &sh.ns, &sh.waves, &sh.pf, &sh.lds) == 4)
-            return sh;
-    }
+    EnvOverrides const& env = env_overrides();
+    if (env.has_stream_shape)
+        return {env.stream_shape[0], env.stream_shape[1], env.stream_shape[2], env.stream_shape[3]};
     // measured on MI355X.  Activations that fit the LDS staging area: one strip per wavefront
     // and 8-way split K (two strips on very wide matrices, deeper prefetch on long K).
     if (act_lds_bytes(m, k) <= kMaxActLds)
@@ -321,15 +318,10 @@ int launch_variant(StreamParams sp, hipStream_t stream)
         lds += LDSM >= 2 ? scale_lds_bytes(sp.k_tiles, NS, ZERO) : 0;
         if (lds > kMaxStagedLds)
             return fail(WOQ_ERR_UNSUPPORTED, "staged operands of %zu bytes do not fit the LDS staging area", lds);
-        static bool raised = false; // benign race: the attribute call is idempotent
-        if (lds > 32 * 1024 && !raised)
-        {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<void const*>(kernel),
-                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kMaxStagedLds);
-            if (e != hipSuccess)
-                return fail(WOQ_ERR_RUNTIME, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-            raised = true;
-        }
+        static std::atomic<uint64_t> raised{0}; // one bit per device
+        if (lds > 32 * 1024)
+            if (int rc = raise_lds_once(raised, reinterpret_cast<void const*>(kernel), (int) kMaxStagedLds))
+                return rc;
     }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;

@@ -1,6 +1,7 @@
 // Internal declarations shared by the host code and the kernel launchers of libwoq.
 #pragma once
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -20,6 +21,24 @@ inline int bits_of(int quant_type)
 {
     return quant_type == WOQ_W8_A16 ? 8 : 4;
 }
+
+// Experiment overrides from the environment, read once (at first use) and again by woq_reload_env():
+//   WOQ_FORCE_REGIME=stream|gemm      WOQ_STREAM_SHAPE=ns,waves,pf,lds   WOQ_WIDE_SHAPE=ns,waves,pf | 0
+//   WOQ_STREAM_SLOTS=0                WOQ_GEMM_KERNEL=exact|skinny       WOQ_GEMM_RT=4|8|16
+//   WOQ_GEMM_SPLITS=<n>
+struct EnvOverrides
+{
+    int regime = 0;                // woq_regime; 0 = none
+    bool has_stream_shape = false; // streaming kernels: strips per wavefront, wavefronts, tile rows in flight, LDS mode
+    int stream_shape[4] = {0, 0, 0, 0};
+    int wide_mode = -1;            // wide streaming kernel: -1 built-in rule, 0 off, 1 forced shape
+    int wide_shape[3] = {0, 0, 0};
+    bool slots_off = false;        // no group-slot variants of the streaming kernel
+    int gemm_kernel = 0;           // 0 any, 1 exact-dequantize, 2 deferred-scale
+    int gemm_rt = 0;               // row tiles per wavefront of the exact-dequantize / fp8 kernel
+    int gemm_splits = 0;           // K split of the GEMM regime
+};
+EnvOverrides const& env_overrides();
 
 // rows of K covered by one 1 KiB weight tile (16 columns wide)
 inline int tile_k_of_bits(int bits)
@@ -158,14 +177,8 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
     // rows per expert of a grouped problem (its tiles do not straddle experts)
     int const rows = num_experts > 1 ? (m + num_experts - 1) / num_experts : m;
     int const skinny_rt = (rows <= 32 && bits == 4) ? 2 : 4;
-    char const* forced = std::getenv("WOQ_GEMM_KERNEL");
-    int forced_rt = 0;
-    if (char const* r = std::getenv("WOQ_GEMM_RT"))
-    {
-        int const v = std::atoi(r);
-        if (v == 4 || v == 8 || v == 16)
-            forced_rt = v;
-    }
+    EnvOverrides const& env = env_overrides();
+    int const forced_rt = env.gemm_rt;
     GemmPlan pl{};
     double best = 0;
     bool have = false;
@@ -173,7 +186,7 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
     {
         bool const skinny = cand == 0;
         int const rt = skinny ? skinny_rt : (cand == 1 ? 4 : (cand == 2 ? 8 : 16));
-        if (forced && skinny != !std::strcmp(forced, "skinny"))
+        if (env.gemm_kernel && skinny != (env.gemm_kernel == 2))
             continue;
         if (!skinny && forced_rt && rt != forced_rt)
             continue;
@@ -191,12 +204,8 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
     }
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
-    if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
-    {
-        int const v = std::atoi(f);
-        if (allow_split && v >= 1 && v <= k_tiles)
-            pl.k_splits = v;
-    }
+    if (allow_split && env.gemm_splits >= 1 && env.gemm_splits <= k_tiles)
+        pl.k_splits = env.gemm_splits;
     pl.ws_bytes = split_partial_bytes(m, n, pl.k_splits);
     pl.cost_us = best;
     return pl;
@@ -246,19 +255,9 @@ inline GemmPlan plan_gemm_w4a8(int m, int n, int k)
     GemmPlan pl{};
     pl.skinny = false;
     int const k_tiles = (k + 127) / 128;
-    int forced_rt = 0, forced_splits = 0;
-    if (char const* r = std::getenv("WOQ_GEMM_RT"))
-    {
-        int const v = std::atoi(r);
-        if (v == 4 || v == 8 || v == 16)
-            forced_rt = v;
-    }
-    if (char const* f = std::getenv("WOQ_GEMM_SPLITS"))
-    {
-        int const v = std::atoi(f);
-        if (v >= 1 && v <= k_tiles)
-            forced_splits = v;
-    }
+    EnvOverrides const& env = env_overrides();
+    int const forced_rt = env.gemm_rt;
+    int const forced_splits = env.gemm_splits >= 1 && env.gemm_splits <= k_tiles ? env.gemm_splits : 0;
     bool have = false;
     for (int rt = 4; rt <= 16; rt *= 2)
     {
@@ -307,6 +306,11 @@ struct TacticScope
 bool find_tactic(woq_matmul_args const& a, Tactic& out);
 // float32 split-K bytes the tuned entries of this n, k, quant_algo may use for at most m rows
 size_t tuned_split_bytes(int m, int n, int k, int quant_algo);
+
+// Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncSetAttribute) on the current device, once per
+// device: `raised` holds one bit per device ordinal (ordinals from 64 on share bits, which only
+// repeats the idempotent call).  The sticky HIP error of a failed call is cleared.
+int raise_lds_once(std::atomic<uint64_t>& raised, void const* kernel, int bytes);
 
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;

@@ -41,3 +41,19 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def woq_env(monkeypatch, pkg):
+    """Sets (value) or removes (None) WOQ_* experiment overrides and has the library read them again
+    (it reads the environment once); the previous environment is back in force after the test."""
+    def set_env(**kv):
+        for key, value in kv.items():
+            if value is None:
+                monkeypatch.delenv(key, raising=False)
+            else:
+                monkeypatch.setenv(key, str(value))
+        pkg._lib.lib.woq_reload_env()
+    yield set_env
+    monkeypatch.undo()
+    pkg._lib.lib.woq_reload_env()

@@ -13,10 +13,10 @@ GEMM = 2
 
 
 @pytest.fixture(params=["exact", "skinny"], autouse=True)
-def gemm_kernel(request, monkeypatch):
+def gemm_kernel(request, woq_env):
     """The GEMM regime has two kernels (exact-dequantize 256-row tiles, deferred-scale 64-row tiles);
     every test below runs on each, whatever the library would pick for the shape."""
-    monkeypatch.setenv("WOQ_GEMM_KERNEL", request.param)
+    woq_env(WOQ_GEMM_KERNEL=request.param)
     return request.param
 
 
@@ -89,8 +89,8 @@ def test_gemm_matches_stream_kernel(pkg, oracle, dev):
     assert oracle.max_rel_err(a, b) < 1e-2  # each is within 1e-2 of the oracle; they round differently
 
 
-def test_auto_regime_and_kernel_choice(pkg, oracle, dev, monkeypatch):
-    monkeypatch.delenv("WOQ_GEMM_KERNEL")
+def test_auto_regime_and_kernel_choice(pkg, oracle, dev, woq_env):
+    woq_env(WOQ_GEMM_KERNEL=None)
     for m in (200, 640):
         p = random_problem(oracle, m, 512, 256, 4, 128, "bf16", zero=True, seed=40 + m)
         err = parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p)
@@ -132,12 +132,12 @@ def test_gemm_split_k_reuses_a_dirty_workspace(pkg, oracle, dev):
 
 
 @pytest.mark.parametrize("bits,group,dtype", [(4, 128, "bf16"), (8, 0, "fp16")])
-def test_gemm_split_k_is_bit_reproducible(pkg, oracle, dev, monkeypatch, bits, group, dtype):
+def test_gemm_split_k_is_bit_reproducible(pkg, oracle, dev, woq_env, bits, group, dtype):
     """The K slices are summed in slice order, whichever workgroup finishes first: repeated calls
     return the same bits, on either GEMM kernel (the fixture's) and for several split counts."""
     p = random_problem(oracle, 96, 4096, 512, bits, group, dtype, zero=group != 0, bias=True, seed=13)
     for splits in (2, 5, 8):
-        monkeypatch.setenv("WOQ_GEMM_SPLITS", str(splits))
+        woq_env(WOQ_GEMM_SPLITS=str(splits))
         first = run_product(pkg, oracle, dev, p, GEMM)
         assert parity_err(oracle, first, p) < TOL, splits
         for _ in range(3):

@@ -82,9 +82,9 @@ def test_grouped_prefill_sizes(pkg, oracle, dev):
 
 @pytest.mark.parametrize("regime", [STREAM, GEMM])
 @pytest.mark.parametrize("kernel", ["exact", "skinny"])
-def test_grouped_forced_kernels_agree(pkg, oracle, dev, monkeypatch, regime, kernel):
+def test_grouped_forced_kernels_agree(pkg, oracle, dev, woq_env, regime, kernel):
     """The same problem on each kernel family, whatever AUTO would pick."""
-    monkeypatch.setenv("WOQ_GEMM_KERNEL", kernel)
+    woq_env(WOQ_GEMM_KERNEL=kernel)
     p = grouped_problem(oracle, [20, 3, 0, 50, 33], 768, 272, 4, 128, "fp16", True, False, seed=12)
     out = run_grouped(pkg, oracle, dev, p, regime=regime)
     assert np.isfinite(out).all()

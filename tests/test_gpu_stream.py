@@ -136,11 +136,11 @@ STREAM_SHAPES = ["1,8,4,1", "1,8,6,1", "1,16,4,1", "2,8,4,1", "2,4,4,1", "4,4,2,
 
 @pytest.mark.parametrize("shape", STREAM_SHAPES)
 @pytest.mark.parametrize("M", [1, 5])
-def test_stream_every_launch_shape(pkg, oracle, dev, monkeypatch, shape, M):
+def test_stream_every_launch_shape(pkg, oracle, dev, woq_env, shape, M):
     """Every instantiated (strips per wavefront, wavefronts, prefetch depth, LDS staging) variant
     of the decode kernel, forced through WOQ_STREAM_SHAPE, against the oracle - including a strip
     count that is not a multiple of the strips per wavefront."""
-    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    woq_env(WOQ_STREAM_SHAPE=shape)
     for bits, group, N in [(4, 128, 272), (8, 64, 64), (4, 0, 48)]:
         p = random_problem(oracle, M, 1280, N, bits, group, "bf16", zero=group != 0, pqs=True, seed=M + N)
         err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
@@ -156,13 +156,13 @@ def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
 
 
 @pytest.mark.parametrize("M,K,group,bits", [(1, 8192, 64, 4), (3, 8192, 64, 4), (2, 4160, 64, 4), (5, 4096, 128, 8)])
-def test_stream_long_k_staged_operands(pkg, oracle, dev, monkeypatch, M, K, group, bits):
+def test_stream_long_k_staged_operands(pkg, oracle, dev, woq_env, M, K, group, bits):
     """Long K with four strips per wavefront (launch shape forced): the activations, the group scales / zeros and the
     activation row sums staged in LDS exceed what a thread keeps in registers across the weight
     prefetch (the staging tail loops run), take more than 64 KiB of LDS, and K = 4160 ends in half
     a weight tile whose scales, zeros and row sums must read as zero."""
     N = 16384
-    monkeypatch.setenv("WOQ_STREAM_SHAPE", "4,8,2,1")
+    woq_env(WOQ_STREAM_SHAPE="4,8,2,1")
     p = random_problem(oracle, M, K, N, bits, group, "bf16", zero=True, pqs=True, seed=K + M)
     err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
@@ -170,12 +170,12 @@ def test_stream_long_k_staged_operands(pkg, oracle, dev, monkeypatch, M, K, grou
 
 @pytest.mark.parametrize("M", [2, 4])
 @pytest.mark.parametrize("forced", [False, True])
-def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, monkeypatch, M, forced):
+def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, woq_env, M, forced):
     """Few column groups and a long K (a down projection at M = 2..4): the activations are staged in
     LDS although they take 57 / 115 KiB (by the heuristic up to 3 rows, since one workgroup per CU
     covers the problem anyway; forced for 4)."""
     if forced:
-        monkeypatch.setenv("WOQ_STREAM_SHAPE", "1,8,4,1")
+        woq_env(WOQ_STREAM_SHAPE="1,8,4,1")
     p = random_problem(oracle, M, 14336, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
     err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
@@ -199,12 +199,48 @@ def test_stream_register_activations_long_k(pkg, oracle, dev, K, group):
 
 @pytest.mark.parametrize("shape,M", [("2,8,2,2", 17), ("1,8,2,2", 32), ("2,8,2,0", 25), ("1,8,1,2", 33), ("2,8,1,2", 64),
                                      ("1,8,1,0", 50), ("1,4,1,0", 100), ("1,8,1,0", 128)])
-def test_stream_skinny_m_launch_shapes(pkg, oracle, dev, monkeypatch, shape, M):
+def test_stream_skinny_m_launch_shapes(pkg, oracle, dev, woq_env, shape, M):
     """The launch shapes of 17..128 rows (two, four and eight row tiles per wavefront), with and
     without the group scales staged in LDS: a tile-row count no wavefront count divides, N that ends
     inside a workgroup's strips."""
-    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    woq_env(WOQ_STREAM_SHAPE=shape)
     for bits, group, dtype in [(4, 128, "bf16"), (4, 64, "fp16"), (8, 128, "bf16")]:
         p = random_problem(oracle, M, 1408, 272, bits, group, dtype, zero=True, bias=True, pqs=True, seed=M)
         err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
         assert err < TOL, (shape, bits, group, dtype, err)
+
+
+@pytest.mark.parametrize("shape", ["2,4,4", "1,4,4"])
+@pytest.mark.parametrize("bits,group,dtype,K,N", [(4, 128, "bf16", 2176, 272), (4, 64, "fp16", 1408, 1040),
+                                                  (8, 64, "bf16", 1088, 144), (4, 128, "fp16", 128, 16),
+                                                  (4, 64, "bf16", 4160, 528)])
+def test_wide_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, bits, group, dtype, K, N):
+    """The wide-matrix decode kernel (a wavefront owns whole columns; 16 groups of K share the MFMA
+    rows, scales applied once per 16 groups), forced through WOQ_WIDE_SHAPE on small problems: group
+    counts that end inside a window of 16, K that ends in half a weight tile, N that ends inside a
+    workgroup's strips or inside a wavefront's pair of strips; every optional input."""
+    woq_env(WOQ_WIDE_SHAPE=shape)
+    for zero, bias, pqs in [(True, True, True), (False, False, False), (True, False, False), (False, True, True)]:
+        p = random_problem(oracle, 1, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N)
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+        assert err < TOL, (shape, zero, bias, pqs, err)
+
+
+def test_wide_decode_kernel_is_what_wide_single_row_problems_run_on(pkg, oracle, dev, woq_env):
+    """One row, K <= 4096, at least 1536 column strips: the built-in rule takes the wide kernel (switching it
+    off changes the float32 summation order, hence some output bits, while both stay within the bar), and
+    a one-hot activation returns the dequantized weight row through it."""
+    K, N = 512, 24576 + 48
+    p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=77)
+    auto = run_product(pkg, oracle, dev, p, 0)
+    assert parity_err(oracle, auto, p) < TOL
+    woq_env(WOQ_WIDE_SHAPE="0")
+    other = run_product(pkg, oracle, dev, p, 0)
+    assert parity_err(oracle, other, p) < TOL
+    assert (auto != other).any()
+    woq_env(WOQ_WIDE_SHAPE=None)
+    p["act"] = np.zeros((1, K), np.float32)
+    p["act"][0, 300] = 1.0
+    out = run_product(pkg, oracle, dev, p, 0)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")[300]
+    assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()

@@ -129,11 +129,11 @@ def test_w4a8_streaming_shapes(pkg, oracle, dev, M, K, N):
 @pytest.mark.parametrize("shape", ["1,8,2,0", "1,16,2,0", "2,8,2,0", "2,8,3,0", "2,4,4,0", "4,8,2,0", "1,8,2,1", "1,8,4,1",
                                    "2,8,2,1", "2,4,4,1", "4,8,2,1", "1,8,2,2", "1,8,4,2", "2,8,2,2",
                                    "1,8,2,3", "2,8,2,3", "2,8,3,3", "2,4,4,3", "4,8,2,3"])
-def test_w4a8_streaming_launch_shapes(pkg, oracle, dev, monkeypatch, shape):
+def test_w4a8_streaming_launch_shapes(pkg, oracle, dev, woq_env, shape):
     """Every instantiated launch shape (strips per wavefront, wavefronts, tile rows in flight, LDS mode:
     0 nothing staged, 1 activations, 2 activations + group scales and zeros, 3 scales and zeros only), whatever
     the table would pick: K with a tile-row count that no shape divides, N that ends inside a group."""
-    monkeypatch.setenv("WOQ_STREAM_SHAPE", shape)
+    woq_env(WOQ_STREAM_SHAPE=shape)
     M, K, N = 7, 2176, 272
     prob = oracle.make_w4a8_problem(M, K, N, seed=17, out_dtype="fp16")
     rng = np.random.default_rng(18)
