@@ -97,11 +97,24 @@ def rotated_copies(layer, copies):
     return out
 
 
+_workspaces = {}
+
+
+def workspace_for(pkg, m, layer, dev):
+    """One scratch buffer per (m, n, k, kind), sized by woq_workspace_bytes and reused by every launch
+    (the caller of the library owns the workspace; nothing is allocated inside the timed region)."""
+    key = (m, layer["n"], layer["k"], layer["algo"])
+    if key not in _workspaces:
+        need = pkg._lib.lib.woq_workspace_bytes(m, layer["n"], layer["k"], layer["algo"], pkg._lib.BF16)
+        _workspaces[key] = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+    return _workspaces[key]
+
+
 def launch(pkg, act, layer, out, regime=0):
     F = pkg.functional
     F.woq_matmul_raw(act, None, layer["weight"], layer["scales"], layer["zeros"], None, n=layer["n"], k=layer["k"],
                      group_size=layer["group"], quant_algo=layer["algo"], out_dtype=torch.bfloat16, out=out,
-                     regime=regime)
+                     regime=regime, workspace=workspace_for(pkg, act.shape[0], layer, act.device))
 
 
 def time_graph(fn_body, launches, repeats=1):

@@ -93,8 +93,10 @@ struct StreamShape
     int ns, waves, pf, lds;
 };
 
-StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group)
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group, int const* split_shape)
 {
+    if (split_shape && split_shape[0] != 0) // the K split's own launch shape
+        return {split_shape[0], split_shape[1], split_shape[2], split_shape[3]};
     EnvOverrides const& env = env_overrides();
     if (env.has_stream_shape)
         return {env.stream_shape[0], env.stream_shape[1], env.stream_shape[2], env.stream_shape[3]};
@@ -216,6 +218,52 @@ bool pick_wide_shape(int m, int n, int k, int group, int bits, WideShape& out)
     return false;
 }
 
+// bytes of float32 slabs a streaming launch of m rows splitting K into `slices` needs
+static size_t stream_slab_bytes(int m, int n, int slices)
+{
+    return slices > 1 ? (size_t) slices * (size_t) m * (size_t) n * 4 : 0;
+}
+
+// K slices of a streaming launch (1 = none) and, with a split, the launch shape that goes with it.
+// Splitting pays where the activations, re-read by every workgroup, outweigh the weights on the way
+// from the L2 to the CUs: several rows, long K, few columns (the down projections).  A workgroup then
+// covers more strips over a slice of K, so each activation fragment meets 2-4 times as many weights.
+// Measured on MI355X (int4 g128): 14336 x 4096 at M = 16 18.4 -> 12.8 us, M = 8 14.0 -> 12.2, M = 4
+// 12.3 -> 11.4; 28672 x 8192 at M = 16 39.9 -> 33.5, M = 8 32.5 -> 29.4; nothing to gain at K <= 8192
+// with N >= K or below 4 rows (the finish pass costs ~2.5 us).
+int pick_stream_k_slices(int m, int n, int k, int tile_k, int group, size_t workspace_bytes, int shape[4])
+{
+    (void) group;
+    int const k_tiles = (k + tile_k - 1) / tile_k;
+    int const strips = n / kTileN;
+    shape[0] = 0; // no shape of its own
+    int slices = env_overrides().stream_splits;
+    if (slices <= 0)
+    {
+        slices = 1;
+        Tactic const* t = current_tactic();
+        bool const tuned = t && t->regime == WOQ_REGIME_STREAM && t->ns != 0;
+        if (!tuned && !env_overrides().has_stream_shape && m <= 16 && k >= 8192 && k >= 2 * n)
+        {
+            if (m >= 8 && strips <= 512)
+            {
+                slices = 4;
+                shape[0] = 4, shape[1] = 4, shape[2] = 2, shape[3] = 2;
+            }
+            else if (m >= 4 && strips <= 256)
+            {
+                slices = 2;
+                shape[0] = 2, shape[1] = 8, shape[2] = 2, shape[3] = 2;
+            }
+        }
+    }
+    if (slices > k_tiles)
+        slices = k_tiles;
+    if (m > 16 || stream_slab_bytes(m, n, slices) > workspace_bytes)
+        return 1;
+    return slices;
+}
+
 bool stream_slots_disabled()
 {
     return env_overrides().slots_off;
@@ -245,6 +293,8 @@ EnvOverrides read_env()
     }
     if (char const* e = std::getenv("WOQ_GEMM_SPLITS"))
         o.gemm_splits = std::atoi(e);
+    if (char const* e = std::getenv("WOQ_STREAM_SPLITS"))
+        o.stream_splits = std::atoi(e);
     return o;
 }
 
@@ -415,6 +465,22 @@ size_t smooth_bytes(int m, int k, int quant_algo)
 }
 } // namespace
 
+// float32 slabs the streaming kernel may use for a K split with at most m rows
+static size_t stream_workspace_bytes(int m, int n, int k, int quant_algo)
+{
+    if (quant_algo & WOQ_ALGO_FP8_ALPHA)
+        return 0;
+    int const tile_k = tile_k_of_bits((quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4);
+    size_t need = 0;
+    for (int rows = 1; rows <= (m < 16 ? m : 16); ++rows)
+    {
+        int shape[4];
+        size_t const b = stream_slab_bytes(rows, n, pick_stream_k_slices(rows, n, k, tile_k, 0, (size_t) -1, shape));
+        need = b > need ? b : need;
+    }
+    return need;
+}
+
 // float32 partial buffer of one GEMM-regime call with exactly m rows
 static size_t split_bytes(int m, int n, int k, int quant_algo)
 {
@@ -456,7 +522,9 @@ extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t q
     }
     size_t const tuned = tuned_split_bytes(m, n, k, quant_algo);
     bytes += split > tuned ? split : tuned;
-    return bytes;
+    // the streaming regime's own K split (16-bit activations, at most 16 rows)
+    size_t const stream = stream_workspace_bytes(m, n, k, quant_algo);
+    return bytes > stream ? bytes : stream;
 }
 
 extern "C" int woq_matmul_check(const woq_matmul_args* args)
@@ -599,6 +667,14 @@ extern "C" int woq_matmul_static(const woq_matmul_args* args, void* stream)
         need = gemm_workspace_bytes(p.m, p.n, p.k, a.quant_algo);
     else if (p.w4a8)
         need = smooth_bytes(p.m, p.k, a.quant_algo);
+    else
+    {
+        // the streaming kernel splits K only if it is given room for the slabs: offer the scratch
+        // when they fit, else it runs without the split
+        need = stream_workspace_bytes(p.m, p.n, p.k, a.quant_algo);
+        if (need > (size_t) WOQ_STATIC_SCRATCH_BYTES)
+            need = 0;
+    }
     if (need > (size_t) WOQ_STATIC_SCRATCH_BYTES)
         return fail(WOQ_ERR_WORKSPACE,
             "woq_matmul_static: this call needs %zu bytes of scratch, the static scratch holds %zu; use woq_matmul "

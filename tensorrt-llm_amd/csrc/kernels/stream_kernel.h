@@ -23,6 +23,7 @@
 #include <type_traits>
 
 #include "device_common.h"
+#include "gemm_common.h"
 
 namespace woq
 {
@@ -39,6 +40,15 @@ struct StreamParams
     float alpha;
     int m, n, k;
     int k_tiles;        // ceil(k / TILE_K)
+    int act_stride;     // elements between rows of act (k, unless the launch splits K)
+    int w_strip_tiles;  // weight tiles between neighbouring strips (k_tiles, unless the launch splits K)
+    // K split across workgroups (k_slices > 1): blockIdx.y is the slice, slice_tiles tile rows each.  The
+    // launcher fills k / k_tiles with the LARGEST slice (what the LDS areas are sized for) and k_total
+    // with all of K; the kernel narrows the operands to its slice and stores float32 partial sums into
+    // slab blockIdx.y of `partial` ([k_slices][m][n]) for the finish pass to add up in slice order.
+    int k_slices = 1, slice_tiles = 0, k_total = 0;
+    float* partial = nullptr;
+    int split_shape[4] = {0, 0, 0, 0}; // host side: the launch shape chosen with the K split (ns, waves, pf, lds)
     int strips;         // n / 16
     int groups;         // ceil(strips / NS): column groups, one workgroup each
     int groups_per_xcd; // ceil(groups / 8)
@@ -114,8 +124,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int const c = lane & 15;  // column inside the strip (B operand) / row inside the M-tile (A operand)
     int const kg = lane >> 4; // which 8 of a slab's 32 rows this lane holds
-    int const K = p.k;
+    int const K = p.k;               // the rows of K this workgroup covers
     int const KT = p.k_tiles;
+    uint32_t const AS = (uint32_t) p.act_stride;    // elements between activation rows
+    uint32_t const WS = (uint32_t) p.w_strip_tiles; // tiles between strips
     int const strip0 = group * NS;
 
     u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
@@ -135,7 +147,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // Buffer descriptors: an access past num_records returns 0, which is exactly what rows >= m,
     // the padded tail of K and the scale rows of that tail must contribute - no branches needed.
     constexpr uint32_t kOob = 0x7FFFFFF0u;
-    auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
+    auto const act_rsrc = make_rsrc(p.act, ((uint32_t) (p.m - 1) * AS + (uint32_t) K) * 2u);
     auto const pqs_rsrc = make_rsrc(PQS ? p.pqs : p.act, (uint32_t) K * 2u);
     uint32_t const sz_bytes
         = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
@@ -143,7 +155,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     // weights too go through a descriptor: a prefetch past the last tile row is given an
     // out-of-range offset and costs no memory traffic, so the K loop needs no conditional loads
-    auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+    auto const w_rsrc = make_rsrc(p.weight, ((uint32_t) (p.strips - 1) * WS + (uint32_t) KT) * 1024u);
 
     // strips past the end of N (last group only) are clamped for loads and skipped at the store
     bool const gated = ACT && act_is_gated(p.activation);
@@ -160,7 +172,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         else
             strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
-        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
+        wlane[s] = ((uint32_t) strip_of[s] * WS * 64u + (uint32_t) lane) * 16u;
     }
 
     // LDS-staged activations: row r of the M-tile at byte r * lds_row; rows >= m read row m-1
@@ -203,7 +215,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 {
                     uint32_t const row = mt * 16 + c;
                     st.a[j][mt]
-                        = buffer_load_x4(act_rsrc, k_ok ? (row * (uint32_t) K + (uint32_t) kk) * 2u : kOob);
+                        = buffer_load_x4(act_rsrc, k_ok ? (row * AS + (uint32_t) kk) * 2u : kOob);
                 }
             }
         }
@@ -457,7 +469,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             lds_at = (uint32_t) row * lds_row + ch * 16u;
             sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;
             bool const ok = idx < act_chunks && (int) ch * 8 < K;
-            return ok ? ((uint32_t) row * (uint32_t) K + ch * 8u) * 2u : kOob;
+            return ok ? ((uint32_t) row * AS + ch * 8u) * 2u : kOob;
         };
         auto smooth = [&](u32x4 v, u32x4 sm)
         {
@@ -626,6 +638,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             for (int w2 = 0; w2 < WAVES; ++w2)
                 sum += red_sl[w2][s][row][cc];
             int const ocol = (strip0 + s) * 16 + cc;
+            if (p.partial)
+            {
+                p.partial[(size_t) row * p.n + ocol] = sum; // this K slice's share; the finish pass adds alpha, bias
+                continue;
+            }
             float v = p.alpha * sum;
             if (p.bias)
                 v += E::load(p.bias, ocol);
@@ -694,6 +711,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         for (int w2 = 0; w2 < WAVES; ++w2)
             sum += red[w2][slot][ln];
         int const ocol = (strip0 + s) * 16 + (ln & 15);
+        if (!ACT && p.partial)
+        {
+            p.partial[(size_t) row * p.n + ocol] = sum; // this K slice's share; the finish pass adds alpha, bias
+            continue;
+        }
         float v = p.alpha * sum;
         if (p.bias)
             v += E::load(p.bias, ocol);
@@ -711,6 +733,29 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS, int SLOTS = 1>
 __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
 {
+    if (p.k_slices > 1)
+    {
+        // K split across workgroups: this workgroup's slice becomes the whole problem
+        constexpr int TK = BITS == 4 ? 128 : 64;
+        int const y = (int) blockIdx.y;
+        int const kt0 = y * p.slice_tiles;
+        size_t const k0 = (size_t) kt0 * TK;
+        p.act = static_cast<char const*>(p.act) + k0 * 2;
+        if (PQS)
+            p.pqs = static_cast<char const*>(p.pqs) + k0 * 2;
+        p.weight = static_cast<char const*>(p.weight) + (size_t) kt0 * 1024;
+        if (GROUP != 0)
+        {
+            size_t const srow = k0 / (GROUP != 0 ? GROUP : 1) * (size_t) p.n * 2;
+            p.scales = static_cast<char const*>(p.scales) + srow;
+            if (ZERO)
+                p.zeros = static_cast<char const*>(p.zeros) + srow;
+        }
+        int const k_left = p.k_total - (int) k0;
+        p.k = k_left < p.slice_tiles * TK ? k_left : p.slice_tiles * TK;
+        p.k_tiles = (p.k + TK - 1) / TK;
+        p.partial += (size_t) y * (size_t) p.m * (size_t) p.n;
+    }
     stream_body<DT, BITS, GROUP, PQS, ZERO, MT, NS, WAVES, PF, LDS, false, SLOTS>(p);
 }
 
@@ -779,9 +824,13 @@ inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool 
 
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
-StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group);
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group,
+    int const* split_shape = nullptr);
 // WOQ_STREAM_SLOTS=0 switches the group-slot variants off (for A/B timing)
 bool stream_slots_disabled();
+// K slices (1 = none) of a streaming launch with `workspace_bytes` of scratch; WOQ_STREAM_SPLITS overrides
+// (shape[0] != 0: the launch shape that goes with the split)
+int pick_stream_k_slices(int m, int n, int k, int tile_k, int group, size_t workspace_bytes, int shape[4]);
 
 template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int MT, int NS, int WAVES, int PF, int LDS,
     bool GROUPED = false, int SLOTS = 1>
@@ -812,11 +861,21 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     }
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
-    dim3 grid(sp.groups_per_xcd * 8, GROUPED ? sp.num_experts : 1), block(WAVES * 64);
+    dim3 grid(sp.groups_per_xcd * 8, GROUPED ? sp.num_experts : sp.k_slices), block(WAVES * 64);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "stream kernel launch failed: %s", hipGetErrorString(err));
+    if (!GROUPED && sp.k_slices > 1)
+    {
+        // out = T(alpha * (slab 0 + slab 1 + ...) + bias), in slice order
+        size_t const count = (size_t) sp.m * (size_t) sp.n;
+        hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), dim3(256), 0, stream,
+            sp.out, sp.partial, sp.bias, sp.alpha, sp.m, sp.n, sp.k_slices);
+        err = hipGetLastError();
+        if (err != hipSuccess)
+            return fail(WOQ_ERR_RUNTIME, "split-K finish launch failed: %s", hipGetErrorString(err));
+    }
     return WOQ_OK;
 }
 
@@ -824,7 +883,7 @@ template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK, GROUP);
+    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK, GROUP, sp.split_shape);
     if (GROUP == 0 && sh.lds == 2)
         sh.lds = 0; // per-channel scales are applied once, in the epilogue: nothing to stage
 #define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
@@ -935,6 +994,9 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.n = p.n;
     sp.k = p.k;
     sp.k_tiles = (p.k + TK - 1) / TK;
+    sp.act_stride = p.k;
+    sp.w_strip_tiles = sp.k_tiles;
+    sp.k_total = p.k;
     sp.strips = p.n / kTileN;
     sp.groups = sp.groups_per_xcd = 0;
     sp.expert_rows = p.expert_rows;
@@ -953,6 +1015,29 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
         int rc = WOQ_OK;
         if (try_launch_stream_wide<DT, BITS>(p, sp, s, rc) && rc != WOQ_ERR_UNSUPPORTED)
             return rc;
+    }
+    if (!p.num_experts)
+    {
+        // long K and few columns: split K across workgroups (float32 slabs in the workspace + finish pass)
+        int split_shape[4];
+        int const slices = pick_stream_k_slices(p.m, p.n, p.k, TK, p.group_size, p.workspace_bytes, split_shape);
+        if (slices > 1 && p.workspace)
+        {
+            sp.slice_tiles = (sp.k_tiles + slices - 1) / slices;
+            if (p.group_size > TK) // a slice starts on a group boundary
+                sp.slice_tiles = (sp.slice_tiles + p.group_size / TK - 1) / (p.group_size / TK) * (p.group_size / TK);
+            sp.k_slices = (sp.k_tiles + sp.slice_tiles - 1) / sp.slice_tiles;
+            if (sp.k_slices > 1)
+            {
+                sp.k_tiles = sp.slice_tiles; // the largest slice: what the launch shape and the LDS areas go by
+                sp.k = sp.slice_tiles * TK;
+                sp.partial = static_cast<float*>(p.workspace);
+                for (int i = 0; i < 4; ++i)
+                    sp.split_shape[i] = split_shape[i];
+            }
+            else
+                sp.k_slices = 1;
+        }
     }
     if (p.num_experts)
     {

@@ -25,7 +25,7 @@ inline int bits_of(int quant_type)
 // Experiment overrides from the environment, read once (at first use) and again by woq_reload_env():
 //   WOQ_FORCE_REGIME=stream|gemm      WOQ_STREAM_SHAPE=ns,waves,pf,lds   WOQ_WIDE_SHAPE=ns,waves,pf | 0
 //   WOQ_STREAM_SLOTS=0                WOQ_GEMM_KERNEL=exact|skinny       WOQ_GEMM_RT=4|8|16
-//   WOQ_GEMM_SPLITS=<n>
+//   WOQ_GEMM_SPLITS=<n>               WOQ_STREAM_SPLITS=<n>
 struct EnvOverrides
 {
     int regime = 0;                // woq_regime; 0 = none
@@ -37,6 +37,7 @@ struct EnvOverrides
     int gemm_kernel = 0;           // 0 any, 1 exact-dequantize, 2 deferred-scale
     int gemm_rt = 0;               // row tiles per wavefront of the exact-dequantize / fp8 kernel
     int gemm_splits = 0;           // K split of the GEMM regime
+    int stream_splits = 0;         // K slices of the streaming kernel (0 = built-in rule)
 };
 EnvOverrides const& env_overrides();
 

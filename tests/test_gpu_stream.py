@@ -244,3 +244,39 @@ def test_wide_decode_kernel_is_what_wide_single_row_problems_run_on(pkg, oracle,
     out = run_product(pkg, oracle, dev, p, 0)
     w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")[300]
     assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()
+
+
+@pytest.mark.parametrize("splits", [2, 3, 7])
+@pytest.mark.parametrize("M,bits,group,dtype,K,N", [(16, 4, 128, "bf16", 2176, 272), (5, 4, 64, "fp16", 1408, 144),
+                                                    (9, 8, 0, "bf16", 1088, 64), (2, 4, 128, "bf16", 4096, 48),
+                                                    (1, 4, 128, "fp16", 1536, 528), (40, 8, 128, "bf16", 1024, 272)])
+def test_stream_split_k_forced(pkg, oracle, dev, woq_env, splits, M, bits, group, dtype, K, N):
+    """K split across workgroups (float32 slabs in the workspace, summed in slice order by the finish
+    pass), forced through WOQ_STREAM_SPLITS: slice counts that do not divide the tile rows, a last slice
+    that ends in half a weight tile, staged and register-held activations, the single-row group-slot
+    variant, more than 16 rows (no split: it must still be right); every optional input; the same bits
+    on every call."""
+    woq_env(WOQ_STREAM_SPLITS=splits)
+    for zero, bias, pqs in [(group != 0, True, True), (False, False, False)]:
+        p = random_problem(oracle, M, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + splits)
+        first = run_product(pkg, oracle, dev, p, STREAM)
+        assert parity_err(oracle, first, p) < TOL, (zero, bias, pqs)
+        again = run_product(pkg, oracle, dev, p, STREAM)
+        assert (again.view(np.uint32) == first.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("M,N", [(16, 272), (8, 4096), (4, 528)])
+def test_stream_split_k_by_the_built_in_rule(pkg, oracle, dev, woq_env, M, N):
+    """Long K, few columns, 4..16 rows: the rule splits K when it is given the workspace for the slabs
+    (woq_workspace_bytes asks for it) and does not without one; both are within the bar, and they
+    differ in float32 summation order."""
+    K = 8192
+    p = random_problem(oracle, M, K, N, 4, 128, "bf16", zero=True, bias=True, seed=M + N)
+    L = pkg._lib
+    assert L.lib.woq_workspace_bytes(M, N, K, L.ALGO_ZERO | L.ALGO_BIAS, L.BF16) >= 2 * M * N * 4
+    split = run_product(pkg, oracle, dev, p, STREAM)
+    assert parity_err(oracle, split, p) < TOL
+    woq_env(WOQ_STREAM_SPLITS=1)
+    plain = run_product(pkg, oracle, dev, p, STREAM)
+    assert parity_err(oracle, plain, p) < TOL
+    assert (split != plain).any()
