@@ -94,14 +94,17 @@ typedef enum woq_regime
  *   act              [m, k]            act_dtype (fp16 / bf16; fp8 e4m3 only with FP8_ALPHA)
  *   pre_quant_scale  [k]               out_dtype, required iff quant_algo & PRE_QUANT_SCALE
  *   weight           woq_preprocessed_bytes(k, n, quant_type) bytes from woq_preprocess_weights
- *   scales           [k/group_size, n] or [n] when group_size == 0 (one scale per column);
+ *   scales           [ceil(k/group_size), n] or [n] when group_size == 0 (one scale per column);
  *                    out_dtype, except W4A8 where they hold fp16 whatever out_dtype is
  *   zeros            same shape/type as scales, required iff quant_algo & ZERO
  *   bias             [n]               out_dtype, required iff quant_algo & BIAS
  *   out              [m, n]            out_dtype
  *   n                LOGICAL number of output columns (the reference plugins receive the packed
  *                    column count and multiply it back: `real_n`)
- *   group_size       0 (per-channel, the WeightOnlyQuantMatmul plugin), 64 or 128
+ *   group_size       0 (per-channel, the WeightOnlyQuantMatmul plugin), 64, 128, or - with fp16 / bf16
+ *                    activations - any larger multiple of 64 (what the reference's Hopper kernels accept,
+ *                    launchers/fpA_intB_launcher_sm90.inl:191-198); above 128 the last group may be
+ *                    shorter: scales / zeros then hold ceil(k / group_size) rows
  *   alpha            used only with FP8_ALPHA; otherwise must be 1 or is ignored as in the reference
  *   workspace        device scratch of at least woq_workspace_bytes(...) bytes (may be NULL when
  *                    that is 0)

@@ -351,8 +351,10 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
     else if (w4a8 && !(algo & WOQ_ALGO_PRE_QUANT_SCALE))
         return fail(WOQ_ERR_INVALID_ARGUMENT,
             "W4A8 with fp16/bf16 activations needs PRE_QUANT_SCALE (the smoothing pass is what casts to fp8)");
-    if (a->group_size != 0 && a->group_size != 64 && a->group_size != 128)
-        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 (per-channel), 64 or 128 (got %d)", a->group_size);
+    // 64 and 128 as the reference's kernels for every SM; larger multiples of 64 as its Hopper kernels
+    // ("The group size must a multiple of <K tile>", launchers/fpA_intB_launcher_sm90.inl:191-198)
+    if (a->group_size < 0 || a->group_size % 64)
+        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 (per-channel) or a multiple of 64 (got %d)", a->group_size);
     if (w4a8 && a->group_size != 128)
         return fail(WOQ_ERR_UNSUPPORTED, "W4A8 supports group_size 128 only (got %d)", a->group_size);
     // m == 0 is a no-op (weightOnlyQuantMatmulPlugin.cpp:303): empty tensors may carry null pointers
@@ -371,7 +373,9 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
     int const k_align = w4a8 ? 128 : 64;
     if (a->k % k_align)
         return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of %d (got %d)", k_align, a->k);
-    if (a->group_size && a->k % a->group_size)
+    // a group size above 128 may leave a shorter last group: the tables then hold ceil(k / group_size) rows
+    // (tests/quantization/test_weight_only_groupwise_quant_matmul.py:155, 405-420)
+    if (a->group_size && a->group_size <= 128 && a->k % a->group_size)
         return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of group_size (got %d, %d)", a->k, a->group_size);
     if (a->n % kTileN)
         return fail(WOQ_ERR_BAD_SHAPE, "n must be a multiple of %d (got %d)", kTileN, a->n);
@@ -383,7 +387,8 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
         uint64_t const limit = (uint64_t) 1 << 31;
         uint64_t const act_bytes = (uint64_t) a->m * a->k * (a->act_dtype == WOQ_FP8_E4M3 ? 1 : 2);
         uint64_t const weight_bytes = (uint64_t) a->k * a->n * ((algo & WOQ_ALGO_INT8_WEIGHT) ? 2 : 1) / 2;
-        uint64_t const scale_bytes = (uint64_t) (a->group_size ? a->k / a->group_size : 1) * a->n * 2;
+        uint64_t const scale_bytes
+            = (uint64_t) (a->group_size ? (a->k + a->group_size - 1) / a->group_size : 1) * a->n * 2;
         if (act_bytes >= limit || weight_bytes >= limit || scale_bytes >= limit)
             return fail(WOQ_ERR_UNSUPPORTED,
                 "operand too large: activations, one weight matrix and its scales must each stay below 2 GiB "
@@ -744,7 +749,7 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     if (p.m == 0)
         return WOQ_OK;
     p.weight_stride = woq_preprocessed_bytes(p.k, p.n, p.bits == 8 ? WOQ_W8_A16 : WOQ_W4_A16);
-    p.scale_stride = (size_t) (p.group_size ? p.k / p.group_size : 1) * (size_t) p.n * 2;
+    p.scale_stride = (size_t) (p.group_size ? (p.k + p.group_size - 1) / p.group_size : 1) * (size_t) p.n * 2;
     int const act = args->activation;
     bool const gated = act == WOQ_ACT_SWIGLU || act == WOQ_ACT_GEGLU;
     // without the prefix sums (one expert owning every row) the kernels take the row count from m
@@ -814,9 +819,9 @@ extern "C" int woq_dequantize(void* out, const void* weight, const void* scales,
         return fail(WOQ_ERR_INVALID_ARGUMENT, "dtype must be fp16, bf16 or fp8 e4m3");
     if (k <= 0 || n <= 0 || n % kTileN || k % 32)
         return fail(WOQ_ERR_BAD_SHAPE, "k %% 32 == 0 and n %% 16 == 0 required (got %d, %d)", k, n);
-    if (group_size != 0 && group_size != 64 && group_size != 128)
-        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0, 64 or 128 (got %d)", group_size);
-    if (group_size && k % group_size)
+    if (group_size < 0 || group_size % 64)
+        return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 or a multiple of 64 (got %d)", group_size);
+    if (group_size && group_size <= 128 && k % group_size)
         return fail(WOQ_ERR_BAD_SHAPE, "k must be a multiple of group_size");
     return launch_dequant(out, weight, scales, zeros, k, n, group_size, bits_of(quant_type), dtype, stream);
 }

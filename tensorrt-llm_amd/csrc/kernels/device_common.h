@@ -266,6 +266,39 @@ __device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc,
     return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int) byte_offset, 0, 0);
 }
 
+// ---- row of the scale / zero tables -----------------------------------------------------------------
+// The GROUP = 64 instantiations also serve every larger multiple of 64 ("flexible" group sizes, what
+// the reference's Hopper kernels accept): scales are then applied per 64 rows of K and only the row
+// of the [ceil(k / group), n] tables follows the real group size.  `magic` = ceil(2^32 / (group / 64))
+// for such a group (an exact division by multiplication for every row index that can occur), 0 for a
+// real group of 64.
+template <int GROUP>
+__device__ __forceinline__ uint32_t scale_row(uint32_t k_row, uint32_t magic)
+{
+    if constexpr (GROUP == 64)
+    {
+        uint32_t const seg = k_row >> 6;
+        return magic ? __umulhi(seg, magic) : seg;
+    }
+    else
+        return k_row / (uint32_t) (GROUP != 0 ? GROUP : 1);
+}
+
+// host side: the magic of a group size (0 unless it is a multiple of 64 above 128)
+inline uint32_t scale_row_magic(int group_size)
+{
+    if (group_size <= 128 || group_size % 64)
+        return 0;
+    uint64_t const d = (uint64_t) group_size / 64;
+    return (uint32_t) ((((uint64_t) 1 << 32) + d - 1) / d);
+}
+
+// the kernel instantiation that serves a group size: 0 / 64 / 128 themselves, 64 for larger multiples of 64
+inline int template_group(int group_size)
+{
+    return group_size <= 128 ? group_size : 64;
+}
+
 // ---- epilogue activations (values of the reference's ActivationType,
 // kernels/internal_cutlass_kernels/include/moe_gemm_kernels.h:197-206) -------------------------
 constexpr int kActGelu = 0, kActRelu = 1, kActSilu = 2, kActSwiglu = 3, kActGeglu = 4, kActIdentity = 5;

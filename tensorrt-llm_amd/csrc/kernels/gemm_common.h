@@ -19,6 +19,8 @@ struct GemmParams
     int m, n, k;
     int k_tiles; // ceil(k / TILE_K)
     int strips;  // n / 16
+    int scale_rows = 1;       // rows of the scale / zero tables: ceil(k / group_size)
+    uint32_t group_magic = 0; // see scale_row()
     int tiles_m, tiles_n;
     int k_splits;        // workgroups along K per output tile (blockIdx.y)
     int tiles_per_split; // tile rows of K each of them covers
@@ -52,6 +54,8 @@ __device__ __forceinline__ int paired_strip(bool gated, int first, int s, int st
 
 inline void set_group_fields(GemmParams& gp, MatmulProblem const& p, int tile_rows)
 {
+    gp.scale_rows = p.group_size ? (p.k + p.group_size - 1) / p.group_size : 1;
+    gp.group_magic = scale_row_magic(p.group_size);
     gp.activation = act_is_gated(p.activation) ? p.activation : kActIdentity;
     // behind a non-gated activation the residual is added by the activation pass, not here
     gp.residual = (p.activation == kActIdentity || act_is_gated(p.activation)) ? p.residual : nullptr;

@@ -82,8 +82,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     constexpr uint32_t kOob = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
-    uint32_t const sz_bytes
-        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes = (uint32_t) p.scale_rows * (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
@@ -187,7 +186,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         else if constexpr (GROUP != 0)
         {
             int const q = i - NS, which = q / (NS * SEGS), seg = (q / NS) % SEGS, s = q % NS;
-            uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+            uint32_t const grow = scale_row<GROUP>((uint32_t) (kt * TK + seg * SEG), p.group_magic);
             uint32_t const off = (grow * (uint32_t) p.n * 2u + sc_lane[s]) | past;
             if (which == 0)
                 st.s[s][seg] = buffer_load_u16(sc_rsrc, off);
@@ -583,7 +582,7 @@ int launch_gemm_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream
     set_group_fields(gp, p, plan.rt * 16);
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
-    switch (p.group_size)
+    switch (template_group(p.group_size))
     {
     case 0: return launch_gemm_rt<DT, BITS, 0, false>(gp, plan.rt, s);
     case 64:

@@ -93,8 +93,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
 
     constexpr uint32_t kOob = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
-    uint32_t const sz_bytes
-        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes = (uint32_t) p.scale_rows * (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
@@ -178,7 +177,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
             {
-                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+                uint32_t const grow = scale_row<GROUP>((uint32_t) (kt * TK + seg * SEG), p.group_magic);
                 uint32_t const off = ((grow * (uint32_t) p.n + sc_lane_col) * 2u) | past | sc_lane_oob;
                 char* slot = reinterpret_cast<char*>(stage_sc[buf]->sc[wave]) + seg * (ZERO ? 512 : 256);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -600,7 +599,7 @@ int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stre
     set_group_fields(gp, p, rt * 16);
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
-    switch (p.group_size)
+    switch (template_group(p.group_size))
     {
     case 0: return launch_skinny_variant<DT, BITS, 0, false>(gp, rt, s);
     case 64:

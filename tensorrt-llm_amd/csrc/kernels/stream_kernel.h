@@ -48,8 +48,11 @@ struct StreamParams
     // slab blockIdx.y of `partial` ([k_slices][m][n]) for the finish pass to add up in slice order.
     int k_slices = 1, slice_tiles = 0, k_total = 0;
     float* partial = nullptr;
+    int real_group = 0; // host side: the problem's group size
     int split_shape[4] = {0, 0, 0, 0}; // host side: the launch shape chosen with the K split (ns, waves, pf, lds)
     int strips;         // n / 16
+    int scale_rows = 1;       // rows of the scale / zero tables: ceil(k / group_size)
+    uint32_t group_magic = 0; // see scale_row()
     int groups;         // ceil(strips / NS): column groups, one workgroup each
     int groups_per_xcd; // ceil(groups / 8)
     // grouped problems (rows sorted by expert, expert_rows[e] = rows of experts 0..e, device
@@ -149,8 +152,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     constexpr uint32_t kOob = 0x7FFFFFF0u;
     auto const act_rsrc = make_rsrc(p.act, ((uint32_t) (p.m - 1) * AS + (uint32_t) K) * 2u);
     auto const pqs_rsrc = make_rsrc(PQS ? p.pqs : p.act, (uint32_t) K * 2u);
-    uint32_t const sz_bytes
-        = GROUP != 0 ? (uint32_t) (K / (GROUP != 0 ? GROUP : 1)) * (uint32_t) p.n * 2u : (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes = (uint32_t) p.scale_rows * (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     // weights too go through a descriptor: a prefetch past the last tile row is given an
@@ -184,7 +186,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
     // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
     int const act_rows = ALDS ? (p.m < 16 ? p.m : 16) : 0;
-    int const sc_rows = SCLDS ? (KT * TK + (GROUP ? GROUP : 1) - 1) / (GROUP ? GROUP : 1) : 0;
+    int const sc_rows = SCLDS ? (int) scale_row<GROUP>((uint32_t) (KT * TK - 1), p.group_magic) + 1 : 0;
     constexpr uint32_t SC_ROW = NS * 32u;
     char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
     char* const zr_lds = sc_lds + (uint32_t) sc_rows * SC_ROW;
@@ -224,7 +226,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
             {
-                uint32_t const grow = (uint32_t) ((kt * TK + seg * SEG) / GROUP);
+                uint32_t const grow = scale_row<GROUP>((uint32_t) (kt * TK + seg * SEG), p.group_magic);
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                 {
@@ -252,7 +254,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 int const it_i = gi / SEGS, seg_i = gi % SEGS;
                 bool const ok = it_i < n_my;
                 int const kt_i = wave + it_i * WAVES;
-                uint32_t const grow = (uint32_t) ((kt_i * TK + seg_i * SEG) / GROUP);
+                uint32_t const grow = scale_row<GROUP>((uint32_t) (kt_i * TK + seg_i * SEG), p.group_magic);
                 char const* sp = ok ? sc_lds + grow * SC_ROW + (uint32_t) c * 2u : zero_lds;
                 char const* zp = ok ? zr_lds + grow * SC_ROW + (uint32_t) c * 2u : zero_lds;
                 float const S = *reinterpret_cast<float const*>(
@@ -346,7 +348,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                         if constexpr (SCLDS)
                         {
                             uint32_t const at
-                                = (uint32_t) ((kt * TK + seg * SEG) / (GROUP ? GROUP : 1)) * SC_ROW + (s * 16 + c) * 2u;
+                                = scale_row<GROUP>((uint32_t) (kt * TK + seg * SEG), p.group_magic) * SC_ROW + (s * 16 + c) * 2u;
                             s_raw = *reinterpret_cast<uint16_t const*>(sc_lds + at);
                             if constexpr (ZERO)
                                 z_raw = *reinterpret_cast<uint16_t const*>(zr_lds + at);
@@ -751,6 +753,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_kernel(StreamParams p)
             if (ZERO)
                 p.zeros = static_cast<char const*>(p.zeros) + srow;
         }
+        if (GROUP != 0)
+            p.scale_rows -= (int) (k0 / (GROUP != 0 ? GROUP : 1));
         int const k_left = p.k_total - (int) k0;
         p.k = k_left < p.slice_tiles * TK ? k_left : p.slice_tiles * TK;
         p.k_tiles = (p.k + TK - 1) / TK;
@@ -813,13 +817,14 @@ inline size_t stream_act_lds_bytes(int m, int k, int tile_k)
 
 // bytes of LDS the staged group scales (and zeros) of ns strips and, with sums, the activation row
 // sums take
-inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int ns, bool zeros, bool sums)
+// (`group`: the kernel instantiation's, `real_group`: the problem's - they differ for flexible groups)
+inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int real_group, int ns, bool zeros, bool sums)
 {
     if (group == 0)
         return 0;
     size_t const k_padded = (size_t) ((k + tile_k - 1) / tile_k) * tile_k;
     size_t const seg = group > tile_k ? tile_k : group; // rows of K per activation row sum
-    return (k_padded + group - 1) / group * (size_t) ns * 32 * (zeros ? 2 : 1) + (sums ? k_padded / seg * 64 : 0);
+    return (k_padded + real_group - 1) / real_group * (size_t) ns * 32 * (zeros ? 2 : 1) + (sums ? k_padded / seg * 64 : 0);
 }
 
 
@@ -846,7 +851,7 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     size_t lds = 0;
     if constexpr (LDS != 0)
     {
-        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, NS, ZERO, LDS == 1)
+        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, sp.real_group, NS, ZERO, LDS == 1)
             + (SLOTS > 1 ? 256 : 0); // group slots: a block of zeros behind the staged operands
         // the reduction buffer of the epilogue is static LDS of this variant and shares the CU's 160 KiB
         constexpr size_t kStaticLds = (size_t) WAVES * NS * MT * 4 * 64 * sizeof(float);
@@ -997,6 +1002,9 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     sp.act_stride = p.k;
     sp.w_strip_tiles = sp.k_tiles;
     sp.k_total = p.k;
+    sp.scale_rows = p.group_size ? (p.k + p.group_size - 1) / p.group_size : 1;
+    sp.group_magic = scale_row_magic(p.group_size);
+    sp.real_group = p.group_size;
     sp.strips = p.n / kTileN;
     sp.groups = sp.groups_per_xcd = 0;
     sp.expert_rows = p.expert_rows;
@@ -1016,7 +1024,7 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
         if (try_launch_stream_wide<DT, BITS>(p, sp, s, rc) && rc != WOQ_ERR_UNSUPPORTED)
             return rc;
     }
-    if (!p.num_experts)
+    if (!p.num_experts && p.group_size <= 128)
     {
         // long K and few columns: split K across workgroups (float32 slabs in the workspace + finish pass)
         int split_shape[4];
@@ -1041,7 +1049,7 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     }
     if (p.num_experts)
     {
-        switch (p.group_size)
+        switch (template_group(p.group_size))
         {
         case 0: return launch_stream_grouped<DT, BITS, 0, false>(sp, s);
         case 64:
@@ -1060,7 +1068,7 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
                     : launch_stream_shaped<DT, BITS, G, true, false>(sp, mt, s);                                       \
     return zero ? launch_stream_shaped<DT, BITS, G, false, true>(sp, mt, s)                                            \
                 : launch_stream_shaped<DT, BITS, G, false, false>(sp, mt, s);
-    switch (p.group_size)
+    switch (template_group(p.group_size))
     {
     case 0:
         if (pqs)

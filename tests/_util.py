@@ -17,7 +17,7 @@ def random_problem(oracle, M, K, N, bits, group, dtype, zero=False, bias=False, 
     rng = np.random.default_rng(seed)
     lo = -(1 << (bits - 1))
     q = rng.integers(lo, -lo, size=(K, N)).astype(np.int8)
-    gshape = (K // group, N) if group else (N,)
+    gshape = (-(-K // group), N) if group else (N,)  # a group size above 128 may leave a shorter last group
     scales = oracle.round_to(rng.uniform(0.002, 0.02, gshape).astype(np.float32) * (16.0 / (1 << bits)), dtype)
     p = dict(q=q, scales=scales, zeros=None, bias=None, pqs=None, bits=bits, group=group, dtype=dtype, M=M, K=K, N=N)
     if zero:

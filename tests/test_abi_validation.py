@@ -27,6 +27,9 @@ def test_valid_combinations(pkg):
     assert status(pkg)[0] == 0
     assert status(pkg, zeros=0x5000, quant_algo=L.ALGO_ZERO)[0] == 0
     assert status(pkg, bias=0x5000, quant_algo=L.ALGO_BIAS, group_size=64)[0] == 0
+    # multiples of 64 above 128 (the reference's Hopper kernels), also with a shorter last group
+    assert status(pkg, k=768, group_size=192)[0] == 0
+    assert status(pkg, k=512, group_size=320)[0] == 0
     assert status(pkg, pre_quant_scale=0x5000, quant_algo=L.ALGO_PRE_QUANT_SCALE)[0] == 0
     assert status(pkg, group_size=0, quant_algo=L.ALGO_INT8_WEIGHT, act_dtype=L.FP16, out_dtype=L.FP16)[0] == 0
     assert status(pkg, m=0)[0] == 0                                     # m == 0 is a no-op, not an error
@@ -37,6 +40,8 @@ def test_valid_combinations(pkg):
     (dict(scales=None), -1, "scales"),
     (dict(act=None), -1, "NULL"),
     (dict(group_size=32), -3, "group_size"),
+    (dict(group_size=96), -3, "multiple of 64"),
+    (dict(quant_algo=8, act_dtype=2, group_size=256), -3, "128"),
     (dict(k=96), -2, "multiple of 64"),
     (dict(k=576, group_size=128), -2, "group_size"),
     (dict(n=250), -2, "multiple of 16"),

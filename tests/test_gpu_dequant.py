@@ -11,15 +11,15 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("group", [0, 64, 128])
+@pytest.mark.parametrize("group", [0, 64, 128, 192, 256])
 @pytest.mark.parametrize("zero", [False, True])
 def test_dequantize_bit_exact(pkg, oracle, dev, dtype, bits, group, zero):
     K, N = 320, 96
-    if group and K % group:
-        K = 384
+    if 0 < group <= 128 and K % group:
+        K = 384  # (groups above 128 may end in a shorter group: 320 = 192 + 128 = 256 + 64)
     rng = np.random.default_rng(bits * 100 + group + zero)
     q = rng.integers(-(1 << (bits - 1)), 1 << (bits - 1), size=(K, N)).astype(np.int8)
-    gshape = (K // group, N) if group else (N,)
+    gshape = (-(-K // group), N) if group else (N,)
     s = oracle.round_to(np.exp(rng.uniform(-8, 1, gshape)).astype(np.float32), dtype)
     z = oracle.round_to((rng.standard_normal(gshape) * np.exp(rng.uniform(-8, 1, gshape))).astype(np.float32),
                         dtype) if zero and group else None

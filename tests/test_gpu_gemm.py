@@ -143,3 +143,22 @@ def test_gemm_split_k_is_bit_reproducible(pkg, oracle, dev, woq_env, bits, group
         for _ in range(3):
             again = run_product(pkg, oracle, dev, p, GEMM)
             assert (again.view(np.uint32) == first.view(np.uint32)).all(), splits
+
+
+# the reference's own grid for group sizes beyond 128 (m, n, k, dtype, pre-quant scale, zeros, bias, group:
+# tests/quantization/test_weight_only_groupwise_quant_matmul.py:405-420, its Hopper-only
+# test_hopper_flexible_groups) plus a longer K; k = 256 with groups of 192 leaves a last group of 64 rows
+FLEXIBLE = [(32, 1024, 256, "fp16", True, True, False, 192), (32, 2048, 384, "bf16", True, False, True, 256),
+            (64, 2048, 1024, "fp16", True, False, False, 320), (200, 528, 1536, "bf16", False, True, True, 192),
+            (96, 272, 4096, "bf16", True, True, True, 256)]
+
+
+@pytest.mark.parametrize("m,n,k,dtype,pqs,zero,bias,group", FLEXIBLE)
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gemm_flexible_group_sizes(pkg, oracle, dev, m, n, k, dtype, pqs, zero, bias, group, bits):
+    """Group sizes that are multiples of 64 above 128, on either GEMM kernel (the fixture's), int4 and
+    int8, split K included (k = 4096 at 96 rows)."""
+    p = random_problem(oracle, m, k, n, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=group + m)
+    assert p["scales"].shape[0] == -(-k // group)
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
+    assert err < TOL, err

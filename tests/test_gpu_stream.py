@@ -280,3 +280,17 @@ def test_stream_split_k_by_the_built_in_rule(pkg, oracle, dev, woq_env, M, N):
     plain = run_product(pkg, oracle, dev, p, STREAM)
     assert parity_err(oracle, plain, p) < TOL
     assert (split != plain).any()
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 40])
+@pytest.mark.parametrize("bits,group,dtype,K,N", [(4, 192, "fp16", 256, 1024), (4, 256, "bf16", 384, 2048),
+                                                  (4, 320, "fp16", 1024, 528), (8, 192, "bf16", 1088, 272),
+                                                  (4, 256, "bf16", 4160, 144)])
+def test_stream_flexible_group_sizes(pkg, oracle, dev, M, bits, group, dtype, K, N):
+    """Group sizes that are multiples of 64 above 128 (the reference's Hopper kernels take them) on the
+    streaming kernels: staged and register-held activations, the single-row group-slot variant, a last
+    group that is shorter than the others, K that ends in half a weight tile."""
+    for zero, bias, pqs in [(True, True, True), (False, False, False)]:
+        p = random_problem(oracle, M, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=group + M)
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+        assert err < TOL, (zero, bias, pqs, err)
