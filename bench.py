@@ -36,10 +36,30 @@ HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0
 CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# calibrated with a 256 MiB copy (profiles/stream_gemv_gate_up_m1_hbm_traffic.md); counters cannot
-# be read from inside this process, so the figure is the recorded one
-DOMINANT_TRAFFIC_BYTES = 62_640_000
+TRAFFIC_PROFILE = "profiles/stream_gemv_gate_up_m1_hbm_traffic.md"
+
+
+def recorded_traffic_bytes():
+    """HBM bytes per launch of the dominant kernel as the tracked rocprofv3 --pmc summary records them
+    (FETCH_SIZE / WRITE_SIZE runs calibrated with a 256 MiB copy; the line `traffic_bytes_per_launch: N`
+    of TRAFFIC_PROFILE).  Counters cannot be read from inside this process; None when the summary is
+    missing or does not name the kernel this library now launches for the shape."""
+    import os
+    import re
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
+    k = re.search(r"^kernel:\s*(\S+)", text, re.M)
+    if not m or not k or k.group(1) != DOMINANT_KERNEL:
+        return None
+    return int(m.group(1))
+
+
+# the kernel the library launches for gate_up at M = 1 (named in the rocprof summaries)
+DOMINANT_KERNEL = "stream_wide_kernel<1,4,128,false,true,2,4,4,16>"
 
 
 def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
@@ -183,8 +203,10 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
 
 
 def bench_cpu_baseline(layers, acts, m=1, budget_s=15.0):
-    """The reference's CPU path (tensorrt_llm/quantization/functional.py:269-290 semantics):
-    dequantize with torch, then a float32 matmul, on the host cores."""
+    """The reference's CPU path (tensorrt_llm/quantization/functional.py:269-290 semantics) on the host
+    cores, two timings: (i) dequantize with torch, then a float32 matmul - `value`; (ii) the float32
+    matmul alone on weights dequantized beforehand - `matmul_only`.  Both in the metric's unit, i.e.
+    the step's algorithmic bytes (of the QUANTIZED operands) per second."""
     from __graft_entry__ import import_oracle
     o = import_oracle()
     host = []
@@ -192,18 +214,30 @@ def bench_cpu_baseline(layers, acts, m=1, budget_s=15.0):
         l = layers[i][0]
         host.append((acts[k].float().cpu(), l["q"].cpu(), l["scales"].float().cpu(), l["zeros"].float().cpu()))
     per_step_bytes = sum(algorithmic_bytes(m, k, n) for _, k, n in SHAPES_8B)
-    times = []
-    t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
-        t0 = time.perf_counter()
-        for a, q, s, z in host:
-            o.torch_cpu_dequant_matmul(a, q, s, z, GROUP)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+
+    def median_time(fn, budget, most):
+        times = []
+        t_start = time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_start < budget and len(times) < most):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    med, passes = median_time(lambda: [o.torch_cpu_dequant_matmul(a, q, s, z, GROUP) for a, q, s, z in host],
+                              budget_s, 20)
+    # (ii): weights dequantized once, outside the timed region
+    dense = []
+    for a, q, s, z in host:
+        w = q.to(torch.float32) * s.repeat_interleave(GROUP, dim=0) + z.repeat_interleave(GROUP, dim=0)
+        dense.append((a, w))
+    med_mm, passes_mm = median_time(lambda: [a @ w for a, w in dense], budget_s / 3, 40)
     return dict(value=round(per_step_bytes / med / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
-                sample="%d passes over the same 4-matmul step (torch dequant + fp32 matmul), median %.1f ms"
-                       % (len(times), med * 1e3))
+                matmul_only=round(per_step_bytes / med_mm / 1e9, 3),
+                sample="%d passes over the same 4-matmul step (torch dequant + fp32 matmul), median %.1f ms; "
+                       "%d passes of the fp32 matmuls alone on pre-dequantized weights, median %.1f ms"
+                       % (passes, med * 1e3, passes_mm, med_mm * 1e3))
 
 
 def bench_gemm(pkg, dev, m=4096, reps=40):
@@ -231,7 +265,12 @@ def bench_gemm(pkg, dev, m=4096, reps=40):
         lib_tf = 2.0 * m * n * k / (lib_sec / reps) / 1e12
         return dict(shape=name, m=m, us=round(sec * 1e6, 1), tflops=round(tf, 1),
                     frac_of_bf16_peak=round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                    library_dense_bf16_gemm_tflops=round(lib_tf, 1))
+                    library_dense_bf16_gemm_tflops=round(lib_tf, 1),
+                    # the M = 4096 half of the metric in the shape of `roofline`
+                    roofline={"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                              "kernel": "gemm_kernel<bf16,int4,g128,zeros,RT=16> on gate_up K=%d N=%d M=%d" % (k, n, m),
+                              "flop_per_launch": 2.0 * m * n * k, "us_per_launch": round(sec * 1e6, 1)})
     except Exception as e:  # the decode line is still valid without the prefill extra
         return dict(error=str(e)[:200])
 
@@ -343,7 +382,7 @@ def run_for_counters(pkg, dev, mode, reps=20):
     for r in range(reps):
         launch(pkg, act, layers[r % copies], out)
     torch.cuda.synchronize()
-    print(json.dumps({"mode": "dominant", "kernel": "stream_kernel on gate_up K=4096 N=28672 M=1",
+    print(json.dumps({"mode": "dominant", "kernel": DOMINANT_KERNEL + " on gate_up K=4096 N=28672 M=1",
                       "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n), "launches": reps}))
 
 
@@ -456,6 +495,61 @@ def run_moe_sweep(pkg, dev):
         torch.cuda.empty_cache()
 
 
+def run_ceilings(pkg, dev):
+    """What the hardware allows, with this file's own timing (HIP graph replays, buffers rotating through
+    1 GiB so that nothing is served from the last-level cache): plain streaming reads at the byte counts
+    of the benchmark's GEMVs, an empty launch, and matrix-instruction-only kernels.  One JSON line."""
+    import ctypes
+    lib = pkg._lib.lib
+    stream_of = lambda: ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    pool = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(4096, dtype=torch.uint8, device=dev)
+    out = {"mode": "ceilings", "reads": [], "hbm_peak_gbs": HBM_PEAK_GBS}
+    # algorithmic bytes of the M = 1 GEMVs: 8B o_proj, qkv, down, gate_up, 70B gate_up (rounded to 64 KiB)
+    for label, nbytes in [("8b_o_proj 8.9 MB", 8929280), ("8b_qkv 13.4 MB", 13389824), ("8b_down 31.2 MB", 31232000),
+                          ("8b_gate_up 62.5 MB", 62455808), ("70b_gate_up 250 MB", 250478592)]:
+        nbytes = nbytes // 65536 * 65536
+        copies = (1 << 30) // nbytes
+        best = None
+        for kib, u in [(4, 4), (8, 8), (16, 8), (32, 4), (64, 8)]:
+            def body(reps=40):
+                for r in range(reps):
+                    pkg._lib.check(lib.woq_probe_read(ctypes.c_void_p(pool.data_ptr() + (r % copies) * nbytes), nbytes, kib, u,
+                                                      ctypes.c_void_p(sink.data_ptr()), stream_of()))
+            body(3)
+            torch.cuda.synchronize()
+            _, sec, launches = time_graph(body, 40, repeats=3)
+            us = sec / launches * 1e6
+            if best is None or us < best[0]:
+                best = (us, kib, u)
+        out["reads"].append({"like": label, "bytes": nbytes, "us": round(best[0], 2), "gbs": round(nbytes / best[0] / 1e3, 1),
+                             "frac_of_peak": round(nbytes / best[0] / 1e3 / HBM_PEAK_GBS, 4),
+                             "kib_per_wave": best[1], "loads_in_flight": best[2]})
+
+    def empty(reps=200):
+        for _ in range(reps):
+            pkg._lib.check(lib.woq_probe_empty(ctypes.c_void_p(sink.data_ptr()), stream_of()))
+    empty(5)
+    torch.cuda.synchronize()
+    _, sec, launches = time_graph(empty, 200, repeats=3)
+    out["empty_launch_us"] = round(sec / launches * 1e6, 3)
+    for kind, name, peak in [(0, "v_mfma_f32_16x16x32_bf16", MFMA_BF16_PEAK_TFLOPS),
+                             (1, "v_mfma_f32_16x16x128_f8f6f4 (e4m3)", MFMA_FP8_PEAK_TFLOPS)]:
+        flop = [0.0]
+
+        def body(reps=4):
+            for _ in range(reps):
+                flop[0] = lib.woq_probe_mfma(kind, 20000, 256, ctypes.c_void_p(sink.data_ptr()), stream_of())
+        body(1)
+        torch.cuda.synchronize()
+        _, sec, launches = time_graph(body, 4, repeats=3)
+        tf = flop[0] / (sec / launches) / 1e12
+        out.setdefault("mfma", []).append({"instruction": name, "tflops": round(tf, 1), "peak": peak,
+                                           "frac_of_peak": round(tf / peak, 4),
+                                           "ms_per_launch": round(sec / launches * 1e3, 3)})
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -464,7 +558,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
     ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "w4a8_decode", "moe_decode",
-                                       "sweep"],
+                                       "sweep", "ceilings"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
@@ -486,6 +580,9 @@ def main():
         else:
             run_sweep(pkg, dev, args.sweep, args.tuned)
         return
+    if args.mode == "ceilings":
+        run_ceilings(pkg, dev)
+        return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode)
         return
@@ -501,8 +598,9 @@ def main():
                                "bf16 scales+zeros, decode GEMV M=1; %d rotating weight copies" % r["copies"],
                    "m": 1, "group_size": GROUP, "weight_bits": 4},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": DOMINANT_TRAFFIC_BYTES,
-                     "kernel": "stream_kernel<bf16,int4,g128,MT=1> on gate_up K=4096 N=28672",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic_bytes(),
+                     "traffic_source": TRAFFIC_PROFILE,
+                     "kernel": DOMINANT_KERNEL + " on gate_up K=4096 N=28672",
                      "bytes_per_launch": r["dom_bytes"], "us_per_launch": round(r["dom_dur"] * 1e6, 3)},
         "per_shape": r["per_shape"],
         "event_ms_per_step": round(r["ev_s"] / args.steps * 1e3, 5),

@@ -319,6 +319,19 @@ int woq_rmsnorm_prequant(void* out, const void* x, const void* gamma, const void
 int woq_dequantize(void* out, const void* weight, const void* scales, const void* zeros, int32_t k, int32_t n,
     int32_t group_size, int32_t quant_type, int32_t dtype, void* stream);
 
+/* ---- measurement probes (no counterpart in the reference) -------------------------------------- */
+
+/* What the hardware allows, measured with the same harness as the kernels (bench.py --mode ceilings).
+ * woq_probe_read: a plain streaming read of `bytes` of device memory (every wavefront reads
+ * kib_per_wave contiguous KiB, loads_in_flight of 1, 2, 4 or 8 16-byte loads per lane outstanding);
+ * `sink` is 4 KiB of device memory.  woq_probe_empty: a kernel that does nothing.  woq_probe_mfma:
+ * nothing but matrix instructions (kind 0: v_mfma_f32_16x16x32_bf16, 1: v_mfma_f32_16x16x128_f8f6f4
+ * on e4m3) on `workgroups` x 4 wavefronts; returns the floating-point operations of the launch
+ * (negative on a bad argument). */
+int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream);
+int woq_probe_empty(void* sink, void* stream);
+double woq_probe_mfma(int kind, int iters, int workgroups, void* sink, void* stream);
+
 /* ---- misc ------------------------------------------------------------------------------------ */
 
 /* The WOQ_* environment variables (experiment overrides of the built-in kernel choices) are read

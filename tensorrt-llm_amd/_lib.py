@@ -84,6 +84,9 @@ def _load():
         "woq_describe_tactic": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_char_p, sz]),
         "woq_export_tactics": (sz, [ctypes.c_char_p, sz]),
         "woq_import_tactics": (ctypes.c_int, [ctypes.c_char_p]),
+        "woq_probe_read": (ctypes.c_int, [vp, sz, i32, i32, vp, vp]),
+        "woq_probe_empty": (ctypes.c_int, [vp, vp]),
+        "woq_probe_mfma": (ctypes.c_double, [i32, i32, i32, vp, vp]),
         "woq_reload_env": (None, []),
         "woq_last_error": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),

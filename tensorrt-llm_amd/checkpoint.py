@@ -12,11 +12,30 @@ calls per tensor.  Same arithmetic, same argument conventions:
   * the op takes signed weights q = u - 8 (u - 128) and ADDITIVE, pre-scaled zeros
     `zero = (8 - qzero - [GPTQ]) * scale` (128 for int8), functional.py:1010-1014.
 
+  * ModelOpt AWQ (the reference's own quantizer): `weight` int8 [N/2, K] (two output channels per
+    byte, signed nibbles), `weight_scale` [N, K/g], `input_quantizer._pre_quant_scale` [K]; for W4A8
+    also the per-tensor `activation_scaling_factor` and `weights_scaling_factor_2`, folded by the
+    loader (tensorrt_llm/models/modeling_utils.py:1626-1682): `postprocess_modelopt_awq`, `fold_w4a8`.
+  * q / k / v (or gate / up) tensors that arrive separately are concatenated along N first
+    (functional.py:932-944): `concat_gptq_parts`, and list arguments of `postprocess_modelopt_awq`.
+
 Returned tensors are what `weight_only_groupwise_quant_matmul` takes: `weight` in this library's
 gfx950 layout (opaque bytes), `weights_scaling_factor` [K/g, N] and `zero` [K/g, N] in `dtype`.
 All tensors are CPU tensors, as in the reference's loader.
+
+`load_trtllm_linear` reads one linear layer of a TensorRT-LLM checkpoint (`rank<r>.safetensors` +
+`config.json`, docs/source/architecture/checkpoint.md:94-176; tensor names of
+quantization/layers.py:744-751, 998-1037) whose `weight` was already laid out by the reference's
+preprocess for some SM, decodes that layout and re-lays it out for gfx950.
+
+The three small helpers `unpack_int32_into_int8`, `change_qkv_leading_dim` and `pad_like` follow the
+reference's helpers of the same names closely (functional.py:833-872): each has one obvious
+implementation, and the loaders above call them with the reference's argument conventions.
 """
 from __future__ import annotations
+
+import json
+import os
 
 import torch
 
@@ -127,3 +146,196 @@ def postprocess_autoawq(qweight: torch.Tensor, scales: torch.Tensor, qzeros: tor
     q_signed = unpack_int32_into_int8(qweight, True) - 8  # functional.py:948-949
     qz = unpack_int32_into_int8(qzeros, True)
     return _finish(q_signed.contiguous(), scales, qz, 4, False, dtype, tp_split, padded_shape, num_heads)
+
+
+def concat_gptq_parts(parts):
+    """[(qweight, scales, qzeros), ...] of layers that share their input (q, k, v or gate, up) -> one
+    (qweight, scales, qzeros) with the output columns side by side.  All three GPTQ / AutoAWQ tensors
+    keep N (or N/8) in their last dimension, so this is a concatenation along it
+    (functional.py:939-943: `torch.cat(weights[i::len(weights) // 3], dim=1)`)."""
+    return tuple(torch.cat([p[i] for p in parts], dim=1) for i in range(3))
+
+
+def fold_w4a8(weights_scaling_factor: torch.Tensor, prequant_scaling_factor: torch.Tensor,
+              activation_scaling_factor: torch.Tensor, weights_scaling_factor_2: torch.Tensor):
+    """The W4A8 loader fold (tensorrt_llm/models/modeling_utils.py:1661-1682), in its order of
+    operations: the group scales are divided by the per-tensor weight scale in their own type and then
+    stored as float16 (the fp8 kernels read half scales whatever the activation type:
+    weightOnlyGroupwiseQuantMatmulPlugin.cpp:254); the smoothing vector is divided by the per-tensor
+    activation scale (so that smoothed activations land in the e4m3 range); alpha = their product
+    restores the magnitude in the epilogue.  Returns the four tensors under the reference's names."""
+    act_sf = torch.as_tensor(activation_scaling_factor)
+    wsf2 = torch.as_tensor(weights_scaling_factor_2)
+    return {
+        "weights_scaling_factor": (weights_scaling_factor / wsf2).to(torch.float16).contiguous(),
+        "prequant_scaling_factor": (prequant_scaling_factor / act_sf).contiguous(),
+        "alpha": (act_sf.to(torch.float32) * wsf2.to(torch.float32)).reshape(1),
+        "activation_scaling_factor": act_sf,
+    }
+
+
+def postprocess_modelopt_awq(weight, weight_scale, pre_quant_scale, dtype=torch.float16, *, group_size: int = 128,
+                             activation_scaling_factor=None, weights_scaling_factor_2=None, tp_split=None):
+    """ModelOpt AWQ tensors of one linear layer -> {"weight", "weights_scaling_factor",
+    "prequant_scaling_factor"} (+ "alpha", "activation_scaling_factor" for W4A8, when the two
+    per-tensor factors are given).
+
+    `weight` int8 [N/2, K]: byte (j, k) holds output channels 2j (low nibble) and 2j + 1 of input k as
+    signed 4-bit values; its transpose is the row-major packed [K, N/2] tensor the preprocess takes
+    (modeling_utils.py:1645-1648; functional.py:950-957 unpacks and re-packs the same nibbles).
+    `weight_scale` [N, K/g] (any shape with that many elements in that order: functional.py:918-931
+    reshapes what ModelOpt exports) becomes [K/g, N]; `pre_quant_scale` [K] becomes [1, K].
+    Lists of tensors (q, k, v that arrive separately) are concatenated along N; the smoothing vector is
+    shared, the first one is taken (functional.py:932-937).  `tp_split` = (dim, size, rank) as in
+    postprocess_gptq, applied to each part before the concatenation as the reference does."""
+    w4a8 = activation_scaling_factor is not None
+    weights = list(weight) if isinstance(weight, (list, tuple)) else [weight]
+    scales = list(weight_scale) if isinstance(weight_scale, (list, tuple)) else [weight_scale]
+    pqs = pre_quant_scale[0] if isinstance(pre_quant_scale, (list, tuple)) else pre_quant_scale
+    if len(weights) != len(scales):
+        raise ValueError("as many weight_scale tensors as weight tensors are required")
+    packed, scale_parts = [], []
+    for w, sc in zip(weights, scales):
+        if w.dtype != torch.int8 or w.dim() != 2:
+            raise ValueError("ModelOpt AWQ weights are int8 [N/2, K]")
+        k = w.shape[1]
+        if k % group_size:
+            raise ValueError("in_features must be a multiple of the group size")
+        wt = w.T.contiguous()  # [K, N/2], row-major, even column in the low nibble
+        st = sc.reshape(w.shape[0] * 2, k // group_size).T  # [K/g, N]
+        if tp_split is not None:
+            tp_dim, tp_size, tp_rank = tp_split
+            wt = wt.chunk(tp_size, tp_dim)[tp_rank]
+            st = st.chunk(tp_size, tp_dim)[tp_rank]
+        packed.append(wt)
+        scale_parts.append(st)
+    wt = torch.cat(packed, dim=1).contiguous()
+    st = torch.cat(scale_parts, dim=1).to(dtype).contiguous()
+    pqs = pqs.to(dtype).reshape(1, -1)
+    if tp_split is not None and tp_split[0] == 0:  # row-parallel: the smoothing vector follows the rows of K
+        pqs = pqs.chunk(tp_split[1], 1)[tp_split[2]]
+    act_type = torch.float8_e4m3fn if w4a8 else dtype
+    out = {"weight": ops.preprocess_weights_for_mixed_gemm(wt, torch.quint4x2, act_type),
+           "weights_scaling_factor": st, "prequant_scaling_factor": pqs.contiguous()}
+    if w4a8:
+        if weights_scaling_factor_2 is None:
+            raise ValueError("W4A8 needs weights_scaling_factor_2 next to activation_scaling_factor")
+        out.update(fold_w4a8(st, out["prequant_scaling_factor"], activation_scaling_factor, weights_scaling_factor_2))
+    return out
+
+
+# quant_algo strings of a checkpoint's config.json (tensorrt_llm/quantization/mode.py QuantAlgo) that
+# name a weight-only linear layer: (weight bits, groupwise?, fp8 activations?)
+_QUANT_ALGOS = {"W8A16": (8, False, False), "W4A16": (4, False, False), "W4A16_AWQ": (4, True, False),
+                "W4A8_AWQ": (4, True, True), "W4A16_GPTQ": (4, True, False), "W8A16_GPTQ": (8, True, False)}
+
+
+def load_trtllm_linear(checkpoint, prefix: str, *, sm_arch: int, quant_algo: str | None = None,
+                       group_size: int | None = None, rank: int = 0):
+    """One weight-only linear layer of a TensorRT-LLM checkpoint -> the operands of this library's matmul.
+
+    `checkpoint`: a checkpoint directory (`config.json` + `rank<rank>.safetensors`) or a dict of
+    tensors.  `prefix`: the layer's name, e.g. "transformer.layers.0.mlp.fc".  `sm_arch`: the SM the
+    checkpoint's weights were preprocessed for (the byte layout differs: 90 has no column
+    interleave; the checkpoint does not record it).  `quant_algo` / `group_size` default to
+    config.json's `quantization` section.
+
+    Tensors read (quantization/layers.py:744-751 per-channel, :998-1037 groupwise):
+      <prefix>.weight                   int8 [K, N*bits/8], or typed as the activation dtype
+                                        ([K, N/4] halfs for int4, [K, N/2] for int8)
+      <prefix>.per_channel_scale        [N]                 (W8A16 / W4A16)
+      <prefix>.weights_scaling_factor   [K/g, N]            (groupwise; float16 bits for W4A8)
+      <prefix>.zero                     [K/g, N]            optional
+      <prefix>.prequant_scaling_factor  [1, K]              optional (AWQ)
+      <prefix>.alpha                    [1] float32         W4A8
+      <prefix>.bias                     [N]                 optional
+    Returns a dict: weight (gfx950 layout), scales, zeros, pre_quant_scale, bias (None where absent),
+    alpha, n, k, group_size, quant_algo (the op's bit flags), bits, w4a8."""
+    if isinstance(checkpoint, (str, os.PathLike)):
+        from safetensors import safe_open
+        cfg_path = os.path.join(checkpoint, "config.json")
+        if os.path.exists(cfg_path):
+            with open(cfg_path) as f:
+                q = json.load(f).get("quantization", {})
+            quant_algo = quant_algo or q.get("quant_algo")
+            group_size = group_size if group_size is not None else q.get("group_size")
+        tensors = {}
+        with safe_open(os.path.join(checkpoint, "rank%d.safetensors" % rank), framework="pt", device="cpu") as f:
+            for key in f.keys():
+                if key.startswith(prefix + "."):
+                    tensors[key] = f.get_tensor(key)
+    else:
+        tensors = {k: v for k, v in checkpoint.items() if k.startswith(prefix + ".")}
+    if quant_algo not in _QUANT_ALGOS:
+        raise ValueError("quant_algo %r is not a weight-only algorithm this loader knows (%s)"
+                         % (quant_algo, ", ".join(sorted(_QUANT_ALGOS))))
+    bits, groupwise, w4a8 = _QUANT_ALGOS[quant_algo]
+    get = lambda name: tensors.get(prefix + "." + name)
+    weight = get("weight")
+    if weight is None:
+        raise KeyError(prefix + ".weight")
+    weight = weight.contiguous().view(torch.int8)  # groupwise layers type the bytes as the activation dtype
+    k, n = weight.shape[0], weight.shape[1] * 8 // bits
+    quant_type = torch.int8 if bits == 8 else torch.quint4x2
+    act_type = torch.float8_e4m3fn if w4a8 else torch.float16
+    row_major = ops.import_reference_weights(weight, quant_type, act_type, sm_arch)
+    out = {"weight": ops.preprocess_weights_for_mixed_gemm(row_major, quant_type, act_type), "n": n, "k": k,
+           "bits": bits, "w4a8": w4a8, "zeros": None, "pre_quant_scale": None, "alpha": 1.0, "bias": get("bias")}
+    from .functional import BIAS, ZERO, PRE_QUANT_SCALE, FP8_ALPHA, INT8_WEIGHT
+    algo = (INT8_WEIGHT if bits == 8 and groupwise else 0) | (BIAS if out["bias"] is not None else 0)
+    if not groupwise:
+        scales = get("per_channel_scale")
+        if scales is None:
+            raise KeyError(prefix + ".per_channel_scale")
+        out.update(scales=scales.reshape(-1).contiguous(), group_size=0)
+    else:
+        scales = get("weights_scaling_factor")
+        if scales is None:
+            raise KeyError(prefix + ".weights_scaling_factor")
+        if not group_size:
+            group_size = k // scales.shape[0]
+        if w4a8:  # float16 values stored under the activation dtype's name
+            scales = scales.contiguous().view(torch.float16)
+        out.update(scales=scales.contiguous(), group_size=int(group_size))
+        zero, pqs = get("zero"), get("prequant_scaling_factor")
+        if zero is not None:
+            out["zeros"] = (zero.contiguous().view(torch.float16) if w4a8 else zero).contiguous()
+            algo |= ZERO
+        if pqs is not None:
+            out["pre_quant_scale"] = pqs.reshape(-1).contiguous()
+            algo |= PRE_QUANT_SCALE
+        if w4a8:
+            alpha = get("alpha")
+            if alpha is None:
+                raise KeyError(prefix + ".alpha")
+            out["alpha"] = float(alpha.reshape(-1)[0])
+            algo |= FP8_ALPHA
+    out["quant_algo"] = algo
+    return out
+
+
+def linear_forward(layer: dict, x: torch.Tensor, device=None) -> torch.Tensor:
+    """Runs a layer returned by load_trtllm_linear on the GPU: moves its tensors there on first use and
+    calls the matching op (per-channel: weight_only_quant_matmul's kernel, groupwise: the groupwise one;
+    the bias of a per-channel layer, which that plugin does not take, is added afterwards as the
+    reference's layer does, quantization/layers.py:769-776)."""
+    from . import functional as F
+    device = device or x.device
+    if "_dev" not in layer:
+        layer["_dev"] = {key: (v.to(device) if isinstance(v, torch.Tensor) else v) for key, v in layer.items()
+                         if key in ("weight", "scales", "zeros", "pre_quant_scale", "bias")}
+    d = layer["_dev"]
+    if layer["group_size"] == 0:
+        algo = F.INT8_WEIGHT if layer["bits"] == 8 else 0
+        out = F.woq_matmul_raw(x, None, d["weight"], d["scales"], None, None, n=layer["n"], k=layer["k"], group_size=0,
+                               quant_algo=algo, out_dtype=x.dtype)
+        return out if d["bias"] is None else out + d["bias"]
+    out_dtype = x.dtype if x.dtype != torch.float8_e4m3fn else (d["bias"].dtype if d["bias"] is not None
+                                                                 else torch.float16)
+    algo = layer["quant_algo"]
+    pqs = d["pre_quant_scale"]
+    if x.dtype == torch.float8_e4m3fn:  # activations already smoothed and cast
+        algo &= ~F.PRE_QUANT_SCALE
+        pqs = None
+    return F.woq_matmul_raw(x, pqs, d["weight"], d["scales"], d["zeros"], d["bias"], n=layer["n"], k=layer["k"],
+                            group_size=layer["group_size"], quant_algo=algo, alpha=layer["alpha"], out_dtype=out_dtype)

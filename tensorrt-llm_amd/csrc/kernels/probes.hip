@@ -1,0 +1,134 @@
+// Measurement probes: what the hardware allows, measured with the same harness as the kernels
+// (bench.py --mode ceilings).  No counterpart in the reference.
+//   woq_probe_read   plain streaming read of a buffer: every lane one 16-byte load per KiB, a wavefront
+//                    reads `kib_per_wave` contiguous KiB with `U` loads in flight - the HBM ceiling
+//                    the weight-streaming kernels are measured against
+//   woq_probe_empty  a kernel that does nothing: the cost of a launch
+//   woq_probe_mfma   nothing but matrix instructions on every SIMD: the matrix-core ceiling
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+
+namespace woq
+{
+namespace
+{
+template <int U>
+__global__ void __launch_bounds__(256) probe_read_kernel(u32x4 const* __restrict__ src, size_t kib_per_wave, size_t waves,
+    unsigned* sink)
+{
+    size_t const wave = (size_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (wave >= waves)
+        return;
+    u32x4 const* q = src + wave * kib_per_wave * 64 + (threadIdx.x & 63);
+    u32x4 acc = {0, 0, 0, 0};
+    for (size_t i = 0; i < kib_per_wave; i += U)
+    {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            v[u] = q[(i + u) * 64];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            acc ^= v[u];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) // never true for the benchmark's data: keeps the loads
+        sink[wave & 1023] = 1;
+}
+
+__global__ void probe_empty_kernel(unsigned* sink)
+{
+    if (sink == nullptr)
+        sink[0] = 1;
+}
+
+// 16 independent accumulators per wavefront, ITERS rounds: the matrix core never waits for a result
+template <int KIND>
+__global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters)
+{
+    f32x4 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    u32x4 a = {0x3C003C00u + threadIdx.x, 0x38003800u, 0x3C003C00u, 0x38003800u};
+    u32x4 b = a;
+    typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+    u32x8 a8 = {0x38383838u + threadIdx.x, 0x38383838u, 0x30303030u, 0x38383838u, 0x30303030u, 0x38383838u, 0x30303030u,
+        0x38383838u};
+    u32x8 b8 = a8;
+    for (int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+        {
+            if constexpr (KIND == 0)
+                asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a), "v"(b));
+            else
+                asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a8), "v"(b8));
+        }
+    }
+    mma_drain();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        s += acc[i][0];
+    sink[(blockIdx.x * 256 + threadIdx.x) & 1023] = s;
+}
+} // namespace
+} // namespace woq
+
+using namespace woq;
+
+extern "C" int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream)
+{
+    if (!src || !sink || kib_per_wave <= 0 || bytes < (size_t) kib_per_wave * 1024)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: src, sink and a buffer of at least one wavefront's share");
+    if (kib_per_wave % loads_in_flight)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: kib_per_wave must be a multiple of loads_in_flight");
+    size_t const waves = bytes / ((size_t) kib_per_wave * 1024);
+    dim3 const grid((unsigned) ((waves + 3) / 4)), block(256);
+    auto s = static_cast<hipStream_t>(stream);
+    auto const* p = static_cast<u32x4 const*>(src);
+    auto* k = static_cast<unsigned*>(sink);
+    switch (loads_in_flight)
+    {
+    case 1: hipLaunchKernelGGL(probe_read_kernel<1>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
+    case 2: hipLaunchKernelGGL(probe_read_kernel<2>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
+    case 4: hipLaunchKernelGGL(probe_read_kernel<4>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
+    case 8: hipLaunchKernelGGL(probe_read_kernel<8>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
+    default: return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: loads_in_flight must be 1, 2, 4 or 8");
+    }
+    hipError_t const err = hipGetLastError();
+    return err == hipSuccess ? WOQ_OK : fail(WOQ_ERR_RUNTIME, "probe launch failed: %s", hipGetErrorString(err));
+}
+
+extern "C" int woq_probe_empty(void* sink, void* stream)
+{
+    if (!sink)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_empty: sink is NULL");
+    hipLaunchKernelGGL(probe_empty_kernel, dim3(256), dim3(64), 0, static_cast<hipStream_t>(stream),
+        static_cast<unsigned*>(sink));
+    hipError_t const err = hipGetLastError();
+    return err == hipSuccess ? WOQ_OK : fail(WOQ_ERR_RUNTIME, "probe launch failed: %s", hipGetErrorString(err));
+}
+
+extern "C" double woq_probe_mfma(int kind, int iters, int workgroups, void* sink, void* stream)
+{
+    if (!sink || iters <= 0 || workgroups <= 0 || (kind != 0 && kind != 1))
+    {
+        fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_mfma: kind 0 (bf16 16x16x32) or 1 (fp8 16x16x128), iters, workgroups > 0");
+        return -1.0;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    if (kind == 0)
+        hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3(workgroups), dim3(256), 0, s, static_cast<float*>(sink), iters);
+    else
+        hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3(workgroups), dim3(256), 0, s, static_cast<float*>(sink), iters);
+    if (hipGetLastError() != hipSuccess)
+    {
+        fail(WOQ_ERR_RUNTIME, "probe launch failed");
+        return -1.0;
+    }
+    double const per_instr = kind == 0 ? 2.0 * 16 * 16 * 32 : 2.0 * 16 * 16 * 128;
+    return per_instr * 16.0 * iters * 4.0 * workgroups; // floating-point operations of the launch
+}

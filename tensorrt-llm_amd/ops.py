@@ -153,29 +153,30 @@ def _symmetric_quantize_last_axis_of_batched_matrix(weight: torch.Tensor, quant_
 
 
 def _register_torch_ops() -> None:
-    """Registers the ops as torch.ops.trtllm.* so code written against the reference finds them."""
-    try:
-        define = torch.library.define
-        impl = torch.library.impl
-        defs = {
-            "symmetric_quantize_last_axis_of_batched_matrix":
-                ("(Tensor weight, ScalarType quant_type) -> Tensor[]", symmetric_quantize_last_axis_of_batched_matrix),
-            "_symmetric_quantize_last_axis_of_batched_matrix":
-                ("(Tensor weight, ScalarType quant_type) -> Tensor[]", _symmetric_quantize_last_axis_of_batched_matrix),
-            "preprocess_weights_for_mixed_gemm":
-                ("(Tensor weight, ScalarType quant_type, ScalarType activation_type) -> Tensor",
-                 preprocess_weights_for_mixed_gemm),
-            "unpack_int4_packed_tensor_to_int8": ("(Tensor weight) -> Tensor", unpack_int4_packed_tensor_to_int8),
-            "pack_int8_tensor_to_packed_int4": ("(Tensor weight) -> Tensor", pack_int8_tensor_to_packed_int4),
-        }
-        for name, (schema, fn) in defs.items():
-            qual = "trtllm::" + name
-            if hasattr(torch.ops.trtllm, name):
-                continue
-            define(qual, schema)
-            impl(qual, "CPU")(fn)
-    except Exception:  # registration is a convenience; the python functions above are the interface
-        pass
+    """Registers the ops as torch.ops.trtllm.* so that code written against the reference (its
+    conversion scripts and tests call them by these names) finds them.  A failure here is an error:
+    the promise that such code runs unchanged would otherwise break silently."""
+    defs = {
+        "symmetric_quantize_last_axis_of_batched_matrix":
+            ("(Tensor weight, ScalarType quant_type) -> Tensor[]", symmetric_quantize_last_axis_of_batched_matrix),
+        "_symmetric_quantize_last_axis_of_batched_matrix":
+            ("(Tensor weight, ScalarType quant_type) -> Tensor[]", _symmetric_quantize_last_axis_of_batched_matrix),
+        "preprocess_weights_for_mixed_gemm":
+            ("(Tensor weight, ScalarType quant_type, ScalarType activation_type) -> Tensor",
+             preprocess_weights_for_mixed_gemm),
+        "unpack_int4_packed_tensor_to_int8": ("(Tensor weight) -> Tensor", unpack_int4_packed_tensor_to_int8),
+        "pack_int8_tensor_to_packed_int4": ("(Tensor weight) -> Tensor", pack_int8_tensor_to_packed_int4),
+    }
+    for name, (schema, fn) in defs.items():
+        qual = "trtllm::" + name
+        if hasattr(torch.ops.trtllm, name):  # this module imported twice in one process
+            continue
+        torch.library.define(qual, schema)
+        torch.library.impl(qual, "CPU")(fn)
 
+
+REGISTERED_TORCH_OPS = ("symmetric_quantize_last_axis_of_batched_matrix", "_symmetric_quantize_last_axis_of_batched_matrix",
+                        "preprocess_weights_for_mixed_gemm", "unpack_int4_packed_tensor_to_int8",
+                        "pack_int8_tensor_to_packed_int4")
 
 _register_torch_ops()

@@ -147,3 +147,156 @@ def test_checkpoint_tensors_run_through_the_matmul(pkg, oracle, dev, fmt):
     # and the folded zeros mean (u - zp) * scale up to the rounding of the zero tensor
     w_true = (u - np.repeat(zp, g, axis=0)) * np.repeat(s_bf, g, axis=0)
     assert np.abs(w - w_true).max() <= np.abs(w_true).max() * 2.0 ** -7
+
+
+# ---- ModelOpt AWQ, the W4A8 fold, q / k / v concatenation ------------------------------------------
+
+
+def _modelopt_pack(q_signed):
+    """[K, N] signed int4 -> ModelOpt's int8 [N/2, K]: output channels 2j (low nibble) and 2j + 1 of
+    input k share byte (j, k)."""
+    u = (q_signed.T.astype(np.int16) & 0xF).astype(np.uint8)  # [N, K]
+    return torch.from_numpy((u[0::2] | (u[1::2] << 4)).view(np.int8).copy())
+
+
+def test_modelopt_awq_layer_and_separate_qkv(pkg):
+    """The transposed int8 tensor, the [N, K/g] scales and the smoothing vector of ModelOpt's export become
+    the op's operands; q, k, v given separately are the same as one fused layer."""
+    K, g = 256, 128
+    rng = np.random.default_rng(5)
+    parts = [rng.integers(-8, 8, size=(K, n)).astype(np.int8) for n in (64, 32, 32)]
+    scales = [rng.uniform(0.002, 0.02, size=(p.shape[1], K // g)).astype(np.float32) for p in parts]
+    pqs = torch.from_numpy(rng.uniform(0.5, 2.0, K).astype(np.float32))
+    one = pkg.checkpoint.postprocess_modelopt_awq(_modelopt_pack(parts[0]), torch.from_numpy(scales[0]).reshape(-1), pqs,
+                                                  torch.bfloat16, group_size=g)
+    assert (_decode(pkg, one["weight"], K, 4) == parts[0]).all()
+    assert torch.equal(one["weights_scaling_factor"], torch.from_numpy(scales[0].T.copy()).to(torch.bfloat16))
+    assert one["prequant_scaling_factor"].shape == (1, K)
+    fused = pkg.checkpoint.postprocess_modelopt_awq([_modelopt_pack(p) for p in parts],
+                                                    [torch.from_numpy(s) for s in scales], [pqs, pqs, pqs],
+                                                    torch.bfloat16, group_size=g)
+    assert (_decode(pkg, fused["weight"], K, 4) == np.concatenate(parts, axis=1)).all()
+    want = torch.from_numpy(np.concatenate([s.T for s in scales], axis=1)).to(torch.bfloat16)
+    assert torch.equal(fused["weights_scaling_factor"], want)
+    # column-parallel split of every part before the concatenation, as the reference's loader does
+    half = pkg.checkpoint.postprocess_modelopt_awq([_modelopt_pack(p) for p in parts],
+                                                   [torch.from_numpy(s) for s in scales], pqs, torch.bfloat16,
+                                                   group_size=g, tp_split=(1, 2, 1))
+    assert (_decode(pkg, half["weight"], K, 4) == np.concatenate([p[:, p.shape[1] // 2:] for p in parts], axis=1)).all()
+
+
+def test_gptq_parts_concatenate_along_n(pkg):
+    K, g = 128, 64
+    us, zps, scs = zip(*[_quantized(K, n, g, 20 + n) for n in (32, 16, 16)])
+    parts = [(_pack_rows_gptq(u, 8, 4), torch.from_numpy(s), _pack_cols(zp - 1, list(range(8))))
+             for u, zp, s in zip(us, zps, scs)]
+    out = pkg.checkpoint.postprocess_gptq(*pkg.checkpoint.concat_gptq_parts(parts), torch.float16)
+    q, s, z = _expected(pkg, np.concatenate(us, 1), np.concatenate(zps, 1), np.concatenate(scs, 1), 4, torch.float16)
+    assert (_decode(pkg, out["weight"], K, 4) == q).all() and torch.equal(out["zero"], z)
+
+
+def test_w4a8_fold_is_the_loaders_and_the_oracles(pkg, oracle):
+    """fold_w4a8 follows the reference loader's order of operations (modeling_utils.py:1661-1682):
+    hand-computed values, and agreement with the oracle's benchmark-input generator, which folds the same
+    factors on its own (float32 group scales / wsf2 -> float16; smoothing / act_sf; alpha = act_sf * wsf2)."""
+    f = pkg.checkpoint.fold_w4a8(torch.tensor([[0.5, 0.25], [1.0, 3.0]]), torch.tensor([[2.0, 4.0]]),
+                                 torch.tensor(0.5), torch.tensor(0.125))
+    assert torch.equal(f["weights_scaling_factor"], torch.tensor([[4.0, 2.0], [8.0, 24.0]], dtype=torch.float16))
+    assert torch.equal(f["prequant_scaling_factor"], torch.tensor([[4.0, 8.0]]))
+    assert f["alpha"].dtype == torch.float32 and f["alpha"].item() == 0.0625
+    M, K, N = 4, 256, 64
+    prob = oracle.make_w4a8_problem(M, K, N, seed=9, out_dtype="bf16")
+    # the same unfolded inputs, recomputed as the generator defines them
+    q, scale = oracle.make_w4_groupwise_sym(K, N, 128, 9, "fp32")
+    rng = np.random.default_rng(9 + 7)
+    smooth = oracle.round_to(rng.uniform(0.5, 2.0, size=(K,)).astype(np.float32), "bf16")
+    act = oracle.make_activations(M, K, 9 + 13, "bf16")
+    act_sf = np.float32(np.abs(act * smooth).max() / 448.0)
+    wsf2 = np.float32(np.abs(q.astype(np.float32).reshape(K // 128, 128, N) * scale[:, None, :]).max() / 448.0)
+    f = pkg.checkpoint.fold_w4a8(torch.from_numpy(scale), torch.from_numpy(smooth), torch.tensor(act_sf),
+                                 torch.tensor(wsf2))
+    assert (f["weights_scaling_factor"].float().numpy() == prob["scales"]).all()
+    assert (oracle.round_to(f["prequant_scaling_factor"].numpy(), "bf16") == prob["pre_quant_scale"]).all()
+    assert f["alpha"].item() == np.float32(prob["alpha"])
+
+
+# ---- TensorRT-LLM checkpoints (reference-layout weights) ---------------------------------------------
+
+import json
+import os
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+CKPTS = sorted(d for d in os.listdir(GOLDEN) if d.startswith("trtllm_ckpt_"))
+
+
+def _fixture(name):
+    from safetensors.torch import load_file
+    path = os.path.join(GOLDEN, name)
+    with open(os.path.join(path, "config.json")) as f:
+        cfg = json.load(f)
+    return path, cfg, load_file(os.path.join(path, "rank0.safetensors"))
+
+
+@pytest.mark.parametrize("name", CKPTS)
+def test_load_trtllm_linear_decodes_the_reference_layout(pkg, name):
+    """Every fixture checkpoint (tests/golden/make_trtllm_checkpoint.py: weights in the reference's SM80 /
+    SM89 / SM90 layouts, W8A16, W4A16, AWQ, GPTQ and W4A8 flavours) loads into this library's layout
+    holding exactly the quantized values it was made from; the other tensors pass through under the op's
+    argument names."""
+    path, cfg, raw = _fixture(name)
+    fx = cfg["_fixture"]
+    layer = pkg.checkpoint.load_trtllm_linear(path, fx["layer"], sm_arch=fx["sm_arch"])
+    q = raw["_expected.%s.q" % fx["layer"]].numpy()
+    assert (layer["k"], layer["n"]) == (fx["k"], fx["n"]) == q.shape
+    act_type = torch.float8_e4m3fn if layer["w4a8"] else torch.float16
+    qt = torch.quint4x2 if layer["bits"] == 4 else torch.int8
+    back = pkg.ops.unprocess_weights_for_mixed_gemm(layer["weight"], fx["k"], qt, act_type)
+    back = pkg.ops.unpack_int4_packed_tensor_to_int8(back).numpy() if layer["bits"] == 4 else back.numpy()
+    assert (back == q).all()
+    quant = cfg["quantization"]
+    assert layer["group_size"] == (quant["group_size"] or 0)
+    assert (layer["zeros"] is not None) == quant["has_zero_point"]
+    assert (layer["pre_quant_scale"] is not None) == quant["pre_quant_scale"]
+    F = pkg.functional
+    assert bool(layer["quant_algo"] & F.FP8_ALPHA) == (quant["quant_algo"] == "W4A8_AWQ")
+    if layer["w4a8"]:
+        assert layer["scales"].dtype == torch.float16 and abs(layer["alpha"] - 0.0123) < 1e-9
+    # a wrong SM decodes to other values (80 and 90 differ by the column interleave)
+    other = 90 if fx["sm_arch"] != 90 else 80
+    wrong = pkg.checkpoint.load_trtllm_linear(path, fx["layer"], sm_arch=other)
+    assert not torch.equal(wrong["weight"], layer["weight"])
+
+
+def test_load_trtllm_linear_errors(pkg):
+    path, cfg, raw = _fixture("trtllm_ckpt_w4a16_awq_sm80")
+    layer = cfg["_fixture"]["layer"]
+    with pytest.raises(KeyError):
+        pkg.checkpoint.load_trtllm_linear(path, "transformer.layers.9.mlp.fc", sm_arch=80)
+    with pytest.raises(ValueError, match="quant_algo"):
+        pkg.checkpoint.load_trtllm_linear(raw, layer, sm_arch=80, quant_algo="FP8")
+    # a dict of tensors instead of a directory, the algorithm given by the caller
+    again = pkg.checkpoint.load_trtllm_linear(raw, layer, sm_arch=80, quant_algo="W4A16_AWQ")
+    assert torch.equal(again["weight"], pkg.checkpoint.load_trtllm_linear(path, layer, sm_arch=80)["weight"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", CKPTS)
+@pytest.mark.parametrize("M", [3, 40])
+def test_trtllm_checkpoint_layer_runs_through_the_matmul(pkg, oracle, dev, name, M):
+    """End to end: checkpoint directory -> loader -> GPU matmul == the oracle's dequantize-then-matmul on
+    the values the fixture was made from (streaming kernel at 3 rows, GEMM kernels at 40)."""
+    path, cfg, raw = _fixture(name)
+    fx = cfg["_fixture"]
+    layer = pkg.checkpoint.load_trtllm_linear(path, fx["layer"], sm_arch=fx["sm_arch"])
+    dt = {"float16": "fp16", "bfloat16": "bf16"}[cfg["dtype"]]
+    tdt = {"fp16": torch.float16, "bf16": torch.bfloat16}[dt]
+    rng = np.random.default_rng(M)
+    act = oracle.round_to(rng.standard_normal((M, fx["k"])).astype(np.float32), dt)
+    out = pkg.checkpoint.linear_forward(layer, torch.from_numpy(act).to(tdt).to(dev))
+    torch.cuda.synchronize()
+    f32 = lambda x: None if x is None else x.float().numpy()
+    q = raw["_expected.%s.q" % fx["layer"]].numpy()
+    ref = oracle.woq_matmul_ref(act, q, f32(layer["scales"]), f32(layer["zeros"]), f32(layer["bias"]),
+                                f32(layer["pre_quant_scale"]), layer["alpha"], layer["group_size"], dt,
+                                w4a8=layer["w4a8"])
+    assert oracle.max_rel_err(out.float().cpu().numpy(), ref) < 1e-2

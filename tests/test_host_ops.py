@@ -134,3 +134,28 @@ def test_host_float16_conversions_roundtrip(pkg):
         _, scales = pkg.ops.symmetric_quantize_last_axis_of_batched_matrix(w.to(dt), torch.quint4x2)
         expect = ((w.to(dt).float().abs().max(0).values) * 0.125).to(dt)
         assert (scales == expect).all()
+
+
+def test_every_op_is_reachable_through_torch_ops_trtllm(pkg):
+    """The five ops the reference registers for weight preparation (thop/weightOnlyQuantOp.cpp:358-369),
+    called the way its conversion scripts and tests call them - by name under torch.ops.trtllm, positional
+    arguments, torch dtypes for the ScalarType parameters - give what the python functions give."""
+    T = torch.ops.trtllm
+    for name in pkg.ops.REGISTERED_TORCH_OPS:
+        assert hasattr(T, name), name
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn((128, 64), generator=g, dtype=torch.float16)
+    for qt in (torch.int8, torch.quint4x2):
+        processed, scales = T.symmetric_quantize_last_axis_of_batched_matrix(w, qt)
+        want = pkg.ops.symmetric_quantize_last_axis_of_batched_matrix(w, qt)
+        assert torch.equal(processed, want[0]) and torch.equal(scales, want[1])
+        unprocessed, processed2, scales2 = T._symmetric_quantize_last_axis_of_batched_matrix(w, qt)
+        assert torch.equal(processed2, processed) and torch.equal(scales2, scales)
+        again = T.preprocess_weights_for_mixed_gemm(unprocessed, qt, torch.float16)
+        assert torch.equal(again, processed)
+    q = torch.randint(-8, 8, (16, 32), generator=g, dtype=torch.int8)
+    packed = T.pack_int8_tensor_to_packed_int4(q)
+    assert packed.shape == (16, 16) and torch.equal(T.unpack_int4_packed_tensor_to_int8(packed), q)
+    # the fp8 activation type selects the W4A8 flavour (get_ft_quant_type, thop/weightOnlyQuantOp.cpp:41-62)
+    a8 = T.preprocess_weights_for_mixed_gemm(packed.repeat(8, 2).contiguous(), torch.quint4x2, torch.float8_e4m3fn)
+    assert a8.shape == (128, 32)
