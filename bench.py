@@ -534,19 +534,22 @@ def run_ceilings(pkg, dev):
     _, sec, launches = time_graph(empty, 200, repeats=3)
     out["empty_launch_us"] = round(sec / launches * 1e6, 3)
     for kind, name, peak in [(0, "v_mfma_f32_16x16x32_bf16", MFMA_BF16_PEAK_TFLOPS),
+                             (2, "v_mfma_f32_32x32x16_bf16", MFMA_BF16_PEAK_TFLOPS),
                              (1, "v_mfma_f32_16x16x128_f8f6f4 (e4m3)", MFMA_FP8_PEAK_TFLOPS)]:
-        flop = [0.0]
+        for random_operands in (0, 1):
+            flop = [0.0]
 
-        def body(reps=4):
-            for _ in range(reps):
-                flop[0] = lib.woq_probe_mfma(kind, 20000, 256, ctypes.c_void_p(sink.data_ptr()), stream_of())
-        body(1)
-        torch.cuda.synchronize()
-        _, sec, launches = time_graph(body, 4, repeats=3)
-        tf = flop[0] / (sec / launches) / 1e12
-        out.setdefault("mfma", []).append({"instruction": name, "tflops": round(tf, 1), "peak": peak,
-                                           "frac_of_peak": round(tf / peak, 4),
-                                           "ms_per_launch": round(sec / launches * 1e3, 3)})
+            def body(reps=8):
+                for _ in range(reps):
+                    flop[0] = lib.woq_probe_mfma(kind, random_operands, 20000, 256, ctypes.c_void_p(sink.data_ptr()),
+                                                 stream_of())
+            body(1)
+            torch.cuda.synchronize()
+            _, sec, launches = time_graph(body, 8, repeats=3)
+            tf = flop[0] / (sec / launches) / 1e12
+            out.setdefault("mfma", []).append({"instruction": name, "operands": "random" if random_operands else "constant",
+                                               "tflops": round(tf, 1), "peak": peak, "frac_of_peak": round(tf / peak, 4),
+                                               "ms_per_launch": round(sec / launches * 1e3, 3)})
     print(json.dumps(out))
 
 

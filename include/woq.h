@@ -326,11 +326,13 @@ int woq_dequantize(void* out, const void* weight, const void* scales, const void
  * kib_per_wave contiguous KiB, loads_in_flight of 1, 2, 4 or 8 16-byte loads per lane outstanding);
  * `sink` is 4 KiB of device memory.  woq_probe_empty: a kernel that does nothing.  woq_probe_mfma:
  * nothing but matrix instructions (kind 0: v_mfma_f32_16x16x32_bf16, 1: v_mfma_f32_16x16x128_f8f6f4
- * on e4m3) on `workgroups` x 4 wavefronts; returns the floating-point operations of the launch
- * (negative on a bad argument). */
+ * on e4m3, 2: v_mfma_f32_32x32x16_bf16) on `workgroups` x 4 wavefronts, multiplying the same operand registers every time
+ * (random_operands 0: least switching activity) or four pseudo-random operand pairs in turn (1: what
+ * the power management sustains under real data); returns the floating-point operations of the
+ * launch (negative on a bad argument). */
 int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream);
 int woq_probe_empty(void* sink, void* stream);
-double woq_probe_mfma(int kind, int iters, int workgroups, void* sink, void* stream);
+double woq_probe_mfma(int kind, int random_operands, int iters, int workgroups, void* sink, void* stream);
 
 /* ---- misc ------------------------------------------------------------------------------------ */
 
@@ -340,6 +342,13 @@ double woq_probe_mfma(int kind, int iters, int workgroups, void* sink, void* str
 void woq_reload_env(void);
 
 const char* woq_last_error(void);
+
+/* Which kernel the last matmul call of this thread launched, as text: "gemm exact rt=16 splits=1
+ * persistent=1", "gemm skinny rt=4 splits=2", "stream mt=.. ns=.. waves=.. pf=.. slots=.. k_slices=..",
+ * "stream wide ns=.. waves=.. pf=.. slots=..", "gemm w4a8 ...", "stream w4a8 ..."; empty before the
+ * first call.  For tests of the dispatch rules and for tuning scripts; no counterpart in the
+ * reference.  The pointer stays valid until the thread's next call of this function. */
+const char* woq_last_launch(void);
 int woq_abi_version(void);
 int woq_layout_version(void);
 

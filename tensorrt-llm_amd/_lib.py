@@ -86,9 +86,10 @@ def _load():
         "woq_import_tactics": (ctypes.c_int, [ctypes.c_char_p]),
         "woq_probe_read": (ctypes.c_int, [vp, sz, i32, i32, vp, vp]),
         "woq_probe_empty": (ctypes.c_int, [vp, vp]),
-        "woq_probe_mfma": (ctypes.c_double, [i32, i32, i32, vp, vp]),
+        "woq_probe_mfma": (ctypes.c_double, [i32, i32, i32, i32, vp, vp]),
         "woq_reload_env": (None, []),
         "woq_last_error": (ctypes.c_char_p, []),
+        "woq_last_launch": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),
         "woq_layout_version": (ctypes.c_int, []),
     }

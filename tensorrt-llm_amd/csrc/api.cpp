@@ -264,6 +264,32 @@ int pick_stream_k_slices(int m, int n, int k, int tile_k, int group, size_t work
     return slices;
 }
 
+int gemm_persistent_workgroups()
+{
+    if (env_overrides().persist_off)
+        return 0;
+    // CU count per device ordinal, asked once (0: not yet known)
+    static std::atomic<int> cus[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    {
+        (void) hipGetLastError();
+        return 0;
+    }
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0)
+    {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        {
+            (void) hipGetLastError();
+            return 0;
+        }
+        n = n / 8 * 8;
+        cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 bool stream_slots_disabled()
 {
     return env_overrides().slots_off;
@@ -295,6 +321,8 @@ EnvOverrides read_env()
         o.gemm_splits = std::atoi(e);
     if (char const* e = std::getenv("WOQ_STREAM_SPLITS"))
         o.stream_splits = std::atoi(e);
+    if (char const* e = std::getenv("WOQ_GEMM_PERSIST"))
+        o.persist_off = e[0] == '0';
     return o;
 }
 

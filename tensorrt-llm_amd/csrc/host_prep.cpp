@@ -231,6 +231,36 @@ constexpr int kPermW4A8[32] = {0, 1, 2, 3, 16, 17, 18, 19, 4, 5, 6, 7, 20, 21, 2
 
 using namespace woq;
 
+namespace
+{
+struct LaunchNote
+{
+    char const* fmt = nullptr;
+    int v[6] = {};
+};
+thread_local LaunchNote g_launch_note;
+thread_local char g_launch_text[160] = "";
+} // namespace
+
+void woq::note_launch(char const* fmt, int a, int b, int c, int d, int e, int f)
+{
+    g_launch_note = LaunchNote{fmt, {a, b, c, d, e, f}};
+}
+
+extern "C" const char* woq_last_launch(void)
+{
+    LaunchNote const& n = g_launch_note;
+    g_launch_text[0] = 0;
+    if (n.fmt)
+    {
+#pragma GCC diagnostic push
+#pragma GCC diagnostic ignored "-Wformat-nonliteral"
+        std::snprintf(g_launch_text, sizeof g_launch_text, n.fmt, n.v[0], n.v[1], n.v[2], n.v[3], n.v[4], n.v[5]);
+#pragma GCC diagnostic pop
+    }
+    return g_launch_text;
+}
+
 extern "C" const char* woq_last_error(void)
 {
     return g_last_error;

@@ -56,6 +56,12 @@ struct Elem<WOQ_BF16>
         asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 
+    // c = a x b: the first product of a new sum (the old value of c is dead: no input operand for it)
+    static __device__ __forceinline__ void mma_first(u32x4 a, u32x4 b, f32x4& c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+    }
+
     static __device__ __forceinline__ float lo(uint32_t pair)
     {
         return bit_cast<float>(pair << 16);
@@ -112,6 +118,11 @@ struct Elem<WOQ_FP16>
     static __device__ __forceinline__ void mma_acc(u32x4 a, u32x4 b, f32x4& c)
     {
         asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+
+    static __device__ __forceinline__ void mma_first(u32x4 a, u32x4 b, f32x4& c)
+    {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
     }
 
     static __device__ __forceinline__ float lo(uint32_t pair)

@@ -30,6 +30,11 @@ namespace woq
 
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
 
+// Workgroups of a persistent launch: the CU count of the current device rounded down to a multiple
+// of 8 (one per CU, the same number on every XCD); 0 switches the persistent kernels off
+// (WOQ_GEMM_PERSIST=0).
+int gemm_persistent_workgroups();
+
 // amdgpu_waves_per_eu(1, 1): one wavefront per SIMD is the design point (256 accumulator
 // registers per lane); without it the register allocator chases a higher occupancy it cannot
 // reach and parks live values in the accumulator file, shuffling them around every step.
@@ -38,9 +43,17 @@ constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent wor
 //        prefill; 8 / 4 for skinny M, where a 256-row tile would mostly multiply padding.
 // SPLITK several workgroups share one output tile, each covering a slice of K, and add their
 //        partial sums into a float32 buffer (skinny M x narrow N would otherwise leave most CUs idle).
-template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK>
+// PERSIST one workgroup per CU walks several output tiles (tile b, b + gridDim.x, ...).  The last tile
+//        row of a tile already requests the first A tile and weights of the NEXT tile, and the
+//        outputs of a finished tile are converted and stored between the matrix instructions of
+//        the next tile's first tile row (each accumulator block right before it is cleared for
+//        reuse): neither the first-load latency of a tile nor its burst of 128 KiB of stores is
+//        paid with the matrix core idle.  Plain epilogue only (bias; no activation, no residual);
+//        K must be an even number of tile rows; m * n * 2 < 2 GiB (outputs go through a descriptor).
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, bool PERSIST = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_kernel(GemmParams p)
 {
+    static_assert(!(PERSIST && SPLITK), "a persistent workgroup owns whole tiles");
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
@@ -55,16 +68,26 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     __shared__ u32x4 a_buf1[A_BYTES / 16];
 
     // ---- which output tile: XCD-contiguous chunks, m fastest inside groups of kGemmGroupM ------
+    // (virtual block vb: the block index itself, or with PERSIST the block index plus a multiple of
+    // the grid size, which is a multiple of 8 - a workgroup stays on its XCD's chunk of the order)
     int const total = p.tiles_m * p.tiles_n;
     int const per_xcd = (total + 7) / 8;
-    int const t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if ((int) (blockIdx.x >> 3) >= per_xcd || t >= total)
+    auto tile_of = [&](int vb, int& tm_, int& tn_) -> bool
+    {
+        int const t = (vb & 7) * per_xcd + (vb >> 3);
+        if ((vb >> 3) >= per_xcd || t >= total)
+            return false;
+        int const in_group = kGemmGroupM * p.tiles_n;
+        int const first_m = (t / in_group) * kGemmGroupM;
+        int const gsz = p.tiles_m - first_m < kGemmGroupM ? p.tiles_m - first_m : kGemmGroupM;
+        tm_ = first_m + (t % in_group) % gsz;
+        tn_ = (t % in_group) / gsz;
+        return true;
+    };
+    int vb = (int) blockIdx.x;
+    int tm, tn;
+    if (!tile_of(vb, tm, tn))
         return;
-    int const in_group = kGemmGroupM * p.tiles_n;
-    int const first_m = (t / in_group) * kGemmGroupM;
-    int const gsz = p.tiles_m - first_m < kGemmGroupM ? p.tiles_m - first_m : kGemmGroupM;
-    int tm = first_m + (t % in_group) % gsz;
-    int const tn = (t % in_group) / gsz;
     if (p.expert_rows && !select_expert(p, tm, kGemmBM))
         return;
 
@@ -77,8 +100,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int const kt_begin = SPLITK ? (int) blockIdx.y * p.tiles_per_split : 0;
     int const KT = SPLITK ? (kt_begin + p.tiles_per_split < p.k_tiles ? kt_begin + p.tiles_per_split : p.k_tiles)
                           : p.k_tiles;
-    int const m0 = tm * kGemmBM;
-    int const strip0 = tn * (kGemmBN / 16) + wave * NS;
+    int m0 = tm * kGemmBM;
+    int strip0 = tn * (kGemmBN / 16) + wave * NS;
+    uint32_t tile_oob = 0; // PERSIST: kOob once there is no further tile (every request reads zeros)
 
     constexpr uint32_t kOob = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K * 2u);
@@ -108,13 +132,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // per-column scale of the per-channel mode (GROUP == 0) is loaded once
     float pc_scale[NS];
     uint32_t pc_scale2[NS]; // the raw 16-bit value in both halves
+    // the same for the tile row after the current one (PERSIST: another tile's columns at a tile boundary)
+    float pc_scale_n[NS];
+    uint32_t pc_scale2_n[NS];
     if constexpr (GROUP == 0)
     {
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
-            pc_scale[s] = E::load(p.scales, strip_of[s] * 16 + c);
-            pc_scale2[s] = (uint32_t) static_cast<uint16_t const*>(p.scales)[strip_of[s] * 16 + c] * 0x10001u;
+            pc_scale[s] = pc_scale_n[s] = E::load(p.scales, strip_of[s] * 16 + c);
+            pc_scale2[s] = pc_scale2_n[s]
+                = (uint32_t) static_cast<uint16_t const*>(p.scales)[strip_of[s] * 16 + c] * 0x10001u;
         }
     }
 
@@ -135,8 +163,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     constexpr int DMA_OPS = FRAGS / 4;
     static_assert(4 % SLABS == 0 && FRAGS % 4 == 0, "fragment to wavefront mapping");
     int const dma_j = wave % SLABS;
-    uint32_t const dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
-                                       + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
+    uint32_t dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
+                                 + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
         * 2u;
     int const dma_lane_k = dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8); // k of this lane inside a tile row
     uint32_t const dma_piece_stride = (uint32_t) (4 / SLABS) * 16u * (uint32_t) K * 2u;
@@ -145,7 +173,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         // out of range (sign bit of K-1-k or of KT-1-kt set) -> an offset the descriptor rejects;
         // rows past M fall outside the descriptor by themselves
         int const kk = kt * TK + dma_lane_k;
-        return (dma_lane_base + (uint32_t) kt * (uint32_t) (TK * 2)) | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob);
+        return (dma_lane_base + (uint32_t) kt * (uint32_t) (TK * 2))
+            | (((uint32_t) (K - 1 - kk) | (uint32_t) (KT - 1 - kt)) & kOob) | tile_oob;
     };
     auto dma_piece = [&](auto* buf, uint32_t base, int i)
     {
@@ -180,7 +209,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         sc_lane[s] = (uint32_t) (strip_of[s] * 16 + c) * 2u;
     auto fetch_piece = [&](BStage& st, int kt, int i)
     {
-        uint32_t const past = (uint32_t) (KT - 1 - kt) & kOob; // kt >= KT: every load of the step reads zeros
+        uint32_t const past = ((uint32_t) (KT - 1 - kt) & kOob) | tile_oob; // kt >= KT: every load of the step reads zeros
         if (i < NS)
             st.w[i] = buffer_load_x4(w_rsrc, wlane[i] + ((uint32_t) kt * 1024u | past));
         else if constexpr (GROUP != 0)
@@ -217,7 +246,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     constexpr int A_AHEAD = 3;
     u32x4 b_cur[NS], b_nxt[NS];
 
-    auto scale_of = [&](BStage const& st, int s, int seg, float& sc, float& zr)
+    auto scale_of = [&](BStage const& st, int s, int seg, float& sc, float& zr, bool next_step = false)
     {
         if constexpr (GROUP != 0)
         {
@@ -226,13 +255,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         else
         {
-            sc = pc_scale[s];
+            sc = next_step ? pc_scale_n[s] : pc_scale[s];
             zr = 0.f;
         }
     };
 
     // the same as packed half-precision pairs (s, s) and (z, z), from the raw 16-bit values
-    auto scale_pair_of = [&](BStage const& st, int s, int seg, uint32_t& s2, uint32_t& z2)
+    auto scale_pair_of = [&](BStage const& st, int s, int seg, uint32_t& s2, uint32_t& z2, bool next_step = false)
     {
         if constexpr (GROUP != 0)
         {
@@ -241,13 +270,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         else
         {
-            s2 = pc_scale2[s];
+            s2 = next_step ? pc_scale2_n[s] : pc_scale2[s];
             z2 = 0u;
         }
     };
 
-    auto compute = [&](auto const* buf, BStage const& st, BStage& st_next, auto* buf_next, int kt_next)
+    // PERSIST: where the finished tile's outputs go (set when the workgroup moves on to its next tile)
+    [[maybe_unused]] auto const out_rsrc = make_rsrc(p.out, (uint32_t) p.m * (uint32_t) p.n * 2u);
+    // byte offset of (row m0 + c, column strip0*16 + kg*4) of the tile to store (the launcher only
+    // takes this path when N is a multiple of the tile width and there is no bias: every strip of
+    // the tile exists, rows past M fall outside the descriptor); kOob: no finished tile yet
+    [[maybe_unused]] uint32_t prev_off = kOob;
+    [[maybe_unused]] uint32_t const rt_stride = 16u * (uint32_t) p.n * 2u; // bytes between row tiles of the output
+    auto store_block = [&](int rt, int s)
     {
+        // read out through explicit AGPR-source moves: a plain use of the block by VALU code would make
+        // the allocator keep every accumulator in the VGPR half of the file across the whole loop
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[rt][s][r]));
+        u32x2 const o = {E::pack(p.alpha * v[0], p.alpha * v[1]), E::pack(p.alpha * v[2], p.alpha * v[3])};
+        // the row-tile offset belongs in the vector offset: the descriptor's range check does not
+        // see the scalar offset, and rows past M must be dropped by it
+        __builtin_amdgcn_raw_buffer_store_b64(o, out_rsrc, (int) (prev_off + (uint32_t) rt * rt_stride + (uint32_t) s * 32u), 0, 0);
+    };
+
+    auto compute = [&](auto first_tag, auto const* buf, BStage const& st, BStage& st_next, auto* buf_next, int kt_next)
+    {
+        constexpr bool FIRST = decltype(first_tag)::value; // first tile row of a tile (PERSIST only)
         char const* a_base = reinterpret_cast<char const*>(buf) + a_lane_off;
         constexpr int ITERS = SLABS * RT;
         uint32_t const next_base = dma_base(kt_next);
@@ -302,7 +353,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                         {
                             if (stage == 0)
                             {
-                                scale_of(src, s, jn / SEG_SLABS, sc[x], zr[x]);
+                                scale_of(src, s, jn / SEG_SLABS, sc[x], zr[x], !same_step);
                                 sc[x] *= BITS == 4 ? 16.f : 1.f;
                             }
                             else if (stage == 1)
@@ -323,7 +374,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                         else
                         {
                             if (stage == 0)
-                                scale_pair_of(src, s, jn / SEG_SLABS, s2[x], z2[x]);
+                                scale_pair_of(src, s, jn / SEG_SLABS, s2[x], z2[x], !same_step);
                             else if (stage == 1)
                             {
                                 if constexpr (BITS == 4)
@@ -342,6 +393,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
                 {
+                    if constexpr (FIRST)
+                    {
+                        // the block's sums of the previous tile leave (rows past M and strips past N
+                        // fall outside the descriptor) right before the block starts the new tile's sum
+                        if (j == 0)
+                            store_block(rt, s);
+                    }
                     // weights as the first operand: the accumulator holds the TRANSPOSED 16x16 block,
                     // lane (kg, c) the four consecutive columns kg*4 .. kg*4+3 of output row c, so the
                     // epilogue moves 8 bytes per lane and block instead of 2
@@ -349,6 +407,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     // 64 consecutive bytes per row and instruction)
                     if constexpr (SPLITK)
                         E::mma_acc(a_cur, b_cur[s], acc[rt][s]);
+                    else if (FIRST && j == 0)
+                        E::mma_first(b_cur[s], a_cur, acc[rt][s]); // the block starts the new tile's sum
                     else
                         E::mma_acc(b_cur[s], a_cur, acc[rt][s]);
                     conv_stage(s);
@@ -377,14 +437,97 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // Before each barrier a wavefront waits for its own A-tile DMAs explicitly: the wait the
     // compiler derives for them may be placed behind the barrier, where it no longer says anything
     // about the fragments the OTHER wavefronts moved.
-    for (int kt = kt_begin; kt < KT; kt += 2)
+    if constexpr (!PERSIST)
     {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
-        compute(a_buf0, st0, st1, a_buf1, kt + 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        compute(a_buf1, st1, st0, a_buf0, kt + 2); // past the end of K both operands read as zeros: no branch needed
+        for (int kt = kt_begin; kt < KT; kt += 2)
+        {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads(); // A(kt) has landed for every wavefront; everyone is done reading buffer 1
+            compute(std::false_type{}, a_buf0, st0, st1, a_buf1, kt + 1);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            compute(std::false_type{}, a_buf1, st1, st0, a_buf0, kt + 2); // past the end of K both operands read as zeros: no branch needed
+        }
+    }
+    else
+    {
+        // Tiles one after the other (KT is even: every tile starts on buffer 0).  The second tile row
+        // of a tile's last pair requests tile row 0 of the NEXT tile: the per-tile values are switched
+        // over right before it - its own matrix instructions need operands and accumulators only.
+        // Straight-line code around a plain inner loop (KT >= 4): the first tile row, the second, the
+        // pairs in between, and the last pair with the switch-over.  A branch that chose between the
+        // first-tile-row code and the ordinary one inside the loop, or a loop left from its middle,
+        // makes the allocator keep second copies of the accumulators, and all 256 AGPRs are theirs.
+        auto step_barrier = [&]()
+        {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+        };
+        do
+        {
+            step_barrier();
+            compute(std::true_type{}, a_buf0, st0, st1, a_buf1, 1);
+            step_barrier();
+            compute(std::false_type{}, a_buf1, st1, st0, a_buf0, 2);
+            for (int kt = 2; kt < KT - 2; kt += 2)
+            {
+                step_barrier();
+                compute(std::false_type{}, a_buf0, st0, st1, a_buf1, kt + 1);
+                step_barrier();
+                compute(std::false_type{}, a_buf1, st1, st0, a_buf0, kt + 2);
+            }
+            step_barrier();
+            compute(std::false_type{}, a_buf0, st0, st1, a_buf1, KT - 1);
+            step_barrier();
+            {
+                {
+                    // this tile's outputs: stored during the next tile's first tile row (or below)
+                    prev_off = ((uint32_t) (m0 + c) * (uint32_t) p.n + (uint32_t) (strip0 * 16 + kg * 4)) * 2u;
+                    vb += (int) gridDim.x;
+                    if (tile_of(vb, tm, tn))
+                    {
+                        m0 = tm * kGemmBM;
+                        strip0 = tn * (kGemmBN / 16) + wave * NS;
+#pragma unroll
+                        for (int s = 0; s < NS; ++s)
+                        {
+                            strip_of[s] = paired_strip(false, strip0, s, p.strips, strip_ok[s]);
+                            wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
+                            sc_lane[s] = (uint32_t) (strip_of[s] * 16 + c) * 2u;
+                            if constexpr (GROUP == 0)
+                            {
+                                pc_scale_n[s] = E::load(p.scales, strip_of[s] * 16 + c);
+                                pc_scale2_n[s]
+                                    = (uint32_t) static_cast<uint16_t const*>(p.scales)[strip_of[s] * 16 + c] * 0x10001u;
+                            }
+                        }
+                        dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
+                                            + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
+                            * 2u;
+                    }
+                    else
+                        tile_oob = kOob;
+                }
+                compute(std::false_type{}, a_buf1, st1, st0, a_buf0, 0);
+            }
+            if constexpr (GROUP == 0)
+            {
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    pc_scale[s] = pc_scale_n[s];
+                    pc_scale2[s] = pc_scale2_n[s];
+                }
+            }
+        } while (!tile_oob);
+        // the last tile's outputs
+        mma_drain();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                store_block(rt, s);
+        return;
     }
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
@@ -531,12 +674,31 @@ int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;
+        note_launch("gemm exact rt=%d splits=%d persistent=0", RT, gp.k_splits);
         hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, true>), grid, block, 0, stream, gp);
         hipLaunchKernelGGL((gemm_finish_partial<DT>), dim3((unsigned) ((count / 4 + 255) / 256)), block, 0, stream,
             gp.out, gp.partial, gp.bias, gp.alpha, gp.m, gp.n, gp.k_splits);
     }
     else
-        hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);
+    {
+        // prefill-sized problems: one persistent workgroup per CU when that means at least two tiles each
+        int const cus = gemm_persistent_workgroups();
+        bool persist = false;
+        if constexpr (RT == 16)
+            persist = cus > 0 && total > cus && gp.k_tiles % 2 == 0 && gp.k_tiles >= 4 && gp.n % kGemmBN == 0
+                && !gp.bias && !gp.expert_rows && gp.num_experts == 0 && gp.activation == kActIdentity && !gp.residual
+                && (uint64_t) gp.m * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 31)
+                // byte offsets of the padded last row tile, and of the rejected offset plus 15 row tiles, stay below 2^32
+                && (uint64_t) gp.tiles_m * (RT * 16) * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 32) && gp.n < (1 << 22);
+        note_launch("gemm exact rt=%d splits=1 persistent=%d", RT, (int) persist);
+        if (persist)
+        {
+            if constexpr (RT == 16)
+                hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false, true>), dim3(cus), block, 0, stream, gp);
+        }
+        else
+            hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);
+    }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "gemm kernel launch failed: %s", hipGetErrorString(err));

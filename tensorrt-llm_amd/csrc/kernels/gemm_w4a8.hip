@@ -302,6 +302,7 @@ int launch_w4a8_variant(GemmParams const& gp, hipStream_t stream)
 {
     int const total = gp.tiles_m * gp.tiles_n;
     dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(256);
+    note_launch("gemm w4a8 rt=%d splits=%d", RT, gp.k_splits);
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;

@@ -545,6 +545,7 @@ int launch_skinny_rt(GemmParams const& gp, hipStream_t stream)
 {
     int const total = gp.tiles_m * gp.tiles_n;
     dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(kSkinnyWaves * 64), block256(256);
+    note_launch("gemm skinny rt=%d splits=%d", RT, gp.k_splits);
     if (gp.k_splits > 1)
     {
         size_t const count = (size_t) gp.m * gp.n;

@@ -867,6 +867,9 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8, GROUPED ? sp.num_experts : sp.k_slices), block(WAVES * 64);
+    note_launch(GROUPED ? "stream grouped mt=%d ns=%d waves=%d pf=%d slots=%d experts=%d"
+                        : "stream mt=%d ns=%d waves=%d pf=%d slots=%d k_slices=%d",
+        MT, NS, WAVES, PF, SLOTS, GROUPED ? sp.num_experts : sp.k_slices);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)

@@ -326,6 +326,7 @@ int launch_variant(StreamParams sp, hipStream_t stream)
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    note_launch("stream w4a8 ns=%d waves=%d pf=%d lds=%d", NS, WAVES, PF, LDSM);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)

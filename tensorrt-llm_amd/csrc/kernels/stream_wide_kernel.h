@@ -342,6 +342,7 @@ int launch_stream_wide_variant(StreamParams sp, hipStream_t stream)
     sp.groups = (sp.strips + NS * WAVES - 1) / (NS * WAVES); // workgroups
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    note_launch("stream wide ns=%d waves=%d pf=%d slots=%d", NS, WAVES, PF, SLOTS);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)

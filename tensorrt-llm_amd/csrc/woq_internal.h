@@ -17,6 +17,10 @@ namespace woq
 // records a message for woq_last_error() on this thread and returns `code`
 int fail(int code, char const* fmt, ...) __attribute__((format(printf, 2, 3)));
 
+// remembers what woq_last_launch() reports for this thread (`fmt` must be a string literal with up
+// to six %d; formatted only when asked for)
+void note_launch(char const* fmt, int a = 0, int b = 0, int c = 0, int d = 0, int e = 0, int f = 0);
+
 inline int bits_of(int quant_type)
 {
     return quant_type == WOQ_W8_A16 ? 8 : 4;
@@ -25,7 +29,7 @@ inline int bits_of(int quant_type)
 // Experiment overrides from the environment, read once (at first use) and again by woq_reload_env():
 //   WOQ_FORCE_REGIME=stream|gemm      WOQ_STREAM_SHAPE=ns,waves,pf,lds   WOQ_WIDE_SHAPE=ns,waves,pf | 0
 //   WOQ_STREAM_SLOTS=0                WOQ_GEMM_KERNEL=exact|skinny       WOQ_GEMM_RT=4|8|16
-//   WOQ_GEMM_SPLITS=<n>               WOQ_STREAM_SPLITS=<n>
+//   WOQ_GEMM_SPLITS=<n>               WOQ_STREAM_SPLITS=<n>              WOQ_GEMM_PERSIST=0
 struct EnvOverrides
 {
     int regime = 0;                // woq_regime; 0 = none
@@ -38,6 +42,7 @@ struct EnvOverrides
     int gemm_rt = 0;               // row tiles per wavefront of the exact-dequantize / fp8 kernel
     int gemm_splits = 0;           // K split of the GEMM regime
     int stream_splits = 0;         // K slices of the streaming kernel (0 = built-in rule)
+    bool persist_off = false;      // WOQ_GEMM_PERSIST=0: no persistent prefill kernels
 };
 EnvOverrides const& env_overrides();
 

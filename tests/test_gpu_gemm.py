@@ -162,3 +162,42 @@ def test_gemm_flexible_group_sizes(pkg, oracle, dev, m, n, k, dtype, pqs, zero, 
     assert p["scales"].shape[0] == -(-k // group)
     err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
+
+
+def _last_launch(pkg):
+    return (pkg._lib.lib.woq_last_launch() or b"").decode()
+
+
+# more 256 x 256 tiles than the chip has CUs, N a multiple of 256, an even number (>= 4) of weight tile
+# rows, no bias: the shapes that take the persistent kernel; M ragged against the tile and against 16
+PERSISTENT = [(4000, 512, 8192, 4, 128, "bf16", True), (2250, 1024, 16384, 4, 64, "fp16", True),
+              (2250, 960, 16384, 4, 64, "bf16", False), (4096, 512, 8192, 8, 0, "fp16", False),
+              (3000, 256, 12288, 8, 128, "bf16", True), (2304, 1024, 8192, 4, 0, "bf16", False)]
+
+
+@pytest.mark.parametrize("m,k,n,bits,group,dtype,zero", PERSISTENT)
+def test_gemm_persistent_tile_loop(pkg, oracle, dev, woq_env, gemm_kernel, m, k, n, bits, group, dtype, zero):
+    """One workgroup per CU walking several tiles (the next tile's first loads requested during the
+    current tile's last tile row, the outputs stored between the next tile's first matrix
+    instructions) returns the bits of the one-tile-per-workgroup launch, which in turn meets the
+    oracle's bar."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel has no persistent form")
+    p = random_problem(oracle, m, k, n, bits, group, dtype, zero=zero, seed=m + k)
+    out = run_product(pkg, oracle, dev, p, GEMM)
+    assert "persistent=1" in _last_launch(pkg), _last_launch(pkg)
+    woq_env(WOQ_GEMM_PERSIST="0")
+    plain = run_product(pkg, oracle, dev, p, GEMM)
+    assert "persistent=0" in _last_launch(pkg), _last_launch(pkg)
+    assert (out.view(np.uint32) == plain.view(np.uint32)).all()
+    assert parity_err(oracle, out, p) < TOL
+
+
+def test_gemm_persistent_needs_whole_tiles_and_no_bias(pkg, oracle, dev, gemm_kernel):
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel has no persistent form")
+    for n, bias in [(8192 + 16, False), (8192, True)]:
+        p = random_problem(oracle, 4000, 512, n, 4, 128, "bf16", zero=True, bias=bias, seed=n)
+        out = run_product(pkg, oracle, dev, p, GEMM)
+        assert "persistent=0" in _last_launch(pkg), _last_launch(pkg)
+        assert parity_err(oracle, out, p) < TOL
