@@ -131,11 +131,76 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // operands of step kt+1 (32 half-operands of 4 weights), then the 4 MFMAs of row tile rt.
     constexpr int A_AHEAD = 2;
     auto slab_at = [](int pos) { return ((pos & 1) << 1) | (pos >> 1); }; // its own inverse
-    // conversion unit cu = (strip, slab, half, pair): 2 weights -> 16 bits of the operand set
+    // conversion unit cu = (strip, slab, half, pair): 2 weights -> 16 bits of the operand set.  The
+    // same arithmetic as dequant2_fp8 (w4a8_common.h), cut into four stages so that the main loop can
+    // run each stage of a unit behind a different matrix instruction: issued back to back, every
+    // instruction of the chain mask -> byte-to-float -> FMA -> pack waits for the one before it.
+    struct ConvState
+    {
+        uint32_t src[2][2]; // masked / sign-flipped source word of (slab parity, pair)
+        float v[16][2];     // the two values of the units in flight (unit % 16: at most 12 are)
+    };
+    auto conv_stage = [&](ConvState& cs, u32x8 (&b)[NS], BStage const& st, int cu, int stage)
+    {
+        int const s = cu / 16, j = (cu / 4) % 4, h = (cu / 2) % 2, pr = cu % 2;
+        uint32_t& src = cs.src[j & 1][pr];
+        float(&v)[2] = cs.v[cu % 16];
+        if (stage == 0)
+        {
+            if (h != 0)
+                return; // the unit with h = 0 made the word for both
+            uint32_t const w = st.w[s][j];
+            if constexpr (ZERO)
+                src = pr == 0 ? (w ^ 0x88888888u) : ((w ^ 0x88888888u) >> 4); // biased -> two's complement nibbles
+            else
+                src = (pr == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
+            // opaque: the byte-to-float conversions read the word as it is; and, like the two below, an
+            // anchor in the order of the volatile statements (the matrix instructions): the next stage's
+            // instructions cannot be moved up to this one's
+            asm volatile("" : "+v"(src));
+        }
+        else if (stage == 1)
+        {
+            if constexpr (ZERO)
+            {
+                v[0] = cvt_off_f32_i4_byte(src, h);
+                v[1] = cvt_off_f32_i4_byte(src, h + 2);
+            }
+            else
+            {
+                v[0] = (float) ((src >> (8 * h)) & 0xFF);
+                v[1] = (float) ((src >> (8 * h + 16)) & 0xFF);
+            }
+            asm volatile("" : "+v"(v[0]), "+v"(v[1]));
+        }
+        else if (stage == 2)
+        {
+            float const sc = EH::from_bits(st.s[s]);
+            if constexpr (ZERO)
+            {
+                float const zr = EH::from_bits(st.z[s]);
+                v[0] = __builtin_fmaf(v[0], 16.f * sc, zr);
+                v[1] = __builtin_fmaf(v[1], 16.f * sc, zr);
+            }
+            else
+            {
+                v[0] = __builtin_fmaf(v[0], sc, -8.f * sc);
+                v[1] = __builtin_fmaf(v[1], sc, -8.f * sc);
+            }
+            asm volatile("" : "+v"(v[0]), "+v"(v[1]));
+        }
+        else
+        {
+            int const idx = slab_at(j) * 2 + h; // slab j sits at operand position slab_at(j)
+            b[s][idx] = pr == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) b[s][idx], false)
+                                : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) b[s][idx], true);
+        }
+    };
+    // all four stages of one unit at once (prologue)
     auto convert_unit = [&](u32x8 (&b)[NS], BStage const& st, int cu)
     {
         int const s = cu / 16, j = (cu / 4) % 4, h = (cu / 2) % 2, pr = cu % 2;
-        int const idx = slab_at(j) * 2 + h; // slab j sits at operand position slab_at(j)
+        int const idx = slab_at(j) * 2 + h;
         float const sc = EH::from_bits(st.s[s]);
         float const zr = ZERO ? EH::from_bits(st.z[s]) : 0.f;
         b[s][idx] = dequant2_fp8<ZERO, false>(b[s][idx], st.w[s][j], h, pr, sc, zr);
@@ -166,6 +231,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
         for (int i = 0; i < A_AHEAD && i < RT; ++i)
             a_ring[i] = a_read(i);
+        // the conversion pipeline's head: the stages that the first matrix instructions expect done
+        constexpr int PER0 = UNITS / (RT * NS);
+        ConvState cs;
+#pragma unroll
+        for (int lead = 0; lead < 3; ++lead)
+#pragma unroll
+            for (int stage = 0; stage < 3 - lead; ++stage)
+#pragma unroll
+                for (int x = 0; x < PER0; ++x)
+                    if (lead * PER0 + x < UNITS)
+                        conv_stage(cs, b_make, st_conv, lead * PER0 + x, stage);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
@@ -199,10 +275,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
                 else
                     mma_fp8_acc(b_use[s], a_cur, acc[rt][s]);
+                // behind matrix instruction t: the pack of the units whose FMAs went behind t - 1, the
+                // FMAs of those converted behind t - 2, and so on (PER units per instruction)
                 constexpr int PER = UNITS / (RT * NS);
+                int const t = rt * NS + s;
 #pragma unroll
-                for (int cu = (rt * NS + s) * PER; cu < (rt * NS + s + 1) * PER; ++cu)
-                    convert_unit(b_make, st_conv, cu);
+                for (int stage = 3; stage >= 0; --stage)
+#pragma unroll
+                    for (int x = 0; x < PER; ++x)
+                    {
+                        int const cu = (t + 3 - stage) * PER + x;
+                        if (cu < UNITS)
+                            conv_stage(cs, b_make, st_conv, cu, stage);
+                    }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
