@@ -269,7 +269,7 @@ def bench_gemm(pkg, dev, m=4096, reps=40):
                     # the M = 4096 half of the metric in the shape of `roofline`
                     roofline={"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                              "kernel": "gemm_kernel<bf16,int4,g128,zeros,RT=16> on gate_up K=%d N=%d M=%d" % (k, n, m),
+                              "kernel": "gemm_kernel<bf16,int4,g128,zeros,RT=16,persistent> on gate_up K=%d N=%d M=%d" % (k, n, m),
                               "flop_per_launch": 2.0 * m * n * k, "us_per_launch": round(sec * 1e6, 1)})
     except Exception as e:  # the decode line is still valid without the prefill extra
         return dict(error=str(e)[:200])

@@ -282,6 +282,22 @@ int woq_unpreprocess_weights(void* dst_row_major, const void* src, int64_t exper
 int woq_import_reference_weights(void* dst_row_major, const void* src_reference_layout, int64_t experts, int64_t k,
     int64_t n, int32_t quant_type, int32_t arch);
 
+/* The single steps of the reference's preprocess on packed row-major weights, as its torch debug
+ * operators expose them (thop/weightOnlyQuantOp.cpp:65-120, 252-281, 371-385; the steps themselves
+ * cutlass_preprocessors.cpp:186-240 permute_B_rows_for_mixed_gemm, :245-385 subbyte_transpose,
+ * :404-507 add_bias_and_interleave_quantized_tensor_inplace).  [experts][k][n] elements of the
+ * quant type's width in `src`; `dst` (same size, must not alias) receives the step's result:
+ * PERMUTE_ROWS keeps the shape, SUBBYTE_TRANSPOSE writes [experts][n][k], ADD_BIAS_AND_INTERLEAVE
+ * works on the flat buffer.  Nothing on the matmul path uses them. */
+enum woq_ref_step
+{
+    WOQ_REF_STEP_PERMUTE_ROWS = 0,
+    WOQ_REF_STEP_SUBBYTE_TRANSPOSE = 1,
+    WOQ_REF_STEP_ADD_BIAS_AND_INTERLEAVE = 2
+};
+int woq_reference_layout_step(void* dst, const void* src, int64_t experts, int64_t k, int64_t n, int32_t quant_type,
+    int32_t step);
+
 /* Per-column symmetric quantizer + preprocess.  Replaces symmetric_quantize<ComputeType, WeightType>
  * (cutlass_preprocessors.cpp:652-762) behind trtllm::symmetric_quantize_last_axis_of_batched_matrix
  * and trtllm::_symmetric_quantize_last_axis_of_batched_matrix (thop/weightOnlyQuantOp.cpp:153-251).

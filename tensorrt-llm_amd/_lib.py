@@ -72,6 +72,7 @@ def _load():
         "woq_preprocess_weights": (ctypes.c_int, [vp, vp, i64, i64, i64, i32]),
         "woq_unpreprocess_weights": (ctypes.c_int, [vp, vp, i64, i64, i64, i32]),
         "woq_import_reference_weights": (ctypes.c_int, [vp, vp, i64, i64, i64, i32, i32]),
+        "woq_reference_layout_step": (ctypes.c_int, [vp, vp, i64, i64, i64, i32, i32]),
         "woq_symmetric_quantize": (ctypes.c_int, [vp, vp, vp, vp, i64, i64, i64, i32, i32, i32]),
         "woq_pack_int4": (ctypes.c_int, [vp, vp, sz]),
         "woq_unpack_int4": (ctypes.c_int, [vp, vp, sz]),

@@ -483,6 +483,85 @@ extern "C" int woq_import_reference_weights(void* dst_row_major, const void* src
     return WOQ_OK;
 }
 
+extern "C" int woq_reference_layout_step(void* dst, const void* src, int64_t experts, int64_t k, int64_t n,
+    int32_t quant_type, int32_t step)
+{
+    if (!dst || !src)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_reference_layout_step: null pointer");
+    if (quant_type != WOQ_W8_A16 && quant_type != WOQ_W4_A16 && quant_type != WOQ_W4_AFP8)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown quant_type %d", quant_type);
+    int const bits = bits_of(quant_type);
+    if (experts < 1 || k < 1 || n < 1 || (k * n * bits) % 32)
+        return fail(WOQ_ERR_BAD_SHAPE, "shape [%lld, %lld] does not fill whole 32-bit words", (long long) k, (long long) n);
+    size_t const mat_bytes = (size_t) (k * n * bits / 8);
+    auto const* s8 = static_cast<uint8_t const*>(src);
+    auto* d8 = static_cast<uint8_t*>(dst);
+    if (step == WOQ_REF_STEP_PERMUTE_ROWS)
+    {
+        // rows move inside blocks of 16 (int8) / 32 (int4) rows: written row i of a block is read row perm[i]
+        int const plen = quant_type == WOQ_W8_A16 ? 16 : 32;
+        int const* perm = quant_type == WOQ_W8_A16 ? kPermW8 : (quant_type == WOQ_W4_A16 ? kPermW4 : kPermW4A8);
+        if (k % plen)
+            return fail(WOQ_ERR_BAD_SHAPE,
+                "Invalid shape for quantized tensor. Number of rows of quantized matrix must be a multiple of %d", plen);
+        if (n % 8)
+            return fail(WOQ_ERR_BAD_SHAPE,
+                "Invalid shape for quantized tensor. On turing/Ampere, the number of cols must be a multiple of 8.");
+        size_t const row_bytes = (size_t) (n * bits / 8);
+        for (int64_t ex = 0; ex < experts; ++ex)
+            parallel_for(k,
+                [&](int64_t row)
+                {
+                    int64_t const from = row - row % plen + perm[row % plen];
+                    std::memcpy(d8 + ex * mat_bytes + row * row_bytes, s8 + ex * mat_bytes + from * row_bytes, row_bytes);
+                });
+        return WOQ_OK;
+    }
+    if (step == WOQ_REF_STEP_SUBBYTE_TRANSPOSE)
+    {
+        // [k][n] -> [n][k] element by element (two int4 elements share a byte on both sides)
+        if ((n * bits) % 8 || (k * bits) % 8)
+            return fail(WOQ_ERR_BAD_SHAPE, "rows and columns must fill whole bytes");
+        for (int64_t ex = 0; ex < experts; ++ex)
+        {
+            std::memset(d8 + ex * mat_bytes, 0, mat_bytes);
+            // output rows (= input columns) are disjoint between threads
+            parallel_for(n,
+                [&](int64_t col)
+                {
+                    for (int64_t row = 0; row < k; ++row)
+                        write_signed(d8 + ex * mat_bytes, col, row, k, bits,
+                            read_signed(s8 + ex * mat_bytes, row, col, n, bits));
+                });
+        }
+        return WOQ_OK;
+    }
+    if (step == WOQ_REF_STEP_ADD_BIAS_AND_INTERLEAVE)
+    {
+        // every element becomes unsigned (+128 / +8); inside each 32-bit word the elements are then
+        // reordered: int8 [0, 2, 1, 3], int4 [0, 2, 4, 6, 1, 3, 5, 7] (written position <- element)
+        int const per_word = 32 / bits;
+        int const bias = 1 << (bits - 1);
+        size_t const words = (size_t) experts * mat_bytes / 4;
+        parallel_for((int64_t) words,
+            [&](int64_t w)
+            {
+                uint8_t const* in = s8 + w * 4;
+                uint32_t out = 0;
+                for (int pos = 0; pos < per_word; ++pos)
+                {
+                    int const elt = pos < per_word / 2 ? 2 * pos : 2 * (pos - per_word / 2) + 1;
+                    int const nib = (in[elt >> 1] >> ((elt & 1) * 4)) & 0xF;
+                    int const v = bits == 8 ? (int) (int8_t) in[elt] : (nib >= 8 ? nib - 16 : nib);
+                    out |= (uint32_t) ((v + bias) & ((1 << bits) - 1)) << (pos * bits);
+                }
+                std::memcpy(d8 + w * 4, &out, 4);
+            });
+        return WOQ_OK;
+    }
+    return fail(WOQ_ERR_INVALID_ARGUMENT, "unknown step %d", step);
+}
+
 extern "C" int woq_symmetric_quantize(void* processed, void* unprocessed, void* scales, const void* weight,
     int64_t experts, int64_t k, int64_t n, int32_t quant_type, int32_t weight_dtype, int32_t scale_dtype)
 {

@@ -8,6 +8,10 @@ cpp/tensorrt_llm/thop/weightOnlyQuantOp.cpp:123-363 (`torch.ops.trtllm.*`):
     preprocess_weights_for_mixed_gemm(weight, quant_type, activation_type) -> processed
     unpack_int4_packed_tensor_to_int8(weight) / pack_int8_tensor_to_packed_int4(weight)
 
+    _permute_B_rows_for_mixed_gemm(weight, quant_type, arch) / _subbyte_transpose(weight, quant_type)
+    _add_bias_and_interleave_int4s(weight) / _add_bias_and_interleave_int8s(weight)
+        (the reference's test-only operators, :65-120, :252-281: single steps of ITS preprocess)
+
 plus two that have no counterpart there: `unprocess_weights_for_mixed_gemm` (inverse of the
 gfx950 layout) and `import_reference_weights` (decode a buffer the REFERENCE preprocessed).
 
@@ -119,6 +123,49 @@ def import_reference_weights(reference_processed: torch.Tensor, quant_type: torc
     return out
 
 
+def _reference_step(weight: torch.Tensor, qt: int, step: int) -> torch.Tensor:
+    _check_cpu_contiguous(weight, "Quantized tensor")
+    if weight.dtype != torch.int8:
+        raise RuntimeError("Quantized tensor must be int8 dtype")
+    experts, k, n = _dims(weight, _bits(qt))
+    out = torch.empty_like(weight)
+    check(lib.woq_reference_layout_step(out.data_ptr(), weight.data_ptr(), experts, k, n, qt, step))
+    return out
+
+
+def _permute_B_rows_for_mixed_gemm(quantized_tensor: torch.Tensor, quant_type: torch.dtype,
+                                   arch_version: int) -> torch.Tensor:
+    """Row permutation of the reference's preprocess (blocks of 16 int8 / 32 int4 rows) on packed
+    row-major weights; `arch_version` is accepted and, as in the reference's function, not consulted."""
+    return _reference_step(quantized_tensor, _quant_type(quant_type), 0)
+
+
+def _subbyte_transpose(quantized_tensor: torch.Tensor, quant_type: torch.dtype) -> torch.Tensor:
+    """Element-granular transpose of packed weights: the result has the input's tensor shape (as in the
+    reference) and holds [n][k] elements."""
+    return _reference_step(quantized_tensor, _quant_type(quant_type), 1)
+
+
+def _add_bias_and_interleave(weight: torch.Tensor, qt: int) -> torch.Tensor:
+    _check_cpu_contiguous(weight)
+    if weight.numel() == 0:
+        raise RuntimeError("weight should not be empty tensor")
+    if weight.dtype != torch.int8:
+        raise RuntimeError("Weight must be a packed int8 tensor" if qt == _lib.W4_A16 else "Weight must be an int8 tensor")
+    out = torch.empty_like(weight)
+    elts = weight.numel() * (8 // _bits(qt))
+    check(lib.woq_reference_layout_step(out.data_ptr(), weight.data_ptr(), 1, 1, elts, qt, 2))
+    return out
+
+
+def _add_bias_and_interleave_int4s(weight: torch.Tensor) -> torch.Tensor:
+    return _add_bias_and_interleave(weight, _lib.W4_A16)
+
+
+def _add_bias_and_interleave_int8s(weight: torch.Tensor) -> torch.Tensor:
+    return _add_bias_and_interleave(weight, _lib.W8_A16)
+
+
 def _symmetric_quantize_helper(weight: torch.Tensor, quant_type: torch.dtype, return_unprocessed: bool):
     _check_cpu_contiguous(weight)
     if weight.numel() == 0:
@@ -166,6 +213,11 @@ def _register_torch_ops() -> None:
              preprocess_weights_for_mixed_gemm),
         "unpack_int4_packed_tensor_to_int8": ("(Tensor weight) -> Tensor", unpack_int4_packed_tensor_to_int8),
         "pack_int8_tensor_to_packed_int4": ("(Tensor weight) -> Tensor", pack_int8_tensor_to_packed_int4),
+        "_permute_B_rows_for_mixed_gemm":
+            ("(Tensor quantized_tensor, ScalarType quant_type, int arch_version) -> Tensor", _permute_B_rows_for_mixed_gemm),
+        "_subbyte_transpose": ("(Tensor quantized_tensor, ScalarType quant_type) -> Tensor", _subbyte_transpose),
+        "_add_bias_and_interleave_int4s": ("(Tensor weight) -> Tensor", _add_bias_and_interleave_int4s),
+        "_add_bias_and_interleave_int8s": ("(Tensor weight) -> Tensor", _add_bias_and_interleave_int8s),
     }
     for name, (schema, fn) in defs.items():
         qual = "trtllm::" + name
@@ -177,6 +229,7 @@ def _register_torch_ops() -> None:
 
 REGISTERED_TORCH_OPS = ("symmetric_quantize_last_axis_of_batched_matrix", "_symmetric_quantize_last_axis_of_batched_matrix",
                         "preprocess_weights_for_mixed_gemm", "unpack_int4_packed_tensor_to_int8",
-                        "pack_int8_tensor_to_packed_int4")
+                        "pack_int8_tensor_to_packed_int4", "_permute_B_rows_for_mixed_gemm", "_subbyte_transpose",
+                        "_add_bias_and_interleave_int4s", "_add_bias_and_interleave_int8s")
 
 _register_torch_ops()

@@ -12,6 +12,10 @@ TOL = 1e-2
 GEMM = 2
 
 
+def _last_launch(pkg):
+    return (pkg._lib.lib.woq_last_launch() or b"").decode()
+
+
 @pytest.fixture(params=["exact", "skinny"], autouse=True)
 def gemm_kernel(request, woq_env):
     """The GEMM regime has two kernels (exact-dequantize 256-row tiles, deferred-scale 64-row tiles);
@@ -79,6 +83,38 @@ def test_gemm_identity_recovers_dequantized_weight_exactly(pkg, oracle, dev, gem
         out = run_product(pkg, oracle, dev, p, GEMM)
         w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 64, dtype)
         assert (out.view(np.uint32) == w.view(np.uint32)).all(), dtype
+
+
+@pytest.mark.parametrize("rt", [4, 8, 16])
+@pytest.mark.parametrize("bits,dtype", [(4, "bf16"), (4, "fp16"), (8, "bf16")])
+def test_gemm_identity_every_tile_height(pkg, oracle, dev, woq_env, gemm_kernel, rt, bits, dtype):
+    """The same bit-exact identity at every tile height (64 / 128 / 256 rows): the accumulators are read
+    behind hand-placed waits that the compiler does not see, and a missed one would show here."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel applies scales to float32 sums, not to single weights")
+    woq_env(WOQ_GEMM_RT=str(rt))
+    K, N = 256, 512
+    p = random_problem(oracle, K, K, N, bits, 64, dtype, zero=True, seed=rt + bits)
+    p["act"] = np.eye(K, dtype=np.float32)
+    out = run_product(pkg, oracle, dev, p, GEMM)
+    assert "rt=%d" % rt in _last_launch(pkg), _last_launch(pkg)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 64, dtype)
+    assert (out.view(np.uint32) == w.view(np.uint32)).all()
+
+
+def test_gemm_identity_through_the_persistent_loop(pkg, oracle, dev, gemm_kernel):
+    """Identity activation on a shape that takes the persistent kernel (258 tiles): the first matrix
+    instruction of every tile starts a fresh sum and the finished tile leaves through the explicit
+    accumulator reads - bit for bit the dequantized weight."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel has no persistent form")
+    K, N = 512, 256 * 129
+    p = random_problem(oracle, K, K, N, 4, 128, "bf16", zero=True, seed=21)
+    p["act"] = np.eye(K, dtype=np.float32)
+    out = run_product(pkg, oracle, dev, p, GEMM)
+    assert "persistent=1" in _last_launch(pkg), _last_launch(pkg)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")
+    assert (out.view(np.uint32) == w.view(np.uint32)).all()
 
 
 def test_gemm_matches_stream_kernel(pkg, oracle, dev):
@@ -162,10 +198,6 @@ def test_gemm_flexible_group_sizes(pkg, oracle, dev, m, n, k, dtype, pqs, zero, 
     assert p["scales"].shape[0] == -(-k // group)
     err = parity_err(oracle, run_product(pkg, oracle, dev, p, GEMM), p)
     assert err < TOL, err
-
-
-def _last_launch(pkg):
-    return (pkg._lib.lib.woq_last_launch() or b"").decode()
 
 
 # more 256 x 256 tiles than the chip has CUs, N a multiple of 256, an even number (>= 4) of weight tile

@@ -159,3 +159,48 @@ def test_every_op_is_reachable_through_torch_ops_trtllm(pkg):
     # the fp8 activation type selects the W4A8 flavour (get_ft_quant_type, thop/weightOnlyQuantOp.cpp:41-62)
     a8 = T.preprocess_weights_for_mixed_gemm(packed.repeat(8, 2).contiguous(), torch.quint4x2, torch.float8_e4m3fn)
     assert a8.shape == (128, 32)
+
+
+def _packed(oracle, q, bits):
+    return torch.from_numpy(q if bits == 8 else oracle.pack_int8_tensor_to_packed_int4(q))
+
+
+def _unpacked(oracle, t, bits):
+    return t.numpy() if bits == 8 else oracle.unpack_int4_packed_tensor_to_int8(t.numpy())
+
+
+@pytest.mark.parametrize("name,qt", [("W8_A16", torch.int8), ("W4_A16", torch.quint4x2)])
+def test_reference_debug_ops_step_by_step(pkg, oracle, name, qt):
+    """The reference's test-only operators (thop/weightOnlyQuantOp.cpp:371-385), called by their
+    torch.ops.trtllm names: each step against plain numpy indexing on the unpacked elements, and their
+    composition (permute, transpose, bias + word interleave - the reference's order without the column
+    interleave, which is what its preprocess does for SM90) against the oracle's byte stream."""
+    T = torch.ops.trtllm
+    bits = oracle.weight_bits(name)
+    K, N = 128, 192
+    rng = np.random.default_rng(bits)
+    q = rng.integers(-(1 << (bits - 1)), 1 << (bits - 1), size=(K, N)).astype(np.int8)
+    perm = np.asarray(oracle._PERM[name])
+    permuted = T._permute_B_rows_for_mixed_gemm(_packed(oracle, q, bits), qt, 80)
+    want = q.reshape(K // perm.size, perm.size, N)[:, perm, :].reshape(K, N)
+    assert (_unpacked(oracle, permuted, bits) == want).all()
+    transposed = T._subbyte_transpose(permuted, qt)
+    assert transposed.shape == permuted.shape  # the reference keeps the tensor shape; the elements are [N][K]
+    assert (_unpacked(oracle, transposed.reshape(N, -1), bits) == want.T).all()
+    interleave = T._add_bias_and_interleave_int8s if bits == 8 else T._add_bias_and_interleave_int4s
+    final = interleave(transposed)
+    flat = want.T.reshape(-1).astype(np.int32) + (1 << (bits - 1))
+    order = np.asarray(oracle._WORD_ORDER[bits])
+    flat = flat.reshape(-1, order.size)[:, order].reshape(-1)
+    assert (final.numpy().view(np.uint8).reshape(-1) == oracle._pack_unsigned(flat, bits)).all()
+    assert (final.numpy().view(np.uint8).reshape(-1) == oracle.ref_preprocess(q, name, 90)).all()
+    # three-dimensional input: every expert on its own
+    q3 = np.stack([q, np.roll(q, 1, axis=0)])
+    p3 = T._permute_B_rows_for_mixed_gemm(_packed(oracle, q3.reshape(-1, N), bits).reshape(2, K, -1), qt, 80)
+    assert torch.equal(p3[0], permuted)
+    t3 = T._subbyte_transpose(p3, qt)
+    assert torch.equal(t3[0], transposed)
+    with pytest.raises(RuntimeError, match="multiple of"):
+        T._permute_B_rows_for_mixed_gemm(_packed(oracle, q[:24], bits), qt, 80)
+    with pytest.raises(RuntimeError, match="int8"):
+        T._subbyte_transpose(torch.zeros((32, 32), dtype=torch.int16), qt)
