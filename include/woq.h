@@ -73,7 +73,9 @@ typedef enum woq_quant_type
 typedef enum woq_regime
 {
     WOQ_REGIME_AUTO = 0,
-    WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 16) */
+    WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 16); with 4 to
+                              16 rows on long-K / narrow-N shapes they split K through the workspace when
+                              it is large enough, and run unsplit when it is not */
     WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMMs: deferred-scale 32/64-row tiles or exact-dequantize 64/128/256-row
                               tiles (whichever is estimated cheaper for the shape), the fp8 kernel for W4A8;
                               may split K through the workspace */
@@ -156,7 +158,8 @@ size_t woq_static_scratch_bytes(void);
 /* Device scratch that is enough for every woq_matmul call of this n, k, quant_algo with AT MOST m
  * rows (pass the largest m, as the reference passes its profile's maxM): a region for smoothed
  * activations (PRE_QUANT_SCALE, GEMM regime) followed by the float32 partial sums of the
- * split-K GEMM that skinny problems use (one [m, n] slab per slice of K, summed in slice order, so
+ * split-K GEMM that skinny problems use, or of the streaming kernels' K split at 4 to 16 rows (one
+ * [m, n] slab per slice of K, summed in slice order, so
  * results are bit-reproducible from run to run; the reference's split-K workspace).  Replaces
  * CutlassFpAIntBGemmRunner::getWorkspaceSize (fpA_intB_gemm_template.h:549-582) plus the
  * plugin's own m*k*sizeof(half) smoothing buffer (weightOnlyGroupwiseQuantMatmulPlugin.cpp:377-379). */

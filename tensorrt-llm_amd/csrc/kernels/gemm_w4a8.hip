@@ -43,7 +43,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int t;
     if (!xcd_tile(p.tiles_m * p.tiles_n, t))
         return;
-    int const tm = t % p.tiles_m, tn = t / p.tiles_m;
+    // m fastest inside groups of 4 m-tiles: the 32 workgroups of an XCD then cover about 4 x 8 tiles and
+    // share 4 activation panels and 8 weight panels in its L2 instead of all 16 activation panels and 2
+    constexpr int kGroupM = 4;
+    int const in_group = kGroupM * p.tiles_n;
+    int const first_m = (t / in_group) * kGroupM;
+    int const gsz = p.tiles_m - first_m < kGroupM ? p.tiles_m - first_m : kGroupM;
+    int const tm = first_m + (t % in_group) % gsz, tn = (t % in_group) / gsz;
 
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -135,61 +141,68 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // same arithmetic as dequant2_fp8 (w4a8_common.h), cut into four stages so that the main loop can
     // run each stage of a unit behind a different matrix instruction: issued back to back, every
     // instruction of the chain mask -> byte-to-float -> FMA -> pack waits for the one before it.
+    NibbleConsts const nib = nibble_consts<WOQ_FP16>(); // 0x000F000F in an SGPR, 0x64006400 (1024 as a pair of halves) in a VGPR
     struct ConvState
     {
-        uint32_t src[2][2]; // masked / sign-flipped source word of (slab parity, pair)
+        uint32_t src[2][2]; // zero-points: sign-flipped source word of (slab parity, pair)
+        uint32_t pw[16];    // no zero-points: the unit's two nibbles as a pair of halves 1024 + u
         float v[16][2];     // the two values of the units in flight (unit % 16: at most 12 are)
     };
     auto conv_stage = [&](ConvState& cs, u32x8 (&b)[NS], BStage const& st, int cu, int stage)
     {
         int const s = cu / 16, j = (cu / 4) % 4, h = (cu / 2) % 2, pr = cu % 2;
-        uint32_t& src = cs.src[j & 1][pr];
         float(&v)[2] = cs.v[cu % 16];
-        if (stage == 0)
+        if constexpr (ZERO)
         {
-            if (h != 0)
-                return; // the unit with h = 0 made the word for both
-            uint32_t const w = st.w[s][j];
-            if constexpr (ZERO)
-                src = pr == 0 ? (w ^ 0x88888888u) : ((w ^ 0x88888888u) >> 4); // biased -> two's complement nibbles
-            else
-                src = (pr == 0 ? w : (w >> 4)) & 0x0F0F0F0Fu;
-            // opaque: the byte-to-float conversions read the word as it is; and, like the two below, an
-            // anchor in the order of the volatile statements (the matrix instructions): the next stage's
-            // instructions cannot be moved up to this one's
-            asm volatile("" : "+v"(src));
-        }
-        else if (stage == 1)
-        {
-            if constexpr (ZERO)
+            // fma(q, s, z) on the two's-complement nibble: q/16 straight from the nibble, times 16 s
+            uint32_t& src = cs.src[j & 1][pr];
+            if (stage == 0)
+            {
+                if (h != 0)
+                    return; // the unit with h = 0 made the word for both
+                uint32_t const w = st.w[s][j] ^ 0x88888888u; // biased -> two's complement nibbles
+                src = pr == 0 ? w : (w >> 4);
+                // (here and below: an anchor in the order of the volatile statements, i.e. of the matrix
+                // instructions - the next stage's instructions cannot be moved up to this one's)
+                asm volatile("" : "+v"(src));
+            }
+            else if (stage == 1)
             {
                 v[0] = cvt_off_f32_i4_byte(src, h);
                 v[1] = cvt_off_f32_i4_byte(src, h + 2);
+                asm volatile("" : "+v"(v[0]), "+v"(v[1]));
             }
-            else
+            else if (stage == 2)
             {
-                v[0] = (float) ((src >> (8 * h)) & 0xFF);
-                v[1] = (float) ((src >> (8 * h + 16)) & 0xFF);
-            }
-            asm volatile("" : "+v"(v[0]), "+v"(v[1]));
-        }
-        else if (stage == 2)
-        {
-            float const sc = EH::from_bits(st.s[s]);
-            if constexpr (ZERO)
-            {
-                float const zr = EH::from_bits(st.z[s]);
+                float const sc = EH::from_bits(st.s[s]), zr = EH::from_bits(st.z[s]);
                 v[0] = __builtin_fmaf(v[0], 16.f * sc, zr);
                 v[1] = __builtin_fmaf(v[1], 16.f * sc, zr);
+                asm volatile("" : "+v"(v[0]), "+v"(v[1]));
             }
-            else
-            {
-                v[0] = __builtin_fmaf(v[0], sc, -8.f * sc);
-                v[1] = __builtin_fmaf(v[1], sc, -8.f * sc);
-            }
-            asm volatile("" : "+v"(v[0]), "+v"(v[1]));
         }
         else
+        {
+            // q s = fma(1024 + u, s, -1032 s) on the stored nibble u = q + 8: elements e0 = 4h + 2pr and
+            // e0 + 1 sit in nibbles e0/2 and e0/2 + 4, i.e. 16 bits apart - one shift and one and-or
+            // make the pair of halves 0x6400 | u = 1024 + u, which the FMA reads directly.  1024 + u,
+            // 1032 s and the result (15 significant bits) are exact in float32: the same single rounding
+            // to e4m3 as fma(q, s, 0).
+            uint32_t& pw = cs.pw[cu % 16];
+            if (stage == 0)
+            {
+                pw = ((st.w[s][j] >> (4 * (2 * h + pr))) & nib.mask) | nib.magic; // one v_and_or_b32
+                asm volatile("" : "+v"(pw));
+            }
+            else if (stage == 2)
+            {
+                float const sc = EH::from_bits(st.s[s]);
+                f16x2 const pair = bit_cast<f16x2>(pw);
+                v[0] = __builtin_fmaf((float) pair[0], sc, -1032.f * sc);
+                v[1] = __builtin_fmaf((float) pair[1], sc, -1032.f * sc);
+                asm volatile("" : "+v"(v[0]), "+v"(v[1]));
+            }
+        }
+        if (stage == 3)
         {
             int const idx = slab_at(j) * 2 + h; // slab j sits at operand position slab_at(j)
             b[s][idx] = pr == 0 ? (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], (int) b[s][idx], false)
@@ -296,7 +309,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // ---- main loop: two steps per iteration so that LDS buffers, operand sets and weight stages
     // are distinct objects.  Step kt multiplies with operand set kt%2 (converted during step kt-1
     // from weight stage kt%2), converts set (kt+1)%2 from stage (kt+1)%2 and refills stage kt%2
-    // with the packed weights of step kt+2.
+    // with the packed weights of step kt+2.  (Requesting the weights a further step ahead - four
+    // stages - measured the same.)
     BStage st0, st1;
     u32x8 b0[NS], b1[NS];
     fp8_saturation_on(); // the conversions rely on it; off again before the epilogue
