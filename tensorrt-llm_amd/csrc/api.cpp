@@ -312,6 +312,11 @@ EnvOverrides read_env()
         o.slots_off = e[0] == '0';
     if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))
         o.gemm_kernel = !std::strcmp(e, "skinny") ? 2 : 1;
+    if (char const* e = std::getenv("WOQ_GEMM_COLS"))
+    {
+        int const v = std::atoi(e);
+        o.gemm_cols = (v == 192 || v == 256) ? v : 0;
+    }
     if (char const* e = std::getenv("WOQ_GEMM_RT"))
     {
         int const v = std::atoi(e);

@@ -34,6 +34,7 @@ struct GemmParams
     // and writes [m, n/2]; the strips of a wavefront then alternate between the two halves of N
     // (see paired_strip).  Other activations are applied by a separate pass.
     int activation = kActIdentity;
+    int tile_cols = 256; // columns of an output tile of the exact-dequantize kernel (256, or 192 for 256-row tiles)
     void const* residual = nullptr; // [m, n_out] in the output type, added last (no split-K with it)
 };
 

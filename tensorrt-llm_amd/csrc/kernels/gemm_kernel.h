@@ -50,7 +50,7 @@ int gemm_persistent_workgroups();
 //        reuse): neither the first-load latency of a tile nor its burst of 128 KiB of stores is
 //        paid with the matrix core idle.  Plain epilogue only (bias; no activation, no residual);
 //        K must be an even number of tile rows; m * n * 2 < 2 GiB (outputs go through a descriptor).
-template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, bool PERSIST = false>
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, bool PERSIST = false, int NS_ = 4>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_kernel(GemmParams p)
 {
     static_assert(!(PERSIST && SPLITK), "a persistent workgroup owns whole tiles");
@@ -58,7 +58,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
     constexpr int kGemmBM = RT * 16;
-    constexpr int NS = 4;                                        // strips (16 columns) per wavefront
+    constexpr int NS = NS_;       // strips (16 columns) per wavefront: 4, or 3 for 192-column tiles (not with gated activations)
+    constexpr int BN = NS * 64;   // columns of the output tile
     constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
     constexpr int SEGS = TK / SEG;
     constexpr int SEG_SLABS = SEG / 32;
@@ -101,7 +102,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int const KT = SPLITK ? (kt_begin + p.tiles_per_split < p.k_tiles ? kt_begin + p.tiles_per_split : p.k_tiles)
                           : p.k_tiles;
     int m0 = tm * kGemmBM;
-    int strip0 = tn * (kGemmBN / 16) + wave * NS;
+    int strip0 = tn * (BN / 16) + wave * NS;
     uint32_t tile_oob = 0; // PERSIST: kOob once there is no further tile (every request reads zeros)
 
     constexpr uint32_t kOob = 0x80000000u;
@@ -333,7 +334,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 // The conversion of this iteration's 16/RT operand registers runs in 4 stages, one
                 // after each of the 4 MFMAs: a wavefront issues in order, so VALU work only runs
                 // under the matrix core when it sits between the matrix instructions.
-                constexpr int CONV = 16 / RT;
+                constexpr int CONV = (NS * 4 + RT - 1) / RT; // NS * 4 operand registers per slab over RT iterations
                 // bf16: q/16 as float (v_cvt_off_f32_i4 / sign-extending byte converts, with byte
                 // selects on the source), float32 FMA with 16*s, packed round to bf16.
                 // fp16: the exponent-magic pair (BASE + u), one packed subtract to the exact q and
@@ -346,6 +347,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     for (int x = 0; x < CONV; ++x)
                     {
                         int const ci = rt * CONV + x, s = ci / 4, pr = ci % 4;
+                        if (ci >= NS * 4)
+                            continue;
                         bool const same_step = j + 1 < SLABS;
                         BStage const& src = same_step ? st : st_next;
                         int const jn = same_step ? j + 1 : 0;
@@ -412,6 +415,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     else
                         E::mma_acc(b_cur[s], a_cur, acc[rt][s]);
                     conv_stage(s);
+                    if (NS < 4 && s == NS - 1) // fewer matrix instructions than stages: the last one takes the rest
+                        for (int rest = NS; rest < 4; ++rest)
+                            conv_stage(rest);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -487,7 +493,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                     if (tile_of(vb, tm, tn))
                     {
                         m0 = tm * kGemmBM;
-                        strip0 = tn * (kGemmBN / 16) + wave * NS;
+                        strip0 = tn * (BN / 16) + wave * NS;
 #pragma unroll
                         for (int s = 0; s < NS; ++s)
                         {
@@ -666,9 +672,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         plain_epilogue(std::false_type{});
 }
 
-template <int DT, int BITS, int GROUP, bool ZERO, int RT>
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, int NS = 4>
 int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
 {
+    static_assert(NS == 4 || RT == 16, "192-column tiles exist for the 256-row kernel only");
     int const total = gp.tiles_m * gp.tiles_n;
     dim3 grid(((total + 7) / 8) * 8, gp.k_splits), block(256);
     if (gp.k_splits > 1)
@@ -685,19 +692,19 @@ int launch_gemm_variant(GemmParams const& gp, hipStream_t stream)
         int const cus = gemm_persistent_workgroups();
         bool persist = false;
         if constexpr (RT == 16)
-            persist = cus > 0 && total > cus && gp.k_tiles % 2 == 0 && gp.k_tiles >= 4 && gp.n % kGemmBN == 0
+            persist = cus > 0 && total > cus && gp.k_tiles % 2 == 0 && gp.k_tiles >= 4 && gp.n % (NS * 64) == 0
                 && !gp.bias && !gp.expert_rows && gp.num_experts == 0 && gp.activation == kActIdentity && !gp.residual
                 && (uint64_t) gp.m * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 31)
                 // byte offsets of the padded last row tile, and of the rejected offset plus 15 row tiles, stay below 2^32
                 && (uint64_t) gp.tiles_m * (RT * 16) * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 32) && gp.n < (1 << 22);
-        note_launch("gemm exact rt=%d splits=1 persistent=%d", RT, (int) persist);
+        note_launch("gemm exact rt=%d splits=1 persistent=%d columns=%d", RT, (int) persist, NS * 64);
         if (persist)
         {
             if constexpr (RT == 16)
-                hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false, true>), dim3(cus), block, 0, stream, gp);
+                hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false, true, NS>), dim3(cus), block, 0, stream, gp);
         }
         else
-            hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false>), grid, block, 0, stream, gp);
+            hipLaunchKernelGGL((gemm_kernel<DT, BITS, GROUP, ZERO, RT, false, false, NS>), grid, block, 0, stream, gp);
     }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
@@ -712,7 +719,10 @@ int launch_gemm_rt(GemmParams const& gp, int rt, hipStream_t s)
     {
     case 4: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 4>(gp, s);
     case 8: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 8>(gp, s);
-    default: return launch_gemm_variant<DT, BITS, GROUP, ZERO, 16>(gp, s);
+    default:
+        if (gp.tile_cols == 192)
+            return launch_gemm_variant<DT, BITS, GROUP, ZERO, 16, 3>(gp, s);
+        return launch_gemm_variant<DT, BITS, GROUP, ZERO, 16>(gp, s);
     }
 }
 
@@ -735,6 +745,19 @@ int launch_gemm_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream
     gp.strips = p.n / kTileN;
     gp.tiles_m = (p.m + plan.rt * 16 - 1) / (plan.rt * 16);
     gp.tiles_n = (p.n + kGemmBN - 1) / kGemmBN;
+    // 192-column tiles where 256-column ones leave the last round over the CUs mostly empty (256-row
+    // tiles, whole K per workgroup): a 192-column tile costs about 0.8 of a 256-column one
+    if (plan.rt == 16 && plan.k_splits == 1 && !act_is_gated(p.activation) && !p.expert_rows && p.n % 192 == 0)
+    {
+        int const cus = gemm_persistent_workgroups() > 0 ? gemm_persistent_workgroups() : 256;
+        int const t256 = gp.tiles_m * gp.tiles_n, t192 = gp.tiles_m * (p.n / 192);
+        int const forced = env_overrides().gemm_cols; // WOQ_GEMM_COLS=192|256
+        if (forced ? forced == 192 : 0.8 * ((t192 + cus - 1) / cus) < 1.0 * ((t256 + cus - 1) / cus) - 1e-9)
+        {
+            gp.tile_cols = 192;
+            gp.tiles_n = p.n / 192;
+        }
+    }
     gp.k_splits = plan.k_splits;
     gp.tiles_per_split = (gp.k_tiles + plan.k_splits - 1) / plan.k_splits;
     gp.tiles_per_split += gp.tiles_per_split & 1; // the main loop walks tile rows in pairs

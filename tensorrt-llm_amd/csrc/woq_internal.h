@@ -30,6 +30,7 @@ inline int bits_of(int quant_type)
 //   WOQ_FORCE_REGIME=stream|gemm      WOQ_STREAM_SHAPE=ns,waves,pf,lds   WOQ_WIDE_SHAPE=ns,waves,pf | 0
 //   WOQ_STREAM_SLOTS=0                WOQ_GEMM_KERNEL=exact|skinny       WOQ_GEMM_RT=4|8|16
 //   WOQ_GEMM_SPLITS=<n>               WOQ_STREAM_SPLITS=<n>              WOQ_GEMM_PERSIST=0
+//   WOQ_GEMM_COLS=192|256
 struct EnvOverrides
 {
     int regime = 0;                // woq_regime; 0 = none
@@ -40,6 +41,7 @@ struct EnvOverrides
     bool slots_off = false;        // no group-slot variants of the streaming kernel
     int gemm_kernel = 0;           // 0 any, 1 exact-dequantize, 2 deferred-scale
     int gemm_rt = 0;               // row tiles per wavefront of the exact-dequantize / fp8 kernel
+    int gemm_cols = 0;             // columns of a 256-row tile of the exact-dequantize kernel (192 needs n % 192 == 0)
     int gemm_splits = 0;           // K split of the GEMM regime
     int stream_splits = 0;         // K slices of the streaming kernel (0 = built-in rule)
     bool persist_off = false;      // WOQ_GEMM_PERSIST=0: no persistent prefill kernels

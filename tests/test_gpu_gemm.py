@@ -233,3 +233,36 @@ def test_gemm_persistent_needs_whole_tiles_and_no_bias(pkg, oracle, dev, gemm_ke
         out = run_product(pkg, oracle, dev, p, GEMM)
         assert "persistent=0" in _last_launch(pkg), _last_launch(pkg)
         assert parity_err(oracle, out, p) < TOL
+
+
+@pytest.mark.parametrize("m,k,n,bits,group,dtype,zero,bias", [
+    (300, 512, 768, 4, 128, "bf16", True, True), (257, 1024, 384, 8, 0, "fp16", False, False),
+    (520, 448, 960, 4, 64, "fp16", True, False), (4000, 512, 192 * 43, 4, 128, "bf16", True, False),
+    (2250, 256, 192 * 120, 8, 128, "bf16", False, False)])
+def test_gemm_192_column_tiles(pkg, oracle, dev, woq_env, gemm_kernel, m, k, n, bits, group, dtype, zero, bias):
+    """256-row tiles of 192 columns (three strips per wavefront): against the oracle, and bit for bit
+    against the 256-column tiles; the last two shapes take the persistent loop."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel has one tile width")
+    p = random_problem(oracle, m, k, n, bits, group, dtype, zero=zero, bias=bias, seed=n)
+    woq_env(WOQ_GEMM_COLS="192", WOQ_GEMM_RT="16", WOQ_GEMM_SPLITS="1")
+    out = run_product(pkg, oracle, dev, p, GEMM)
+    assert "columns=192" in _last_launch(pkg), _last_launch(pkg)
+    if m >= 2000:
+        assert "persistent=1" in _last_launch(pkg), _last_launch(pkg)
+    woq_env(WOQ_GEMM_COLS="256")
+    wide = run_product(pkg, oracle, dev, p, GEMM)
+    assert "columns=256" in _last_launch(pkg), _last_launch(pkg)
+    assert (out.view(np.uint32) == wide.view(np.uint32)).all()
+    assert parity_err(oracle, out, p) < TOL
+
+
+def test_gemm_picks_192_columns_where_256_leave_a_round_mostly_empty(pkg, oracle, dev, gemm_kernel):
+    """Llama-3-8B qkv (N = 6144) at 2048 rows: 192 tiles of 256 columns fill three quarters of the CUs,
+    256 tiles of 192 columns fill them all."""
+    if gemm_kernel == "skinny":
+        pytest.skip("the deferred-scale kernel has one tile width")
+    p = random_problem(oracle, 2048, 256, 6144, 4, 128, "bf16", zero=True, seed=6)
+    out = run_product(pkg, oracle, dev, p, GEMM)
+    assert "columns=192" in _last_launch(pkg), _last_launch(pkg)
+    assert parity_err(oracle, out, p) < TOL
