@@ -131,6 +131,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             return st.z[s];
     };
 
+    NibbleConsts const nib = nibble_consts<WOQ_FP16>();
     // Saturation to +-448 is part of the conversion, but a weight cannot reach it while
     // 8|s| + |z| stays below: one wavefront-wide test per tile row takes the clamp (a quarter of
     // the conversion's instructions) out of the common case.
@@ -147,7 +148,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             for (int j = 0; j < SLABS; ++j)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
-                    b[2 * j + h] = (int) dequant4_fp8<ZERO, CLAMP>(st.w[s][j], h, sc, zr);
+                    b[2 * j + h] = (int) dequant4_fp8<ZERO, CLAMP>(st.w[s][j], h, sc, zr, nib);
             acc[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[s], 0, 0, 0, 0, 0, 0);
         }
     };

@@ -49,10 +49,11 @@ __device__ __forceinline__ uint32_t dequant2_fp8(uint32_t old, uint32_t w, int h
                   : (uint32_t) __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, (int) old, true);
 }
 
-// One dword of the B operand (elements 4h .. 4h+3 of slab dword `w`), same arithmetic.  CLAMP =
+// One dword of the B operand (elements 4h .. 4h+3 of slab dword `w`), same arithmetic
+// (`nib`: nibble_consts<WOQ_FP16>(), the mask 0x000F000F and 1024 as a pair of halves in registers).  CLAMP =
 // false leaves the saturation to +-448 out: for callers that know 8|s| + |z| stays below it.
 template <bool ZERO, bool CLAMP>
-__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, float z)
+__device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, float z, NibbleConsts const& nib)
 {
     float v[4]; // elements 4h, 4h+1, 4h+2, 4h+3: nibble slots 2h, 4+2h, 2h+1, 5+2h
     if constexpr (ZERO)
@@ -66,15 +67,17 @@ __device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, flo
     }
     else
     {
-        // even slots are the low nibbles of bytes, odd slots the high nibbles: bytes h and h+2 of
-        // the two masked words (made opaque so that the byte-to-float conversions read them)
-        uint32_t me = w & 0x0F0F0F0Fu, mo = (w >> 4) & 0x0F0F0F0Fu;
-        asm volatile("" : "+v"(me), "+v"(mo));
-        float const m8s = -8.f * s;
-        v[0] = __builtin_fmaf((float) ((me >> (8 * h)) & 0xFF), s, m8s);
-        v[1] = __builtin_fmaf((float) ((me >> (8 * h + 16)) & 0xFF), s, m8s);
-        v[2] = __builtin_fmaf((float) ((mo >> (8 * h)) & 0xFF), s, m8s);
-        v[3] = __builtin_fmaf((float) ((mo >> (8 * h + 16)) & 0xFF), s, m8s);
+        // slots 2h and 4+2h (elements 4h, 4h+1) are 16 bits apart, and so are slots 2h+1 and 5+2h
+        // (elements 4h+2, 4h+3): a shift and one and-or turn each pair into two halves 0x6400 | u =
+        // 1024 + u, which the FMA reads directly.  q s = fma(1024 + u, s, -1032 s) with u = q + 8:
+        // both constants and the result are exact in float32, so this is fma(q, s, 0) bit for bit.
+        f16x2 const p0 = bit_cast<f16x2>(((w >> (8 * h)) & nib.mask) | nib.magic);
+        f16x2 const p1 = bit_cast<f16x2>(((w >> (8 * h + 4)) & nib.mask) | nib.magic);
+        float const c = -1032.f * s;
+        v[0] = __builtin_fmaf((float) p0[0], s, c);
+        v[1] = __builtin_fmaf((float) p0[1], s, c);
+        v[2] = __builtin_fmaf((float) p1[0], s, c);
+        v[3] = __builtin_fmaf((float) p1[1], s, c);
     }
     if constexpr (CLAMP)
     {
