@@ -278,19 +278,32 @@ __device__ __forceinline__ uint16_t buffer_load_u16(__amdgpu_buffer_rsrc_t rsrc,
 }
 
 // ---- row of the scale / zero tables -----------------------------------------------------------------
-// The GROUP = 64 instantiations also serve every larger multiple of 64 ("flexible" group sizes, what
-// the reference's Hopper kernels accept): scales are then applied per 64 rows of K and only the row
-// of the [ceil(k / group), n] tables follows the real group size.  `magic` = ceil(2^32 / (group / 64))
-// for such a group (an exact division by multiplication for every row index that can occur), 0 for a
-// real group of 64.
+// Group sizes that are multiples of 64 above 128 ("flexible" group sizes, what the reference's Hopper
+// kernels accept) have kernel instantiations of their own, GROUP = kFlexGroup: scales are applied per
+// 64 rows of K as for groups of 64, and only the row of the [ceil(k / group), n] tables follows the
+// real group size: `magic` = ceil(2^32 / (group / 64)), an exact division by multiplication for every
+// row index that can occur.  (Serving them from the GROUP = 64 instantiations through a run-time test
+// cost those 10-30 %: their table addresses no longer folded into immediate offsets.)
+constexpr int kFlexGroup = 1;
+
+// rows of K that share one scale inside a tile of TK rows
+template <int GROUP, int TK>
+constexpr int segment_rows()
+{
+    return GROUP == 0 ? TK : GROUP == kFlexGroup ? 64 : (GROUP > TK ? TK : GROUP);
+}
+
+// rows per group as far as sizes computed on the host go (the segment length for flexible groups)
+constexpr int host_group_rows(int group)
+{
+    return group == kFlexGroup ? 64 : group;
+}
+
 template <int GROUP>
 __device__ __forceinline__ uint32_t scale_row(uint32_t k_row, uint32_t magic)
 {
-    if constexpr (GROUP == 64)
-    {
-        uint32_t const seg = k_row >> 6;
-        return magic ? __umulhi(seg, magic) : seg;
-    }
+    if constexpr (GROUP == kFlexGroup)
+        return __umulhi(k_row >> 6, magic);
     else
         return k_row / (uint32_t) (GROUP != 0 ? GROUP : 1);
 }
@@ -304,10 +317,10 @@ inline uint32_t scale_row_magic(int group_size)
     return (uint32_t) ((((uint64_t) 1 << 32) + d - 1) / d);
 }
 
-// the kernel instantiation that serves a group size: 0 / 64 / 128 themselves, 64 for larger multiples of 64
+// the kernel instantiation that serves a group size: 0 / 64 / 128 themselves, kFlexGroup for larger multiples of 64
 inline int template_group(int group_size)
 {
-    return group_size <= 128 ? group_size : 64;
+    return group_size <= 128 ? group_size : kFlexGroup;
 }
 
 // ---- epilogue activations (values of the reference's ActivationType,

@@ -60,7 +60,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     constexpr int kGemmBM = RT * 16;
     constexpr int NS = NS_;       // strips (16 columns) per wavefront: 4, or 3 for 192-column tiles (not with gated activations)
     constexpr int BN = NS * 64;   // columns of the output tile
-    constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
+    constexpr int SEG = segment_rows<GROUP, TK>(); // rows sharing one scale inside a tile row
     constexpr int SEGS = TK / SEG;
     constexpr int SEG_SLABS = SEG / 32;
     constexpr int A_BYTES = kGemmBM * TK * 2;
@@ -776,6 +776,9 @@ int launch_gemm_typed(MatmulProblem const& p, GemmPlan const& plan, void* stream
     case 128:
         return zero ? launch_gemm_rt<DT, BITS, 128, true>(gp, plan.rt, s)
                     : launch_gemm_rt<DT, BITS, 128, false>(gp, plan.rt, s);
+    case kFlexGroup:
+        return zero ? launch_gemm_rt<DT, BITS, kFlexGroup, true>(gp, plan.rt, s)
+                    : launch_gemm_rt<DT, BITS, kFlexGroup, false>(gp, plan.rt, s);
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 }

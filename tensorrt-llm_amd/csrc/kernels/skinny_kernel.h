@@ -36,7 +36,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     constexpr int SLABS = TK / 32;
     constexpr int kSkinnyBM = RT * 16;                           // RT row tiles per wavefront
     constexpr int NS = kSkinnyBN / 16 / kSkinnyWaves;            // strips (16 columns) per wavefront
-    constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows sharing one scale inside a tile row
+    constexpr int SEG = segment_rows<GROUP, TK>(); // rows sharing one scale inside a tile row
     constexpr int SEGS = TK / SEG;
     constexpr int SEG_SLABS = SEG / 32;
     constexpr int A_BYTES = kSkinnyBM * TK * 2;
@@ -609,6 +609,9 @@ int launch_skinny_typed(MatmulProblem const& p, GemmPlan const& plan, void* stre
     case 128:
         return zero ? launch_skinny_variant<DT, BITS, 128, true>(gp, rt, s)
                     : launch_skinny_variant<DT, BITS, 128, false>(gp, rt, s);
+    case kFlexGroup:
+        return zero ? launch_skinny_variant<DT, BITS, kFlexGroup, true>(gp, rt, s)
+                    : launch_skinny_variant<DT, BITS, kFlexGroup, false>(gp, rt, s);
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 }

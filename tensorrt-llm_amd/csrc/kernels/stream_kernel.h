@@ -107,7 +107,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     using E = Elem<DT>;
     constexpr int TK = BITS == 4 ? 128 : 64;
     constexpr int SLABS = TK / 32;
-    constexpr int SEG = (GROUP == 0 || GROUP > TK) ? TK : GROUP; // rows that share one scale inside a tile
+    constexpr int SEG = segment_rows<GROUP, TK>(); // rows that share one scale inside a tile
     constexpr int SEG_SLABS = SEG / 32;
     constexpr int SEGS = TK / SEG;
     constexpr float OFF = Offset<DT, BITS>::value;
@@ -851,7 +851,7 @@ int launch_stream_variant(StreamParams sp, hipStream_t stream)
     size_t lds = 0;
     if constexpr (LDS != 0)
     {
-        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, GROUP, sp.real_group, NS, ZERO, LDS == 1)
+        lds = (LDS == 1 ? stream_act_lds_bytes(sp.m, sp.k, TK) : 0) + stream_scale_lds_bytes(sp.k, TK, host_group_rows(GROUP), sp.real_group, NS, ZERO, LDS == 1)
             + (SLOTS > 1 ? 256 : 0); // group slots: a block of zeros behind the staged operands
         // the reduction buffer of the epilogue is static LDS of this variant and shares the CU's 160 KiB
         constexpr size_t kStaticLds = (size_t) WAVES * NS * MT * 4 * 64 * sizeof(float);
@@ -891,7 +891,7 @@ template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
-    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK, GROUP, sp.split_shape);
+    StreamShape sh = pick_stream_shape(mt, sp.m, sp.k, sp.strips, sp.k_tiles, TK, host_group_rows(GROUP), sp.split_shape);
     if (GROUP == 0 && sh.lds == 2)
         sh.lds = 0; // per-channel scales are applied once, in the epilogue: nothing to stage
 #define WOQ_SHAPE(MT_, NS_, WAVES_, PF_, LDS_)                                                                         \
@@ -957,7 +957,7 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
     // every expert's column groups run side by side: the grid is num_experts times taller
-    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK, GROUP);
+    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK, host_group_rows(GROUP));
     if (act_is_gated(sp.activation) && sh.ns == 1) // value and gate strips pair up inside a wavefront
         sh = sh.lds == 1 ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, sh.lds};
     if (GROUP == 0 && sh.lds == 2)
@@ -1061,6 +1061,9 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
         case 128:
             return zero ? launch_stream_grouped<DT, BITS, 128, true>(sp, s)
                         : launch_stream_grouped<DT, BITS, 128, false>(sp, s);
+        case kFlexGroup:
+            return zero ? launch_stream_grouped<DT, BITS, kFlexGroup, true>(sp, s)
+                        : launch_stream_grouped<DT, BITS, kFlexGroup, false>(sp, s);
         default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
         }
     }
@@ -1079,6 +1082,7 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
         return launch_stream_shaped<DT, BITS, 0, false, false>(sp, mt, s);
     case 64: WOQ_STREAM_PQS(64)
     case 128: WOQ_STREAM_PQS(128)
+    case kFlexGroup: WOQ_STREAM_PQS(kFlexGroup)
     default: return fail(WOQ_ERR_UNSUPPORTED, "group_size %d", p.group_size);
     }
 #undef WOQ_STREAM_PQS
