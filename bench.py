@@ -560,7 +560,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm128", "w4a8_4096", "w4a8_decode", "moe_decode",
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
