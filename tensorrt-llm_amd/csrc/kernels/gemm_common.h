@@ -106,6 +106,11 @@ __device__ __forceinline__ bool select_expert(GemmParams& p, int& tm, int tile_r
 
 constexpr int kGemmBN = 256; // columns of an output tile (4 wavefronts x 64)
 
+// Workgroups of a persistent launch: the CU count of the current device rounded down to a multiple
+// of 8 (one per CU, the same number on every XCD); 0 switches the persistent kernels off
+// (WOQ_GEMM_PERSIST=0).
+int gemm_persistent_workgroups();
+
 // Output tiles are numbered m-fastest inside a column panel; the 8 XCDs each take one contiguous
 // chunk of that order (workgroup i runs on XCD i % 8), so the workgroups that share weight
 // columns or activation rows also share an L2.

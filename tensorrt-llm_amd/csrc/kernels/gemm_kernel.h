@@ -30,11 +30,6 @@ namespace woq
 
 constexpr int kGemmGroupM = 4; // m-tiles walked together so that concurrent workgroups share panels in L2
 
-// Workgroups of a persistent launch: the CU count of the current device rounded down to a multiple
-// of 8 (one per CU, the same number on every XCD); 0 switches the persistent kernels off
-// (WOQ_GEMM_PERSIST=0).
-int gemm_persistent_workgroups();
-
 // amdgpu_waves_per_eu(1, 1): one wavefront per SIMD is the design point (256 accumulator
 // registers per lane); without it the register allocator chases a higher occupancy it cannot
 // reach and parks live values in the accumulator file, shuffling them around every step.

@@ -26,9 +26,17 @@
 namespace woq
 {
 
-template <int ODT, bool ZERO, int RT, bool SPLITK>
+// PERSIST (256-row tiles, whole K, bf16 output, no bias): one workgroup per CU walks tiles b, b + grid, ...
+// as the 16-bit prefill kernel does (gemm_kernel.h): the last two steps of a tile already request the
+// first weights and the first A tile of the next one, and a finished tile's outputs are read out of
+// the accumulators, scaled, packed and stored right before the matrix instruction that starts each
+// block's new sum.  The 8 us or so that a tile spends outside its main loop (first loads, the
+// conversion of the first operand set, 128 KiB of stores, the relaunch) weigh twice as much here as
+// there: a tile's main loop is half as long.
+template <int ODT, bool ZERO, int RT, bool SPLITK, bool PERSIST = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) gemm_w4a8_kernel(GemmParams p)
 {
+    static_assert(!PERSIST || (RT == 16 && !SPLITK && ODT == WOQ_BF16), "persistent form: 256-row tiles, whole K, bf16 out");
     using EO = Elem<ODT>;
     using EH = Elem<WOQ_FP16>;
     constexpr int TK = 128, SLABS = 4, NS = 4;
@@ -40,16 +48,29 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     __shared__ u32x4 a_buf0[A_BYTES / 16];
     __shared__ u32x4 a_buf1[A_BYTES / 16];
 
-    int t;
-    if (!xcd_tile(p.tiles_m * p.tiles_n, t))
+    // Tile of virtual block vb (the block index, or with PERSIST the block index plus a multiple of the
+    // grid size, which is a multiple of 8): XCD-contiguous chunks of the tile order, m fastest inside
+    // groups of 4 m-tiles - the 32 workgroups of an XCD then cover about 4 x 8 tiles and share 4
+    // activation panels and 8 weight panels in its L2 instead of all 16 activation panels and 2
+    int const total = p.tiles_m * p.tiles_n;
+    int const per_xcd = (total + 7) / 8;
+    auto tile_of = [&](int vb, int& tm_, int& tn_) -> bool
+    {
+        int const t = (vb & 7) * per_xcd + (vb >> 3);
+        if ((vb >> 3) >= per_xcd || t >= total)
+            return false;
+        constexpr int kGroupM = 4;
+        int const in_group = kGroupM * p.tiles_n;
+        int const first_m = (t / in_group) * kGroupM;
+        int const gsz = p.tiles_m - first_m < kGroupM ? p.tiles_m - first_m : kGroupM;
+        tm_ = first_m + (t % in_group) % gsz;
+        tn_ = (t % in_group) / gsz;
+        return true;
+    };
+    int vb = (int) blockIdx.x;
+    int tm, tn;
+    if (!tile_of(vb, tm, tn))
         return;
-    // m fastest inside groups of 4 m-tiles: the 32 workgroups of an XCD then cover about 4 x 8 tiles and
-    // share 4 activation panels and 8 weight panels in its L2 instead of all 16 activation panels and 2
-    constexpr int kGroupM = 4;
-    int const in_group = kGroupM * p.tiles_n;
-    int const first_m = (t / in_group) * kGroupM;
-    int const gsz = p.tiles_m - first_m < kGroupM ? p.tiles_m - first_m : kGroupM;
-    int const tm = first_m + (t % in_group) % gsz, tn = (t % in_group) / gsz;
 
     int const lane = threadIdx.x & 63;
     int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -58,8 +79,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     int const kt_begin = SPLITK ? (int) blockIdx.y * p.tiles_per_split : 0;
     int const KT = SPLITK ? (kt_begin + p.tiles_per_split < p.k_tiles ? kt_begin + p.tiles_per_split : p.k_tiles)
                           : p.k_tiles;
-    int const m0 = tm * BM;
-    int const strip0 = tn * (kGemmBN / 16) + wave * NS;
+    int m0 = tm * BM;
+    int strip0 = tn * (kGemmBN / 16) + wave * NS;
 
     constexpr uint32_t kOob = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K);
@@ -68,15 +89,32 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
 
-    int strip_of[NS];
-    uint32_t wlane[NS], sc_lane[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s)
+    // per-lane request addresses of one tile (PERSIST keeps those of the next tile beside them)
+    struct TileCtx
     {
-        strip_of[s] = strip0 + s < p.strips ? strip0 + s : p.strips - 1;
-        wlane[s] = ((uint32_t) strip_of[s] * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
-        sc_lane[s] = (uint32_t) (strip_of[s] * 16 + c) * 2u;
-    }
+        uint32_t wlane[NS], sc_lane[NS];
+        uint32_t dma_lane_base;
+        uint32_t oob; // kOob: there is no such tile, every request reads zeros
+    };
+    auto make_ctx = [&](int tm_, int tn_, bool valid) -> TileCtx
+    {
+        TileCtx x;
+        int const first = tn_ * (kGemmBN / 16) + wave * NS;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+        {
+            int const strip = first + s < p.strips ? first + s : p.strips - 1;
+            x.wlane[s] = ((uint32_t) strip * (uint32_t) p.k_tiles * 64u + (uint32_t) lane) * 16u;
+            x.sc_lane[s] = (uint32_t) (strip * 16 + c) * 2u;
+        }
+        // A tile -> LDS: wavefront w moves pairs w, w+4, ...: piece i is pair f = w + 4i = half w % 2 of
+        // row tile 2i + w / 2
+        x.dma_lane_base = (uint32_t) (tm_ * BM + (wave / 2) * 16 + (lane >> 2)) * (uint32_t) K
+            + (uint32_t) ((wave % 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) * 16));
+        x.oob = valid ? 0u : 0x80000000u;
+        return x;
+    };
+    TileCtx cur = make_ctx(tm, tn, true);
 
     f32x4 acc[RT][NS];
 #pragma unroll
@@ -85,15 +123,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         for (int s = 0; s < NS; ++s)
             acc[rt][s] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- A tile -> LDS: wavefront w moves pairs w, w+4, ...: piece i is pair f = w + 4i = half
-    // w % 2 of row tile 2i + w / 2; K is a multiple of 128, so only kt >= KT falls out of range
-    // (rows past M fall outside the descriptor by themselves).
+    // ---- A tile -> LDS; K is a multiple of 128, so only kt >= KT falls out of range (rows past M fall
+    // outside the descriptor by themselves).
     constexpr int DMA_OPS = PAIRS / 4;
-    uint32_t const dma_lane_base = (uint32_t) (m0 + (wave / 2) * 16 + (lane >> 2)) * (uint32_t) K
-        + (uint32_t) ((wave % 2) * 64 + (((lane & 3) ^ ((lane >> 4) & 3)) * 16));
     uint32_t const dma_piece_stride = 32u * (uint32_t) K;
-    auto dma_base = [&](int kt) -> uint32_t
-    { return (dma_lane_base + (uint32_t) kt * (uint32_t) TK) | ((uint32_t) (KT - 1 - kt) & kOob); };
+    auto dma_base = [&](int kt, TileCtx const& x) -> uint32_t
+    { return (x.dma_lane_base + (uint32_t) kt * (uint32_t) TK) | ((uint32_t) (KT - 1 - kt) & kOob) | x.oob; };
     auto dma_piece = [&](auto* buf, uint32_t base, int i)
     {
         int const f = wave + i * 4;
@@ -115,15 +150,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         uint16_t z[NS];
     };
     constexpr int FETCH_OPS = NS * (ZERO ? 3 : 2);
-    auto fetch_piece = [&](BStage& st, int kt, int i)
+    auto fetch_piece = [&](BStage& st, int kt, int i, TileCtx const& x)
     {
-        uint32_t const past = (uint32_t) (KT - 1 - kt) & kOob; // kt >= KT: every load of the step reads zeros
+        uint32_t const past = ((uint32_t) (KT - 1 - kt) & kOob) | x.oob; // kt >= KT: every load of the step reads zeros
         if (i < NS)
-            st.w[i] = buffer_load_x4(w_rsrc, wlane[i] + ((uint32_t) kt * 1024u | past));
+            st.w[i] = buffer_load_x4(w_rsrc, x.wlane[i] + ((uint32_t) kt * 1024u | past));
         else
         {
             int const s = (i - NS) % NS;
-            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + sc_lane[s]) | past;
+            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + x.sc_lane[s]) | past;
             if (i < 2 * NS)
                 st.s[s] = buffer_load_u16(sc_rsrc, off);
             else
@@ -220,11 +255,35 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     };
     constexpr int UNITS = NS * SLABS * 4; // 64 per step
 
-    auto compute = [&](auto const* buf, u32x8 const (&b_use)[NS], u32x8 (&b_make)[NS], BStage const& st_conv,
-                       BStage& st_req, auto* buf_next, int kt)
+    // PERSIST: where the finished tile's outputs go: byte offset of (row m0 + c, column strip0 * 16 + kg * 4)
+    // of the tile to store (N is a multiple of the tile width: every strip exists; rows past M fall
+    // outside the descriptor); kOob: no finished tile yet
+    [[maybe_unused]] auto const out_rsrc = make_rsrc(p.out, (uint32_t) p.m * (uint32_t) p.n * 2u);
+    [[maybe_unused]] uint32_t prev_off = kOob;
+    [[maybe_unused]] uint32_t const rt_stride = 16u * (uint32_t) p.n * 2u;
+    auto store_block = [&](int rt, int s)
     {
+        // explicit AGPR-source moves: a plain VALU use of the block would pull every accumulator into the
+        // VGPR half of the file for the whole loop.  The pack to bf16 does not depend on the conversion
+        // mode the main loop runs in (that concerns fp16 and fp8 results only).
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[rt][s][r]));
+        u32x2 const o = {EO::pack(p.alpha * v[0], p.alpha * v[1]), EO::pack(p.alpha * v[2], p.alpha * v[3])};
+        __builtin_amdgcn_raw_buffer_store_b64(o, out_rsrc, (int) (prev_off + (uint32_t) rt * rt_stride + (uint32_t) s * 32u), 0, 0);
+    };
+
+    // One step.  The A tile of step kt_a of tile xa goes to buf_next, the packed weights of step kt_w of
+    // tile xw to st_req (the steps after this one and after the next: the same tile's, or with PERSIST
+    // the next tile's first ones).  first_tag: the first step of a tile in the persistent loop.
+    auto compute = [&](auto first_tag, auto const* buf, u32x8 const (&b_use)[NS], u32x8 (&b_make)[NS],
+                       BStage const& st_conv, BStage& st_req, auto* buf_next, int kt_a, TileCtx const& xa, int kt_w,
+                       TileCtx const& xw)
+    {
+        constexpr bool FIRST = decltype(first_tag)::value;
         char const* a_base = reinterpret_cast<char const*>(buf);
-        uint32_t const next_base = dma_base(kt + 1);
+        uint32_t const next_base = dma_base(kt_a, xa);
         auto a_read = [&](int rt) -> u32x8
         {
             // operand position pos holds slab slab_at(pos) = 0, 2, 1, 3: the two pieces that sit
@@ -271,7 +330,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int q = 0; q < FETCH_OPS; ++q)
                 if (FETCH_FIRST + q * FETCH_WINDOW / FETCH_OPS == rt)
-                    fetch_piece(st_req, kt + 2, q);
+                    fetch_piece(st_req, kt_w, q, xw);
             if (rt + A_AHEAD < RT)
                 a_ring[(rt + A_AHEAD) % (A_AHEAD + 1)] = a_read(rt + A_AHEAD);
             u32x8 const a_cur = a_ring[rt % (A_AHEAD + 1)];
@@ -286,6 +345,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 // bytes per row and instruction)
                 if constexpr (SPLITK)
                     mma_fp8_acc(a_cur, b_use[s], acc[rt][s]);
+                else if constexpr (FIRST)
+                {
+                    store_block(rt, s); // the previous tile's sums leave right before the block starts the new tile's
+                    mma_fp8_first(b_use[s], a_cur, acc[rt][s]);
+                }
                 else
                     mma_fp8_acc(b_use[s], a_cur, acc[rt][s]);
                 // behind matrix instruction t: the pack of the units whose FMAs went behind t - 1, the
@@ -318,28 +382,79 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     for (int s = 0; s < NS; ++s)
         b0[s] = b1[s] = u32x8{0, 0, 0, 0, 0, 0, 0, 0};
     {
-        uint32_t const base = dma_base(kt_begin);
+        uint32_t const base = dma_base(kt_begin, cur);
 #pragma unroll
         for (int i = 0; i < DMA_OPS; ++i)
             dma_piece(a_buf0, base, i);
     }
 #pragma unroll
     for (int i = 0; i < FETCH_OPS; ++i)
-        fetch_piece(st0, kt_begin, i);
+        fetch_piece(st0, kt_begin, i, cur);
 #pragma unroll
     for (int i = 0; i < FETCH_OPS; ++i)
-        fetch_piece(st1, kt_begin + 1, i);
+        fetch_piece(st1, kt_begin + 1, i, cur);
 #pragma unroll
     for (int cu = 0; cu < UNITS; ++cu)
         convert_unit(b0, st0, cu);
-    for (int kt = kt_begin; kt < KT; kt += 2)
+    // A(kt) has landed for every wavefront (at most the FETCH_OPS weight-side loads issued after its
+    // DMAs are still outstanding: loads return in order, and the persistent loop's stores are older than
+    // the last of them too); everyone is done reading the other buffer
+    auto step_barrier = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FETCH_OPS) : "memory"); };
+    std::false_type const plain{};
+    if constexpr (!PERSIST)
     {
-        // A(kt) has landed for every wavefront (at most the FETCH_OPS weight-side loads issued
-        // after its DMAs are still outstanding); everyone is done reading the other buffer
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FETCH_OPS) : "memory");
-        compute(a_buf0, b0, b1, st1, st0, a_buf1, kt);
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(FETCH_OPS) : "memory");
-        compute(a_buf1, b1, b0, st0, st1, a_buf0, kt + 1); // past the end of K both operands read as zeros
+        for (int kt = kt_begin; kt < KT; kt += 2)
+        {
+            step_barrier();
+            compute(plain, a_buf0, b0, b1, st1, st0, a_buf1, kt + 1, cur, kt + 2, cur);
+            step_barrier();
+            compute(plain, a_buf1, b1, b0, st0, st1, a_buf0, kt + 2, cur, kt + 3, cur); // past the end of K both operands read as zeros
+        }
+    }
+    else
+    {
+        // Straight-line first, second and last two steps around a plain inner loop (KT even, >= 4; the
+        // shape the 16-bit kernel's persistent loop has, for the same reason: all 256 AGPRs are
+        // accumulators, and a branch between first-step and ordinary code inside a loop makes the
+        // allocator keep second copies of them).  Step kt multiplies operand set kt % 2 (buffer kt % 2),
+        // converts the weights of step kt + 1 and requests those of step kt + 2 and the A tile of step
+        // kt + 1 - in a tile's last two steps those are the next tile's first ones.
+        bool has_next;
+        do
+        {
+            int tmn = 0, tnn = 0;
+            has_next = tile_of(vb + (int) gridDim.x, tmn, tnn);
+            TileCtx const nxt = make_ctx(tmn, tnn, has_next);
+            step_barrier();
+            compute(std::true_type{}, a_buf0, b0, b1, st1, st0, a_buf1, 1, cur, 2, cur);
+            step_barrier();
+            compute(plain, a_buf1, b1, b0, st0, st1, a_buf0, 2, cur, 3, cur);
+            for (int kt = 2; kt < KT - 2; kt += 2)
+            {
+                step_barrier();
+                compute(plain, a_buf0, b0, b1, st1, st0, a_buf1, kt + 1, cur, kt + 2, cur);
+                step_barrier();
+                compute(plain, a_buf1, b1, b0, st0, st1, a_buf0, kt + 2, cur, kt + 3, cur);
+            }
+            step_barrier();
+            compute(plain, a_buf0, b0, b1, st1, st0, a_buf1, KT - 1, cur, 0, nxt);
+            step_barrier();
+            compute(plain, a_buf1, b1, b0, st0, st1, a_buf0, 0, nxt, 1, nxt);
+            // this tile's outputs: stored during the next tile's first step (or below)
+            prev_off = ((uint32_t) (m0 + c) * (uint32_t) p.n + (uint32_t) (strip0 * 16 + kg * 4)) * 2u;
+            vb += (int) gridDim.x;
+            m0 = tmn * BM;
+            strip0 = tnn * (kGemmBN / 16) + wave * NS;
+            cur = nxt;
+        } while (has_next);
+        mma_drain();
+        fp8_saturation_off();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                store_block(rt, s);
+        return;
     }
 
     // ---- epilogue: out = T(alpha * acc + bias), or partial sums into the float32 buffer --------
@@ -410,7 +525,24 @@ int launch_w4a8_variant(GemmParams const& gp, hipStream_t stream)
             gp.out, gp.partial, gp.bias, gp.alpha, gp.m, gp.n, gp.k_splits);
     }
     else
-        hipLaunchKernelGGL((gemm_w4a8_kernel<ODT, ZERO, RT, false>), grid, block, 0, stream, gp);
+    {
+        // 256-row tiles, bf16 out: one persistent workgroup per CU when that means at least two tiles each
+        int const cus = gemm_persistent_workgroups();
+        bool persist = false;
+        if constexpr (RT == 16 && ODT == WOQ_BF16)
+            persist = cus > 0 && total > cus && gp.k_tiles % 2 == 0 && gp.k_tiles >= 4 && gp.n % kGemmBN == 0 && !gp.bias
+                && (uint64_t) gp.m * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 31)
+                // byte offsets of the padded last row tile, and of the rejected offset plus 15 row tiles, stay below 2^32
+                && (uint64_t) gp.tiles_m * 256 * (uint64_t) gp.n * 2 < ((uint64_t) 1 << 32) && gp.n < (1 << 22);
+        note_launch("gemm w4a8 rt=%d splits=1 persistent=%d", RT, (int) persist);
+        if (persist)
+        {
+            if constexpr (RT == 16 && ODT == WOQ_BF16)
+                hipLaunchKernelGGL((gemm_w4a8_kernel<ODT, ZERO, RT, false, true>), dim3(cus), block, 0, stream, gp);
+        }
+        else
+            hipLaunchKernelGGL((gemm_w4a8_kernel<ODT, ZERO, RT, false>), grid, block, 0, stream, gp);
+    }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "W4A8 gemm kernel launch failed: %s", hipGetErrorString(err));

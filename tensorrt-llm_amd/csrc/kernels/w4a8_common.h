@@ -125,4 +125,10 @@ __device__ __forceinline__ void mma_fp8_acc(u32x8 a, u32x8 b, f32x4& c)
     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
 
+// c = a x b: the first product of a new sum (the old value of c is dead: no input operand for it)
+__device__ __forceinline__ void mma_fp8_first(u32x8 a, u32x8 b, f32x4& c)
+{
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+}
+
 } // namespace woq

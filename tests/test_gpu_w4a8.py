@@ -97,6 +97,28 @@ def test_w4a8_identity_recovers_e4m3_weight(pkg, oracle, dev):
 STREAM, GEMM = 1, 2
 
 
+def _launch(pkg):
+    return (pkg._lib.lib.woq_last_launch() or b"").decode()
+
+
+@pytest.mark.parametrize("M,K,N,with_zeros", [(2250, 512, 7680, False), (4000, 1024, 8192, True), (2304, 768, 8192, False)])
+def test_w4a8_persistent_tile_loop(pkg, oracle, dev, woq_env, M, K, N, with_zeros):
+    """More 256 x 256 tiles than CUs, bf16 output, no bias: one workgroup per CU walks its tiles (the
+    next tile's first weights and A tile requested in the current tile's last two steps, the outputs
+    stored between the next tile's first matrix instructions).  The bits of the one-tile-per-workgroup
+    launch, which in turn meets the oracle's bar; rows ragged against the tile."""
+    prob = oracle.make_w4a8_problem(M, K, N, seed=M + K, out_dtype="bf16")
+    rng = np.random.default_rng(N)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32)) if with_zeros else None
+    out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=zeros, direct_fp8=True, regime=GEMM)
+    assert "persistent=1" in _launch(pkg), _launch(pkg)
+    woq_env(WOQ_GEMM_PERSIST="0")
+    plain, _ = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=zeros, direct_fp8=True, regime=GEMM)
+    assert "persistent=0" in _launch(pkg), _launch(pkg)
+    assert (out.view(np.uint32) == plain.view(np.uint32)).all()
+    assert _perr(oracle, out, ref, prob) < TOL
+
+
 @pytest.mark.parametrize("out_dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("M", [1, 3, 16])
 @pytest.mark.parametrize("direct", [False, True])
