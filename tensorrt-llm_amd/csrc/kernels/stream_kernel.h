@@ -406,10 +406,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         return idx < sc_chunks ? ((uint32_t) row * (uint32_t) p.n + (uint32_t) (strip * 16 + (piece & 1) * 8)) * 2u
                                : kOob;
     };
-    // chunks past the first THREADS (long K): a plain loop after the weight prefetch is under way
+    // chunks past the first 2 * THREADS (long K): a plain loop after the weight prefetch is under way
     auto stage_scales_tail = [&]()
     {
-        for (int idx = threadIdx.x + THREADS; idx < sc_chunks; idx += THREADS)
+        for (int idx = threadIdx.x + 2 * THREADS; idx < sc_chunks; idx += THREADS)
         {
             uint32_t at;
             uint32_t const off = sc_offset(idx, at);
@@ -425,22 +425,35 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         {
             // the staged scales are requested first, the weight and activation prefetch right
             // behind them: loads complete in order, so the barrier waits for the scales only
-            uint32_t s_at;
-            uint32_t const off = sc_offset(threadIdx.x, s_at);
-            u32x4 const sv = buffer_load_x4(sc_rsrc, off);
-            u32x4 zv;
-            if constexpr (ZERO)
-                zv = buffer_load_x4(zr_rsrc, off);
+            uint32_t s_at[2];
+            u32x4 sv[2], zv[2];
+            [[maybe_unused]] bool const second = sc_chunks > THREADS; // uniform
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                if (u == 1 && !second)
+                    continue;
+                uint32_t const off = sc_offset(threadIdx.x + u * THREADS, s_at[u]);
+                sv[u] = buffer_load_x4(sc_rsrc, off);
+                if constexpr (ZERO)
+                    zv[u] = buffer_load_x4(zr_rsrc, off);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < PF; ++i)
                 fetch(st[i], kt_of(i));
             __builtin_amdgcn_sched_barrier(0);
-            if ((int) threadIdx.x < sc_chunks)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
             {
-                *reinterpret_cast<u32x4*>(sc_lds + s_at) = sv;
-                if constexpr (ZERO)
-                    *reinterpret_cast<u32x4*>(zr_lds + s_at) = zv;
+                if (u == 1 && !second)
+                    continue;
+                if ((int) threadIdx.x + u * THREADS < sc_chunks)
+                {
+                    *reinterpret_cast<u32x4*>(sc_lds + s_at[u]) = sv[u];
+                    if constexpr (ZERO)
+                        *reinterpret_cast<u32x4*>(zr_lds + s_at[u]) = zv[u];
+                }
             }
             stage_scales_tail();
             __syncthreads();
@@ -459,9 +472,11 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         // scales / zeros of this workgroup's columns) are requested FIRST, the weight prefetch
         // right behind them: loads complete in order, so the LDS writes and the barrier wait for
         // the small staged loads only while the weights stay in flight.  Each thread holds up to
-        // UA + 2 staged chunks in registers across the prefetch; anything beyond that (long K,
-        // many rows) is staged by a plain loop after it.
-        constexpr int UA = 2;
+        // UA + 2 staged chunks in registers across the prefetch (the third and fourth only when the
+        // activations are that long: a load issued after the weight prefetch completes after it, so
+        // the barrier would wait a whole HBM round trip for it); anything beyond that (long K, many
+        // rows) is staged by a plain loop after it.
+        constexpr int UA = 4;
         int const chunks_per_row = KT * TK / 8; // 16-byte chunks, including the zero-filled tail of K
         int const act_chunks = act_rows * chunks_per_row;
         auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
@@ -498,11 +513,14 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 *reinterpret_cast<float*>(sum_lds + sum_at) = t;
         };
 
-        u32x4 av[UA], pv[UA], sv, zv;
-        uint32_t a_at[UA], sum_at[UA], s_at = 0;
+        u32x4 av[UA], pv[UA], sv[2], zv[2];
+        uint32_t a_at[UA], sum_at[UA], s_at[2] = {0, 0};
+        [[maybe_unused]] bool const second = sc_chunks > THREADS; // uniform
 #pragma unroll
         for (int u = 0; u < UA; ++u)
         {
+            if (u >= 2 && u * THREADS >= act_chunks) // uniform
+                continue;
             uint32_t ch;
             av[u] = buffer_load_x4(act_rsrc, act_offset(threadIdx.x + u * THREADS, a_at[u], ch, sum_at[u]));
             if constexpr (PQS)
@@ -510,10 +528,16 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         if constexpr (SCLDS)
         {
-            uint32_t const off = sc_offset(threadIdx.x, s_at);
-            sv = buffer_load_x4(sc_rsrc, off);
-            if constexpr (ZERO)
-                zv = buffer_load_x4(zr_rsrc, off);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                if (u == 1 && !second)
+                    continue;
+                uint32_t const off = sc_offset(threadIdx.x + u * THREADS, s_at[u]);
+                sv[u] = buffer_load_x4(sc_rsrc, off);
+                if constexpr (ZERO)
+                    zv[u] = buffer_load_x4(zr_rsrc, off);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -523,6 +547,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
 #pragma unroll
         for (int u = 0; u < UA; ++u)
         {
+            if (u >= 2 && u * THREADS >= act_chunks) // uniform
+                continue;
             u32x4 const v = PQS ? smooth(av[u], pv[u]) : av[u];
             if ((int) threadIdx.x + u * THREADS < act_chunks)
                 *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = v;
@@ -531,22 +557,47 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         if constexpr (SCLDS)
         {
-            if ((int) threadIdx.x < sc_chunks)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
             {
-                *reinterpret_cast<u32x4*>(sc_lds + s_at) = sv;
-                if constexpr (ZERO)
-                    *reinterpret_cast<u32x4*>(zr_lds + s_at) = zv;
+                if (u == 1 && !second)
+                    continue;
+                if ((int) threadIdx.x + u * THREADS < sc_chunks)
+                {
+                    *reinterpret_cast<u32x4*>(sc_lds + s_at[u]) = sv[u];
+                    if constexpr (ZERO)
+                        *reinterpret_cast<u32x4*>(zr_lds + s_at[u]) = zv[u];
+                }
             }
         }
-        for (int idx = threadIdx.x + UA * THREADS; idx < act_chunks; idx += THREADS)
+        // (four requests at a time, so that their round trips overlap)
+        for (int base = UA * THREADS; base < act_chunks; base += UA * THREADS)
         {
-            uint32_t at, ch, sum_at;
-            u32x4 v = buffer_load_x4(act_rsrc, act_offset(idx, at, ch, sum_at));
-            if constexpr (PQS)
-                v = smooth(v, buffer_load_x4(pqs_rsrc, ch * 16u));
-            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + at) = v;
-            if constexpr (SUMLDS)
-                stage_sum(v, idx, sum_at);
+            u32x4 tv[UA], tp[UA];
+            uint32_t t_at[UA], t_sum[UA];
+#pragma unroll
+            for (int u = 0; u < UA; ++u)
+            {
+                if (base + u * THREADS >= act_chunks) // uniform
+                    continue;
+                uint32_t ch;
+                tv[u] = buffer_load_x4(act_rsrc, act_offset(base + u * THREADS + threadIdx.x, t_at[u], ch, t_sum[u]));
+                if constexpr (PQS)
+                    tp[u] = buffer_load_x4(pqs_rsrc, ch * 16u);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < UA; ++u)
+            {
+                if (base + u * THREADS >= act_chunks) // uniform
+                    continue;
+                int const idx = base + u * THREADS + threadIdx.x;
+                u32x4 const v = PQS ? smooth(tv[u], tp[u]) : tv[u];
+                if (idx < act_chunks)
+                    *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + t_at[u]) = v;
+                if constexpr (SUMLDS)
+                    stage_sum(v, idx, t_sum[u]);
+            }
         }
         if constexpr (SCLDS)
             stage_scales_tail();

@@ -181,34 +181,87 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     int const n_my = (KT - wave + WAVES - 1) / WAVES;
     Stage st[PF];
     fp8_saturation_on(); // the conversions below rely on it; off again before the epilogue
-#pragma unroll
-    for (int i = 0; i < PF; ++i)
-        fetch(st[i], wave + i * WAVES);
-    __builtin_amdgcn_sched_barrier(0);
     if constexpr (ALDS || SCLDS)
     {
-        // behind the first weight prefetches: the activations come from L2 and land first
+        // Staged operands (the activations, the group scales / zeros of this workgroup's columns) are
+        // requested FIRST, two 16-byte chunks of each per thread, and the weight prefetch right behind
+        // them: loads complete in order, so the LDS writes and the barrier wait for the small staged
+        // loads (from L2) only, while the weights stay in flight.  Longer operands are finished by
+        // plain loops after the prefetch.
+        constexpr int THREADS = WAVES * 64;
+        constexpr int UA = 2;
         int const rows = p.m < 16 ? p.m : 16;
         int const chunks_per_row = K / 16;
-        for (int idx = threadIdx.x; ALDS && idx < rows * chunks_per_row; idx += WAVES * 64)
+        int const act_chunks = ALDS ? rows * chunks_per_row : 0;
+        int const sc_chunks = SCLDS ? KT * NS * 2 : 0; // NS * 2 chunks of 8 columns per tile row of K
+        auto act_src = [&](int idx, uint32_t& at)
         {
-            int const row = idx / chunks_per_row, ch = idx - row * chunks_per_row;
-            u32x4 const v = buffer_load_x4(act_rsrc, (uint32_t) row * (uint32_t) K + (uint32_t) ch * 16u);
-            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + (uint32_t) row * lds_row + (uint32_t) ch * 16u) = v;
-        }
-        // group scales / zeros: 16-byte chunks of 8 columns, NS * 2 per tile row of K; strips past
-        // the end of N are clamped as for the weights
-        for (int idx = threadIdx.x; SCLDS && idx < KT * NS * 2; idx += WAVES * 64)
+            int const row = rows == 1 ? 0 : idx / chunks_per_row, ch = idx - row * chunks_per_row;
+            at = (uint32_t) row * lds_row + (uint32_t) ch * 16u;
+            return idx < act_chunks ? (uint32_t) row * (uint32_t) K + (uint32_t) ch * 16u : kPast;
+        };
+        // strips past the end of N are clamped as for the weights
+        auto sc_src = [&](int idx, uint32_t& at)
         {
             int const kt = idx / (NS * 2), ch = idx - kt * (NS * 2);
             int const strip = strip0 + (ch >> 1) < p.strips ? strip0 + (ch >> 1) : p.strips - 1;
-            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n + (uint32_t) (strip * 16 + (ch & 1) * 8)) * 2u;
-            *reinterpret_cast<u32x4*>(sc_lds + (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u) = buffer_load_x4(sc_rsrc, off);
+            at = (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u;
+            return idx < sc_chunks ? ((uint32_t) kt * (uint32_t) p.n + (uint32_t) (strip * 16 + (ch & 1) * 8)) * 2u : kPast;
+        };
+        u32x4 av[UA], sv[UA], zv[UA];
+        uint32_t a_at[UA], s_at[UA];
+#pragma unroll
+        for (int u = 0; u < UA; ++u)
+        {
+            if (u * THREADS < act_chunks) // uniform
+                av[u] = buffer_load_x4(act_rsrc, act_src(threadIdx.x + u * THREADS, a_at[u]));
+            if (u * THREADS < sc_chunks) // uniform
+            {
+                uint32_t const off = sc_src(threadIdx.x + u * THREADS, s_at[u]);
+                sv[u] = buffer_load_x4(sc_rsrc, off);
+                if constexpr (ZERO)
+                    zv[u] = buffer_load_x4(zr_rsrc, off);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+            fetch(st[i], wave + i * WAVES);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < UA; ++u)
+        {
+            if (u * THREADS < act_chunks && (int) threadIdx.x + u * THREADS < act_chunks)
+                *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + a_at[u]) = av[u];
+            if (u * THREADS < sc_chunks && (int) threadIdx.x + u * THREADS < sc_chunks)
+            {
+                *reinterpret_cast<u32x4*>(sc_lds + s_at[u]) = sv[u];
+                if constexpr (ZERO)
+                    *reinterpret_cast<u32x4*>(zr_lds + s_at[u]) = zv[u];
+            }
+        }
+        for (int idx = threadIdx.x + UA * THREADS; idx < act_chunks; idx += THREADS)
+        {
+            uint32_t at;
+            uint32_t const off = act_src(idx, at);
+            *reinterpret_cast<u32x4*>(reinterpret_cast<char*>(act_lds) + at) = buffer_load_x4(act_rsrc, off);
+        }
+        for (int idx = threadIdx.x + UA * THREADS; idx < sc_chunks; idx += THREADS)
+        {
+            uint32_t at;
+            uint32_t const off = sc_src(idx, at);
+            *reinterpret_cast<u32x4*>(sc_lds + at) = buffer_load_x4(sc_rsrc, off);
             if constexpr (ZERO)
-                *reinterpret_cast<u32x4*>(zr_lds + (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u)
-                    = buffer_load_x4(zr_rsrc, off);
+                *reinterpret_cast<u32x4*>(zr_lds + at) = buffer_load_x4(zr_rsrc, off);
         }
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+            fetch(st[i], wave + i * WAVES);
         __builtin_amdgcn_sched_barrier(0);
     }
     for (int it = 0; it < n_my; it += PF)
