@@ -115,6 +115,13 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     constexpr bool SCLDS = LDS != 0 && GROUP != 0; // group scales / zeros live in LDS
     constexpr bool SUMLDS = ALDS && GROUP != 0;    // and so do the activation row sums
     constexpr int THREADS = WAVES * 64;
+    // Pipeline stages (1 KiB of weights per strip each) a wavefront requests BEFORE the staging barrier:
+    // a CU keeps only some tens of KiB of loads in flight, and a wavefront whose requests do not fit
+    // waits at the issue - in front of its LDS writes, so the whole workgroup's barrier waits with it.
+    // At most two stages and at most 32 KiB per workgroup go first (measured: 16 / 32 / 64 KiB and
+    // one / two / all stages); the rest of the prefetch is requested right after the barrier.
+    constexpr int P0_FIT = 32 / (NS * WAVES) < 1 ? 1 : 32 / (NS * WAVES);
+    constexpr int P0 = P0_FIT < (PF < 2 ? PF : 2) ? P0_FIT : (PF < 2 ? PF : 2);
     extern __shared__ u32x4 act_lds[]; // ALDS: rows x (KT*TK*2 + 16) bytes, then scales, then zeros
 
     int const group = xcd_strip(blockIdx.x, p.groups_per_xcd);
@@ -440,7 +447,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < PF; ++i)
+            for (int i = 0; i < P0; ++i)
                 fetch(st[i], kt_of(i));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -457,6 +464,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
             }
             stage_scales_tail();
             __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = P0; i < PF; ++i)
+                fetch(st[i], kt_of(i));
         }
         else
         {
@@ -541,7 +552,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < PF; ++i)
+        for (int i = 0; i < P0; ++i)
             fetch(st[i], kt_of(i));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -607,6 +618,10 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
                 *reinterpret_cast<u32x4*>(zero_lds + threadIdx.x * 16u) = u32x4{0u, 0u, 0u, 0u};
         }
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = P0; i < PF; ++i)
+            fetch(st[i], kt_of(i));
         __builtin_amdgcn_sched_barrier(0);
     }
 

@@ -224,8 +224,13 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             }
         }
         __builtin_amdgcn_sched_barrier(0);
+        // at most two pipeline stages and 32 KiB of weights per workgroup before the barrier (a CU keeps
+        // only some tens of KiB of loads in flight; a wavefront whose requests do not fit waits at the
+        // issue, in front of its LDS writes); the rest of the prefetch follows the barrier
+        constexpr int P0_FIT = 32 / (NS * WAVES) < 1 ? 1 : 32 / (NS * WAVES);
+        constexpr int P0 = P0_FIT < (PF < 2 ? PF : 2) ? P0_FIT : (PF < 2 ? PF : 2);
 #pragma unroll
-        for (int i = 0; i < PF; ++i)
+        for (int i = 0; i < P0; ++i)
             fetch(st[i], wave + i * WAVES);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -255,6 +260,10 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
                 *reinterpret_cast<u32x4*>(zr_lds + at) = buffer_load_x4(zr_rsrc, off);
         }
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = P0; i < PF; ++i)
+            fetch(st[i], wave + i * WAVES);
         __builtin_amdgcn_sched_barrier(0);
     }
     else
