@@ -93,7 +93,8 @@ struct StreamShape
     int ns, waves, pf, lds;
 };
 
-StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group, int const* split_shape)
+StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group, int const* split_shape,
+    bool three_strips)
 {
     if (split_shape && split_shape[0] != 0) // the K split's own launch shape
         return {split_shape[0], split_shape[1], split_shape[2], split_shape[3]};
@@ -117,11 +118,14 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         // staging pass and the resident workgroups it costs outweigh the shared reads), and with
         // few column groups and at most 3 rows, where one workgroup per CU covers the whole problem
         // anyway (the down projections: long K, N <= 4096)
-        // strips per workgroup: one up to 256 column strips, two up to 512, else four, so that no launch
-        // has between 256 and 512 workgroups (a partly filled second round over the 256 CUs measured
-        // 10-70 % slower than half as many workgroups of twice the width)
-        StreamShape sh = strips > 512 ? StreamShape{4, 8, 2, 1}
-                                      : (strips > 256 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1});
+        // strips per workgroup: one up to 256 column strips, two up to 512, three up to 768, else four, so
+        // that no launch has between 256 and 512 workgroups (a partly filled second round over the 256
+        // CUs measured 10-70 % slower than half as many workgroups of twice the width); three strips
+        // keep 214-256 CUs busy where four would leave 129-192 (3-6 % on N = 9216 ... 12288)
+        StreamShape sh = strips > 768 || (strips > 512 && !three_strips)
+            ? StreamShape{4, 8, 2, 1}
+            : (strips > 512 ? StreamShape{3, 8, 2, 1}
+                            : (strips > 256 ? StreamShape{2, 8, 4, 1} : StreamShape{1, 8, 4, 1}));
         // LDS of one workgroup of the staged variants: activations, group scales + zeros and row sums
         // (at most k * ns + k bytes, group 64 with zeros), the epilogue's reduction buffer
         size_t const scale_unit = group == 0 ? 0 : (size_t) k * 64 / group;
@@ -144,8 +148,8 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         // eight wavefronts of the staged variant keep more loads in flight than the four of the
         // register variant, for up to four rows
         else if (strips > 512 && strips <= 1024 && rows <= 4
-            && act_lds + (size_t) k * 5 <= stream_max_staged_lds(4, 8))
-            return {4, 8, 2, 1};
+            && act_lds + (size_t) k * (sh.ns + 1) <= stream_max_staged_lds(sh.ns, 8))
+            return sh;
         // activations stay in registers; the group scales / zeros (at most k * ns bytes) are still
         // staged while that leaves room for the resident workgroups the shape counts on
         StreamShape reg = strips > 512 ? StreamShape{4, 4, 2, 0}

@@ -896,7 +896,7 @@ inline size_t stream_scale_lds_bytes(int k, int tile_k, int group, int real_grou
 
 // WOQ_STREAM_SHAPE="ns,waves,pf,lds" overrides the heuristic (for tuning sweeps)
 StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int tile_k, int group,
-    int const* split_shape = nullptr);
+    int const* split_shape = nullptr, bool three_strips = true);
 // WOQ_STREAM_SLOTS=0 switches the group-slot variants off (for A/B timing)
 bool stream_slots_disabled();
 // K slices (1 = none) of a streaming launch with `workspace_bytes` of scratch; WOQ_STREAM_SPLITS overrides
@@ -973,6 +973,7 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
         bool const slots_ok = !stream_slots_disabled();
         WOQ_SLOT_SHAPE(1, 8, 4)
         WOQ_SLOT_SHAPE(2, 8, 4)
+        WOQ_SLOT_SHAPE(3, 8, 2)
         WOQ_SLOT_SHAPE(4, 8, 2)
 #undef WOQ_SLOT_SHAPE
     }
@@ -982,6 +983,7 @@ int launch_stream_shaped(StreamParams const& sp, int mt, hipStream_t s)
     WOQ_SHAPE(1, 1, 16, 4, 1)
     WOQ_SHAPE(1, 2, 8, 4, 1)
     WOQ_SHAPE(1, 2, 4, 4, 1)
+    WOQ_SHAPE(1, 3, 8, 2, 1)
     WOQ_SHAPE(1, 4, 4, 2, 1)
     WOQ_SHAPE(1, 4, 4, 4, 1)
     WOQ_SHAPE(1, 4, 8, 2, 1)
@@ -1023,7 +1025,8 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 {
     constexpr int TK = BITS == 4 ? 128 : 64;
     // every expert's column groups run side by side: the grid is num_experts times taller
-    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK, host_group_rows(GROUP));
+    StreamShape sh = pick_stream_shape(1, sp.m < 16 ? sp.m : 16, sp.k, sp.strips * sp.num_experts, sp.k_tiles, TK, host_group_rows(GROUP), nullptr,
+        /*three_strips=*/false); // the grouped kernel comes with one, two or four strips per wavefront
     if (act_is_gated(sp.activation) && sh.ns == 1) // value and gate strips pair up inside a wavefront
         sh = sh.lds == 1 ? StreamShape{2, 8, 4, 1} : StreamShape{2, 8, 2, sh.lds};
     if (GROUP == 0 && sh.lds == 2)

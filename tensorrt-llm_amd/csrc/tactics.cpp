@@ -88,7 +88,7 @@ std::vector<Tactic> candidates(woq_matmul_args const& a, bool stream_allowed)
         };
         if (mt == 1)
         {
-            add(1, 8, 4, 1), add(2, 8, 4, 1), add(4, 8, 2, 1); // a shape whose operands do not fit the LDS is skipped
+            add(1, 8, 4, 1), add(2, 8, 4, 1), add(3, 8, 2, 1), add(4, 8, 2, 1); // a shape whose operands do not fit the LDS is skipped
             add(1, 8, 4, l), add(2, 8, 2, l), add(4, 4, 2, l);
         }
         else if (mt == 2)
