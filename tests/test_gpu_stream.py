@@ -246,6 +246,44 @@ def test_wide_decode_kernel_is_what_wide_single_row_problems_run_on(pkg, oracle,
     assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()
 
 
+def _last_launch(pkg):
+    return (pkg._lib.lib.woq_last_launch() or b"").decode()
+
+
+@pytest.mark.parametrize("M,bits,group,dtype,K,N", [(1, 4, 128, "bf16", 512, 9216), (1, 4, 64, "fp16", 384, 12288 - 16),
+                                                    (2, 4, 128, "bf16", 256, 8208), (4, 8, 64, "bf16", 256, 10240),
+                                                    (1, 8, 0, "fp16", 320, 12288), (3, 4, 0, "bf16", 512, 9232)])
+def test_stream_three_strips_per_workgroup(pkg, oracle, dev, M, bits, group, dtype, K, N):
+    """513 ... 768 column strips and few rows: the built-in rule gives a workgroup three strips (a last
+    workgroup with one or two, N that is not a multiple of 48); every optional input; one-hot rows return
+    the dequantized weight."""
+    for zero, bias, pqs in [(group != 0, True, True), (False, False, False)]:
+        p = random_problem(oracle, M, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + M)
+        out = run_product(pkg, oracle, dev, p, 0)
+        assert "ns=3" in _last_launch(pkg), _last_launch(pkg)
+        assert parity_err(oracle, out, p) < TOL, (zero, bias, pqs)
+    p = random_problem(oracle, M, K, N, bits, group, dtype, zero=group != 0, seed=N)
+    p["act"] = np.zeros((M, K), np.float32)
+    for r in range(M):
+        p["act"][r, (37 * r + 5) % K] = 1.0
+    out = run_product(pkg, oracle, dev, p, 0)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], group, dtype)
+    for r in range(M):
+        row = w[(37 * r + 5) % K]
+        assert (np.abs(out[r] - row) <= np.abs(row) * 2.0 ** -7 + 2.5e-7).all(), r
+
+
+@pytest.mark.parametrize("M,K,group", [(1, 14336, 128), (3, 14336, 64), (1, 20480, 128), (2, 16384 + 64, 64)])
+def test_stream_staged_chunks_beyond_the_first_batch(pkg, oracle, dev, M, K, group):
+    """Activations of more than two (and more than four) 16-byte chunks per thread and group tables of more
+    than one: the chunks a thread keeps across the weight prefetch, the batched loop behind it, a ragged
+    last batch."""
+    p = random_problem(oracle, M, K, 272, 4, group, "bf16", zero=True, bias=True, pqs=True, seed=K + M)
+    out = run_product(pkg, oracle, dev, p, 0)
+    assert "stream" in _last_launch(pkg), _last_launch(pkg)
+    assert parity_err(oracle, out, p) < TOL
+
+
 @pytest.mark.parametrize("splits", [2, 3, 7])
 @pytest.mark.parametrize("M,bits,group,dtype,K,N", [(16, 4, 128, "bf16", 2176, 272), (5, 4, 64, "fp16", 1408, 144),
                                                     (9, 8, 0, "bf16", 1088, 64), (2, 4, 128, "bf16", 4096, 48),
