@@ -116,8 +116,9 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
         // then scales one output row only) up to ~48 KiB, for more rows up to ~20 KiB (M = 2 at
         // K = 4096; beyond that register-held fragments with staged scales measure faster: the
         // staging pass and the resident workgroups it costs outweigh the shared reads), and with
-        // few column groups and at most 3 rows, where one workgroup per CU covers the whole problem
-        // anyway (the down projections: long K, N <= 4096)
+        // few column groups and at most 3 rows (4 rows while K <= 4096: o_proj 4096x4096 at M = 4
+        // 5.9 -> 5.3 us), where one workgroup per CU covers the whole problem anyway (the down
+        // projections: long K, N <= 4096)
         // strips per workgroup: one up to 256 column strips, two up to 512, three up to 768, else four, so
         // that no launch has between 256 and 512 workgroups (a partly filled second round over the 256
         // CUs measured 10-70 % slower than half as many workgroups of twice the width); three strips
@@ -142,7 +143,8 @@ StreamShape pick_stream_shape(int mt, int m, int k, int strips, int k_tiles, int
             if (act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
                 return {1, 8, 4, 1};
         }
-        else if (strips <= 256 && rows <= 3 && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
+        else if (strips <= 256 && (rows <= 3 || (rows == 4 && act_lds <= (size_t) 33 * 1024))
+            && act_lds + (size_t) k * 2 <= stream_max_staged_lds(1, 8))
             return {1, 8, 4, 1};
         // 513..1024 strips run as at most 256 workgroups of four strips: with one workgroup per CU the
         // eight wavefronts of the staged variant keep more loads in flight than the four of the
