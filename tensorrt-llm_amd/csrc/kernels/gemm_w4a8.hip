@@ -180,7 +180,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     struct ConvState
     {
         uint32_t src[2][2]; // zero-points: sign-flipped source word of (slab parity, pair)
-        uint32_t pw[16];    // no zero-points: the unit's two nibbles as a pair of halves 1024 + u
+        uint32_t pw[16];    // no zero-points: the unit's two nibbles as a pair of halves 1024 + u (1024 + 16 u for pr = 1)
+        uint32_t sh;        // no zero-points: the slab word shifted by 8 (made by the unit h = 1, pr = 0 for both pairs)
         float v[16][2];     // the two values of the units in flight (unit % 16: at most 12 are)
     };
     auto conv_stage = [&](ConvState& cs, u32x8 (&b)[NS], BStage const& st, int cu, int stage)
@@ -218,22 +219,31 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         else
         {
             // q s = fma(1024 + u, s, -1032 s) on the stored nibble u = q + 8: elements e0 = 4h + 2pr and
-            // e0 + 1 sit in nibbles e0/2 and e0/2 + 4, i.e. 16 bits apart - one shift and one and-or
-            // make the pair of halves 0x6400 | u = 1024 + u, which the FMA reads directly.  1024 + u,
-            // 1032 s and the result (15 significant bits) are exact in float32: the same single rounding
-            // to e4m3 as fma(q, s, 0).
+            // e0 + 1 sit in nibbles e0/2 and e0/2 + 4, i.e. 16 bits apart - one and-or makes the pair
+            // of halves 0x6400 | u = 1024 + u, which the FMA reads directly.  The pair pr = 1 is taken
+            // where it sits, four bits up (still inside a half's ten fraction bits): 1024 + 16 u, and
+            // q s = fma(1024 + 16 u, s / 16, -72 s); so only the units of h = 1 need a shift, one for
+            // both.  The constants and the result (15 significant bits) are exact in float32: the same
+            // single rounding to e4m3 as fma(q, s, 0).
             uint32_t& pw = cs.pw[cu % 16];
             if (stage == 0)
             {
-                pw = ((st.w[s][j] >> (4 * (2 * h + pr))) & nib.mask) | nib.magic; // one v_and_or_b32
+                if (h == 1 && pr == 0)
+                {
+                    cs.sh = st.w[s][j] >> 8;
+                    asm volatile("" : "+v"(cs.sh));
+                }
+                uint32_t const src = h == 0 ? st.w[s][j] : cs.sh;
+                pw = (src & (pr == 0 ? nib.mask : nib.mask << 4)) | nib.magic; // one v_and_or_b32
                 asm volatile("" : "+v"(pw));
             }
             else if (stage == 2)
             {
                 float const sc = EH::from_bits(st.s[s]);
                 f16x2 const pair = bit_cast<f16x2>(pw);
-                v[0] = __builtin_fmaf((float) pair[0], sc, -1032.f * sc);
-                v[1] = __builtin_fmaf((float) pair[1], sc, -1032.f * sc);
+                float const mul = pr == 0 ? sc : 0.0625f * sc, add = pr == 0 ? -1032.f * sc : -72.f * sc;
+                v[0] = __builtin_fmaf((float) pair[0], mul, add);
+                v[1] = __builtin_fmaf((float) pair[1], mul, add);
                 asm volatile("" : "+v"(v[0]), "+v"(v[1]));
             }
         }

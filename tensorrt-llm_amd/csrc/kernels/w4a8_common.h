@@ -68,16 +68,20 @@ __device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, flo
     else
     {
         // slots 2h and 4+2h (elements 4h, 4h+1) are 16 bits apart, and so are slots 2h+1 and 5+2h
-        // (elements 4h+2, 4h+3): a shift and one and-or turn each pair into two halves 0x6400 | u =
-        // 1024 + u, which the FMA reads directly.  q s = fma(1024 + u, s, -1032 s) with u = q + 8:
-        // both constants and the result are exact in float32, so this is fma(q, s, 0) bit for bit.
-        f16x2 const p0 = bit_cast<f16x2>(((w >> (8 * h)) & nib.mask) | nib.magic);
-        f16x2 const p1 = bit_cast<f16x2>(((w >> (8 * h + 4)) & nib.mask) | nib.magic);
-        float const c = -1032.f * s;
+        // (elements 4h+2, 4h+3).  One and-or turns the first pair into two halves 0x6400 | u = 1024 + u,
+        // which the FMA reads directly: q s = fma(1024 + u, s, -1032 s) with u = q + 8.  The second
+        // pair is taken where it sits, four bits up, still inside the half's ten fraction bits:
+        // 0x6400 | 16 u = 1024 + 16 u, and q s = fma(1024 + 16 u, s / 16, -72 s) - no shift.  The
+        // constants (s / 16, 1032 s, 72 s) and the result are exact in float32, so either form is
+        // fma(q, s, 0) bit for bit.
+        uint32_t const wh = w >> (8 * h);
+        f16x2 const p0 = bit_cast<f16x2>((wh & nib.mask) | nib.magic);
+        f16x2 const p1 = bit_cast<f16x2>((wh & (nib.mask << 4)) | nib.magic);
+        float const c = -1032.f * s, s16 = 0.0625f * s, c16 = -72.f * s;
         v[0] = __builtin_fmaf((float) p0[0], s, c);
         v[1] = __builtin_fmaf((float) p0[1], s, c);
-        v[2] = __builtin_fmaf((float) p1[0], s, c);
-        v[3] = __builtin_fmaf((float) p1[1], s, c);
+        v[2] = __builtin_fmaf((float) p1[0], s16, c16);
+        v[3] = __builtin_fmaf((float) p1[1], s16, c16);
     }
     if constexpr (CLAMP)
     {
