@@ -255,16 +255,29 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         }
     };
 
-    auto compute = [&](int buf, int buf_next, Stage const& st)
+    // With group scales the A tile of the NEXT step has landed when a step starts (its row sums are formed
+    // during the step), so the step can also read the next step's A fragments into registers between its
+    // matrix instructions: the burst of eight-wavefronts-times-eight LDS reads at the top of every step,
+    // and the wait for it, go away.  Two fragment sets alternate (the loop is unrolled by an even number of
+    // steps); with four row tiles the second set does not fit the register file.
+    constexpr bool A_AHEAD = GROUP != 0 && RT <= 2 && (DEPTH + 1) % 2 == 0;
+    auto read_frags = [&](int buf, u32x4 (&a)[RT][SLABS])
     {
         char const* a_base = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off;
-        [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_sc[buf]->sc[wave]) + c * 2;
-        u32x4 a[RT][SLABS];
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
                 a[rt][j] = *reinterpret_cast<u32x4 const*>(a_base + (rt * SLABS + j) * 1024);
+    };
+    auto compute = [&](int buf, int buf_next, Stage const& st, u32x4 (&a_have)[RT][SLABS], u32x4 (&a_make)[RT][SLABS])
+    {
+        [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_sc[buf]->sc[wave]) + c * 2;
+        [[maybe_unused]] char const* a_next_base = reinterpret_cast<char const*>(stage_a[buf_next]->a) + a_lane_off;
+        u32x4 a_local[RT][SLABS];
+        if constexpr (!A_AHEAD)
+            read_frags(buf, a_local);
+        u32x4(&a)[RT][SLABS] = A_AHEAD ? a_have : a_local;
         uint16_t raw_s[NS][SEGS], raw_z[NS][SEGS];
         if constexpr (GROUP != 0)
         {
@@ -350,6 +363,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                         else if (s + 1 < NS)
                             b_nxt[x] = expand_reg(st.w[s + 1], 0, x);
                     }
+                    if constexpr (A_AHEAD)
+                    {
+                        if (s == 0) // one fragment of the next step per mini-block of the first strip
+                            a_make[rt][j] = *reinterpret_cast<u32x4 const*>(a_next_base + (rt * SLABS + j) * 1024);
+                    }
                     if constexpr (GROUP != 0)
                     {
                         if (s == 0 && j == SLABS - 1 && rt == RT - 1)
@@ -403,6 +421,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DEPTH - 1) * (FETCH_OPS + DMA_OPS) + FETCH_OPS) : "memory");
         form_sums(0);
     }
+    u32x4 a_set0[RT][SLABS], a_set1[RT][SLABS];
+    if constexpr (A_AHEAD)
+    {
+        read_frags(0, a_set0);
+    }
     for (int kt = kt_begin; kt < KT; kt += DEPTH + 1)
     {
 #pragma unroll
@@ -415,7 +438,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             fetch_b(st[(u + DEPTH) % (DEPTH + 1)], (u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
             __builtin_amdgcn_sched_barrier(0);
             if (kt + u < KT) // uniform; the requests above go on (they read zeros past the end of K)
-                compute(u, (u + 1) % (DEPTH + 1), st[u]);
+                compute(u, (u + 1) % (DEPTH + 1), st[u], u % 2 == 0 ? a_set0 : a_set1, u % 2 == 0 ? a_set1 : a_set0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
