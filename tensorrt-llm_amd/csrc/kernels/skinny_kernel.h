@@ -259,8 +259,11 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // during the step), so the step can also read the next step's A fragments into registers between its
     // matrix instructions: the burst of eight-wavefronts-times-eight LDS reads at the top of every step,
     // and the wait for it, go away.  Two fragment sets alternate (the loop is unrolled by an even number of
-    // steps); with four row tiles the second set does not fit the register file.
-    constexpr bool A_AHEAD = GROUP != 0 && RT <= 2 && (DEPTH + 1) % 2 == 0;
+    // steps); with four row tiles only half of a second set fits the register file.
+    constexpr bool A_AHEAD = GROUP != 0 && (DEPTH + 1) % 2 == 0;
+    // slabs read ahead: all with two row tiles; with four, half of them where the registers allow (group 128),
+    // the rest at the top of the step
+    constexpr int AH = RT <= 2 ? SLABS : (GROUP == 128 ? SLABS / 2 : 0);
     auto read_frags = [&](int buf, u32x4 (&a)[RT][SLABS])
     {
         char const* a_base = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off;
@@ -274,10 +277,16 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     {
         [[maybe_unused]] char const* sc_base = reinterpret_cast<char const*>(stage_sc[buf]->sc[wave]) + c * 2;
         [[maybe_unused]] char const* a_next_base = reinterpret_cast<char const*>(stage_a[buf_next]->a) + a_lane_off;
-        u32x4 a_local[RT][SLABS];
-        if constexpr (!A_AHEAD)
-            read_frags(buf, a_local);
-        u32x4(&a)[RT][SLABS] = A_AHEAD ? a_have : a_local;
+        u32x4 a[RT][SLABS];
+        {
+            char const* a_base = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off;
+#pragma unroll
+            for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    a[rt][j] = (A_AHEAD && j < AH) ? a_have[rt][j]
+                                                   : *reinterpret_cast<u32x4 const*>(a_base + (rt * SLABS + j) * 1024);
+        }
         uint16_t raw_s[NS][SEGS], raw_z[NS][SEGS];
         if constexpr (GROUP != 0)
         {
@@ -365,7 +374,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                     }
                     if constexpr (A_AHEAD)
                     {
-                        if (s == 0) // one fragment of the next step per mini-block of the first strip
+                        if (s == 0 && j < AH) // one fragment of the next step per mini-block of the first strip
                             a_make[rt][j] = *reinterpret_cast<u32x4 const*>(a_next_base + (rt * SLABS + j) * 1024);
                     }
                     if constexpr (GROUP != 0)

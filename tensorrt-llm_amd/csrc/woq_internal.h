@@ -137,7 +137,7 @@ inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k,
     int const k_tiles = (k + tk - 1) / tk;
     double c;
     if (skinny)
-        c = bits == 4 ? (rt == 2 ? 0.79 : 1.29) : 0.565;
+        c = bits == 4 ? (rt == 2 ? 0.73 : 1.29) : 0.565; // (two row tiles: 0.79 before the A fragments were read a step ahead)
     else
         c = bits == 4 ? 0.807 + 0.108 * rt : 0.642 + 0.0404 * rt;
     // the tiles are dealt to the 8 XCDs (32 CUs each) in equal contiguous runs: the fullest XCD
