@@ -28,7 +28,7 @@ namespace woq
 constexpr int kSkinnyBN = 256;
 constexpr int kSkinnyWaves = 8; // two per SIMD: while one waits at the barrier or for LDS the other issues
 
-template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 4)>
+template <int DT, int BITS, int GROUP, bool ZERO, int RT, bool SPLITK, int DEPTH = (BITS == 4 ? 3 : 5)>
 __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) skinny_kernel(GemmParams p)
 {
     using E = Elem<DT>;
@@ -260,10 +260,10 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // matrix instructions: the burst of eight-wavefronts-times-eight LDS reads at the top of every step,
     // and the wait for it, go away.  Two fragment sets alternate (the loop is unrolled by an even number of
     // steps); with four row tiles only half of a second set fits the register file.
-    constexpr bool A_AHEAD = GROUP != 0 && (DEPTH + 1) % 2 == 0;
-    // slabs read ahead: all with two row tiles; with four, half of them where the registers allow (group 128),
-    // the rest at the top of the step
-    constexpr int AH = RT <= 2 ? SLABS : (GROUP == 128 ? SLABS / 2 : 0);
+    constexpr bool A_AHEAD = (DEPTH + 1) % 2 == 0;
+    // slabs read ahead: all with two row tiles; with four, all of them for int8 (two slabs per step), half
+    // of them for int4 where the registers allow (group 128), the rest at the top of the step
+    constexpr int AH = RT <= 2 ? SLABS : (BITS == 8 ? SLABS : (GROUP == 128 ? SLABS / 2 : 0));
     auto read_frags = [&](int buf, u32x4 (&a)[RT][SLABS])
     {
         char const* a_base = reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off;
@@ -413,7 +413,9 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     // With group scales the A tile of step kt+1 must have landed as well (its row sums are formed
     // during step kt): a step's requests are its A DMAs followed by its weight-side requests, so
     // only the weight-side requests of step kt+1 may still be outstanding.
-    constexpr int WAIT = GROUP != 0 ? (DEPTH - 2) * (FETCH_OPS + DMA_OPS) + FETCH_OPS : (DEPTH - 1) * (FETCH_OPS + DMA_OPS);
+    // (the same when A fragments are read a step ahead)
+    constexpr bool NEXT_A_LANDED = GROUP != 0 || (A_AHEAD && AH > 0);
+    constexpr int WAIT = NEXT_A_LANDED ? (DEPTH - 2) * (FETCH_OPS + DMA_OPS) + FETCH_OPS : (DEPTH - 1) * (FETCH_OPS + DMA_OPS);
     static_assert(DEPTH >= 2 && WAIT < 64, "vmcnt is a 6-bit counter");
     Stage st[DEPTH + 1];
 #pragma unroll
@@ -423,15 +425,15 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         fetch_b(st[i], i, kt_begin + i);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if constexpr (GROUP != 0)
+    if constexpr (NEXT_A_LANDED)
     {
-        // row sums of the first step: its A tile has landed once at most the younger steps and its
-        // own weight-side requests are outstanding
+        // row sums (and fragments) of the first step: its A tile has landed once at most the younger steps
+        // and its own weight-side requests are outstanding
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DEPTH - 1) * (FETCH_OPS + DMA_OPS) + FETCH_OPS) : "memory");
         form_sums(0);
     }
     u32x4 a_set0[RT][SLABS], a_set1[RT][SLABS];
-    if constexpr (A_AHEAD)
+    if constexpr (A_AHEAD && AH > 0)
     {
         read_frags(0, a_set0);
     }
