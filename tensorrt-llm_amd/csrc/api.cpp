@@ -36,7 +36,7 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream);
 int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream);
 
 // plan of a plain (not grouped) 16-bit GEMM-regime call: the tactic in force, else the cost model's
-GemmPlan planned_gemm(int m, int n, int k, int bits)
+GemmPlan planned_gemm(int m, int n, int k, int bits, int group)
 {
     Tactic const* t = current_tactic();
     if (t && t->regime == WOQ_REGIME_GEMM && t->rt != 0 && (t->rt != 2 || (t->skinny && bits == 4)))
@@ -49,14 +49,14 @@ GemmPlan planned_gemm(int m, int n, int k, int bits)
         pl.ws_bytes = split_partial_bytes(m, n, pl.k_splits);
         return pl;
     }
-    return plan_gemm(m, n, k, bits);
+    return plan_gemm(m, n, k, bits, true, 1, group);
 }
 
 int launch_gemm(MatmulProblem const& p, void* stream)
 {
     if (p.w4a8)
         return launch_gemm_w4a8(p, stream);
-    return launch_gemm_planned(p, planned_gemm(p.m, p.n, p.k, p.bits), stream);
+    return launch_gemm_planned(p, planned_gemm(p.m, p.n, p.k, p.bits, p.group_size), stream);
 }
 
 int launch_gemm_planned(MatmulProblem const& p, GemmPlan const& plan, void* stream)
@@ -526,17 +526,23 @@ static size_t stream_workspace_bytes(int m, int n, int k, int quant_algo)
 }
 
 // float32 partial buffer of one GEMM-regime call with exactly m rows
-static size_t split_bytes(int m, int n, int k, int quant_algo)
+// (group: the problem's group size, or -1 for a caller that does not know it - the plan may depend on
+// it, so such a caller gets the larger of the candidates)
+static size_t split_bytes(int m, int n, int k, int quant_algo, int group = -1)
 {
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
         return plan_gemm_w4a8(m, n, k).ws_bytes;
-    return planned_gemm(m, n, k, (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4).ws_bytes;
+    int const bits = (quant_algo & WOQ_ALGO_INT8_WEIGHT) ? 8 : 4;
+    if (group >= 0)
+        return planned_gemm(m, n, k, bits, group).ws_bytes;
+    size_t const a = planned_gemm(m, n, k, bits, -1).ws_bytes, b = planned_gemm(m, n, k, bits, 128).ws_bytes;
+    return a > b ? a : b;
 }
 
 // what one GEMM-regime call with exactly m rows uses
-static size_t gemm_workspace_bytes(int m, int n, int k, int quant_algo)
+static size_t gemm_workspace_bytes(int m, int n, int k, int quant_algo, int group = -1)
 {
-    return smooth_bytes(m, k, quant_algo) + split_bytes(m, n, k, quant_algo);
+    return smooth_bytes(m, k, quant_algo) + split_bytes(m, n, k, quant_algo, group);
 }
 
 extern "C" size_t woq_workspace_bytes(int32_t m, int32_t n, int32_t k, int32_t quant_algo, int32_t act_dtype)
@@ -585,7 +591,7 @@ extern "C" int woq_matmul_check(const woq_matmul_args* args)
     {
         // the W4A8 streaming kernel reads e4m3 activations: 16-bit ones go through the smoothing
         // pass (and its workspace region) in either regime
-        size_t const need = regime == WOQ_REGIME_GEMM ? gemm_workspace_bytes(p.m, p.n, p.k, args->quant_algo)
+        size_t const need = regime == WOQ_REGIME_GEMM ? gemm_workspace_bytes(p.m, p.n, p.k, args->quant_algo, p.group_size)
                                                       : smooth_bytes(p.m, p.k, args->quant_algo);
         if (need && (!p.workspace || p.workspace_bytes < need))
             return fail(WOQ_ERR_WORKSPACE, "workspace of %zu bytes required, %zu given", need,
@@ -708,7 +714,7 @@ extern "C" int woq_matmul_static(const woq_matmul_args* args, void* stream)
     int const regime = pick_regime(&a);
     size_t need = 0;
     if (regime == WOQ_REGIME_GEMM)
-        need = gemm_workspace_bytes(p.m, p.n, p.k, a.quant_algo);
+        need = gemm_workspace_bytes(p.m, p.n, p.k, a.quant_algo, p.group_size);
     else if (p.w4a8)
         need = smooth_bytes(p.m, p.k, a.quant_algo);
     else
@@ -804,7 +810,7 @@ extern "C" int woq_grouped_matmul(const woq_grouped_matmul_args* args, void* str
     if (streaming)
         return launch_stream(p, stream);
     // no K split: the tiles of one expert are not what is short here, and the epilogue fusions need the sums
-    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, p.bits, false, single ? 1 : p.num_experts);
+    GemmPlan const plan = plan_gemm(p.m, p.n, p.k, p.bits, false, single ? 1 : p.num_experts, p.group_size);
     bool const two_pass = act != WOQ_ACT_IDENTITY && !gated;
     if (two_pass)
         p.residual = nullptr; // added behind the activation, by the pass below

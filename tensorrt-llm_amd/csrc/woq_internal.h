@@ -131,13 +131,15 @@ inline long gemm_tiles(int m, int n, int rt)
 //     workgroups are no faster than 192, and 257 take two rounds);
 //   * splitting K costs the reduction launch and the float32 partial slabs (written once, read once).
 // `tiles` is the output tile count of that tile height (for a grouped problem: over all experts).
-inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, int splits)
+inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k, int bits, int splits, int group = -1)
 {
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
     double c;
     if (skinny)
-        c = bits == 4 ? (rt == 2 ? 0.73 : 1.29) : 0.565; // (two row tiles: 0.79 before the A fragments were read a step ahead)
+        // (two row tiles: 0.79 before the A fragments were read a step ahead; four row tiles read half a set
+        // ahead at group size 128 only - `group` is -1 where the caller does not know it)
+        c = bits == 4 ? (rt == 2 ? 0.73 : (group == 128 ? 1.19 : 1.29)) : 0.565;
     else
         c = bits == 4 ? 0.807 + 0.108 * rt : 0.642 + 0.0404 * rt;
     // the tiles are dealt to the 8 XCDs (32 CUs each) in equal contiguous runs: the fullest XCD
@@ -155,17 +157,18 @@ inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k,
 
 // The K split (1 = none) that gemm_cost_us estimates cheapest for this kernel and tile height, and
 // its cost.  A split leaves every workgroup at least four tile rows of K.
-inline double gemm_best_split(bool skinny, int rt, long tiles, int m, int n, int k, int bits, bool allow_split, int& splits)
+inline double gemm_best_split(bool skinny, int rt, long tiles, int m, int n, int k, int bits, bool allow_split, int& splits,
+    int group = -1)
 {
     int const tk = tile_k_of_bits(bits);
     int const k_tiles = (k + tk - 1) / tk;
     splits = 1;
-    double best = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, 1);
+    double best = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, 1, group);
     if (!allow_split || k_tiles < 8)
         return best;
     for (int s = 2; s <= k_tiles / 4 && tiles * s <= 512; ++s)
     {
-        double const t = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, s);
+        double const t = gemm_cost_us(skinny, rt, tiles, m, n, k, bits, s, group);
         if (t < best)
         {
             best = t;
@@ -180,7 +183,7 @@ inline double gemm_best_split(bool skinny, int rt, long tiles, int m, int n, int
 //   * the exact-dequantize kernel with 64-, 128- or 256-row tiles.
 // Environment overrides for experiments: WOQ_GEMM_KERNEL=exact|skinny, WOQ_GEMM_RT=4|8|16 (exact
 // kernel), WOQ_GEMM_SPLITS=<n>
-inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true, int num_experts = 1)
+inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true, int num_experts = 1, int group = -1)
 {
     // rows per expert of a grouped problem (its tiles do not straddle experts)
     int const rows = num_experts > 1 ? (m + num_experts - 1) / num_experts : m;
@@ -200,7 +203,7 @@ inline GemmPlan plan_gemm(int m, int n, int k, int bits, bool allow_split = true
             continue;
         int splits;
         double const cost = gemm_best_split(
-            skinny, rt, (long) num_experts * gemm_tiles(rows, n, rt), m, n, k, bits, allow_split, splits);
+            skinny, rt, (long) num_experts * gemm_tiles(rows, n, rt), m, n, k, bits, allow_split, splits, group);
         if (!have || cost < best)
         {
             have = true;
