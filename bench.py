@@ -356,13 +356,14 @@ def run_for_counters(pkg, dev, mode, reps=20):
                           "algorithmic_bytes_per_launch": by, "launches": reps}))
         return
     _, k, n = SHAPES_8B[2]
-    if mode == "w4a8_4096":
-        run = w4a8_setup(pkg, dev, 4096, k, n)
+    if mode.startswith("w4a8_") and mode[5:].isdigit():
+        m = int(mode[5:])
+        run = w4a8_setup(pkg, dev, m, k, n)
         for r in range(reps):
             run()
         torch.cuda.synchronize()
-        print(json.dumps({"mode": mode, "kernel": "W4A8 GEMM on gate_up K=4096 N=28672 M=4096",
-                          "flop_per_launch": 2.0 * 4096 * n * k, "launches": reps}))
+        print(json.dumps({"mode": mode, "kernel": "W4A8 GEMM on gate_up K=4096 N=28672 M=%d" % m,
+                          "flop_per_launch": 2.0 * m * n * k, "launches": reps}))
         return
     if mode.startswith("gemm"):
         m = int(mode[4:] or 4096)
@@ -560,7 +561,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_decode", "moe_decode",
+    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
