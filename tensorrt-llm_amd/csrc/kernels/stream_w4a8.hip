@@ -132,9 +132,9 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     };
 
     NibbleConsts const nib = nibble_consts<WOQ_FP16>();
-    // Saturation to +-448 is part of the conversion, but a weight cannot reach it while
-    // 8|s| + |z| stays below: one wavefront-wide test per tile row takes the clamp (a quarter of
-    // the conversion's instructions) out of the common case.
+    // Saturation to +-448 is part of the conversion: the wavefront runs with the conversion instruction's
+    // own saturating mode switched on (fp8_saturation_on below), as the tiled kernel does, so no clamp and
+    // no test for scales that could reach the limit is needed.
     auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 a, auto clamp_tag)
     {
         constexpr bool CLAMP = decltype(clamp_tag)::value;
@@ -162,18 +162,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             a[2 * j] = (int) v[0];
             a[2 * j + 1] = (int) v[1];
         }
-        bool may_saturate = false;
-#pragma unroll
-        for (int s = 0; s < NS; ++s)
-        {
-            float const bound = __builtin_fmaf(8.f, __builtin_fabsf(EH::from_bits(scale_bits(st, kt, s))),
-                ZERO ? __builtin_fabsf(EH::from_bits(zero_bits(st, kt, s))) : 0.f);
-            may_saturate |= !(bound <= 440.f); // also true for NaN scales
-        }
-        if (__builtin_amdgcn_ballot_w64(may_saturate) != 0)
-            convert_and_multiply(st, kt, a, std::true_type{});
-        else
-            convert_and_multiply(st, kt, a, std::false_type{});
+        convert_and_multiply(st, kt, a, std::false_type{});
     };
 
     // tile rows of this wavefront: kt = wave + it * WAVES.  Every load tolerates kt >= KT, so
