@@ -73,7 +73,7 @@ typedef enum woq_quant_type
 typedef enum woq_regime
 {
     WOQ_REGIME_AUTO = 0,
-    WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 16); with 4 to
+    WOQ_REGIME_STREAM = 1, /* weight-streaming kernels (decode GEMV; accept m <= 128, W4A8 m <= 32); with 4 to
                               16 rows on long-K / narrow-N shapes they split K through the workspace when
                               it is large enough, and run unsplit when it is not */
     WOQ_REGIME_GEMM = 2    /* tiled MFMA GEMMs: deferred-scale 32/64-row tiles or exact-dequantize 64/128/256-row
@@ -219,8 +219,8 @@ int woq_grouped_matmul_check(const woq_grouped_matmul_args* args);
 
 /* The regime the built-in rule picks for AUTO: STREAM for m <= 16; for 17 <= m <= 64 (16-bit
  * activations) STREAM where the streaming kernel's estimated time is below the GEMM plan's (small n
- * with short k, e.g. 4096 x 4096 up to 64 rows, 8192 x 8192 up to ~20), GEMM otherwise; m <= 16 for
- * W4A8 - crossovers measured on MI355X.  Counterpart of the tactic choice
+ * with short k, e.g. 4096 x 4096 up to 64 rows, 8192 x 8192 up to ~20), GEMM otherwise; for W4A8
+ * STREAM up to 32 rows (24 where k >= 2 n) - crossovers measured on MI355X.  Counterpart of the tactic choice
  * (`m < SMALL_M_FAST_PATH`, weightOnlyQuantMatmulPlugin.h:138 and gemmPluginProfiler.cpp:161-178). */
 int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo);
 

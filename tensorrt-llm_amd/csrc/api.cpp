@@ -478,9 +478,18 @@ extern "C" void woq_reload_env(void)
 extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_algo)
 {
     // W4A8: the streaming kernel converts every weight to e4m3 in registers and still runs at
-    // memory speed for one 16-row tile; beyond that the fp8 GEMM kernel
+    // memory speed for one 16-row tile; with two tiles per wavefront (17..32 rows) it still beats the
+    // fp8 GEMM kernel, whose 64-row tiles convert the same weights for a quarter of the rows, by 8-39 %
+    // on the Llama-3-8B / 70B shapes - except on the long-K, narrow-N ones beyond 24 rows (70B down at
+    // M = 32: 59 against 53 us); beyond that the GEMM kernel
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
-        return m <= kStreamW4a8MaxM ? WOQ_REGIME_STREAM : WOQ_REGIME_GEMM;
+    {
+        if (m <= kStreamW4a8AutoMaxM)
+            return WOQ_REGIME_STREAM;
+        if (m <= kStreamW4a8MaxM && !(m > 24 && k >= 2 * n))
+            return WOQ_REGIME_STREAM;
+        return WOQ_REGIME_GEMM;
+    }
     // Measured crossover on MI355X: one 16-row tile streams weights at GEMV speed.  With 17..64 rows
     // the streaming kernel (no split-K passes) still wins on small matrices with short K: whichever
     // the two fitted cost models estimate cheaper.  Beyond that the MFMA GEMM kernels are faster.

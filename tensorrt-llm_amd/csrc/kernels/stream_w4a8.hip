@@ -26,13 +26,16 @@ namespace woq
 // their A pieces from there; a pipeline stage then holds packed weights and scales only.
 // LDSM 2: the group scales and zeros of the workgroup's columns are staged as well.
 // LDSM 3: only those (activations too large for the LDS come from registers).
-template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
+// MT   16-row tiles of activations per wavefront (1; 2 for 17..32 rows, activations from registers: every
+//      converted B operand then feeds two matrix instructions)
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM, int MT = 1>
 __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 {
     using EO = Elem<ODT>;
     using EH = Elem<WOQ_FP16>;
     constexpr int TK = 128, SLABS = 4;
     constexpr bool ALDS = LDSM == 1 || LDSM == 2; // activation rows staged in LDS
+    static_assert(MT == 1 || !ALDS, "staged activations are for at most 16 rows");
     constexpr bool SCLDS = LDSM >= 2;             // the group scales / zeros of the workgroup's columns staged
     extern __shared__ u32x4 act_lds[]; // ALDS: rows x (K + 16) bytes, then the staged scales, then zeros
 
@@ -47,10 +50,12 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     int const KT = p.k_tiles;
     int const strip0 = group * NS;
 
-    f32x4 acc[NS];
+    f32x4 acc[NS][MT];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
-        acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     constexpr uint32_t kPast = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K);
@@ -86,7 +91,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     struct Stage
     {
         u32x4 w[NS];
-        u32x2 a[ALDS ? 1 : SLABS];
+        u32x2 a[ALDS ? 1 : SLABS][MT];
         uint16_t s[NS];
         uint16_t z[NS];
     };
@@ -101,7 +106,10 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
         {
 #pragma unroll
             for (int j = 0; j < SLABS; ++j)
-                st.a[j] = buffer_load_x2(act_rsrc, (a_lane + (uint32_t) (kt * TK + j * 32)) | past);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    st.a[j][mt] = buffer_load_x2(
+                        act_rsrc, (a_lane + (uint32_t) mt * 16u * (uint32_t) K + (uint32_t) (kt * TK + j * 32)) | past);
         }
         if constexpr (!SCLDS)
         {
@@ -135,7 +143,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     // Saturation to +-448 is part of the conversion: the wavefront runs with the conversion instruction's
     // own saturating mode switched on (fp8_saturation_on below), as the tiled kernel does, so no clamp and
     // no test for scales that could reach the limit is needed.
-    auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 a, auto clamp_tag)
+    auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 const (&a)[MT], auto clamp_tag)
     {
         constexpr bool CLAMP = decltype(clamp_tag)::value;
 #pragma unroll
@@ -149,19 +157,24 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
                     b[2 * j + h] = (int) dequant4_fp8<ZERO, CLAMP>(st.w[s][j], h, sc, zr, nib);
-            acc[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, acc[s], 0, 0, 0, 0, 0, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[s][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[mt], b, acc[s][mt], 0, 0, 0, 0, 0, 0);
         }
     };
     auto compute = [&](Stage const& st, int kt)
     {
-        i32x8 a;
+        i32x8 a[MT];
 #pragma unroll
         for (int j = 0; j < SLABS; ++j)
-        {
-            u32x2 const v = ALDS ? *reinterpret_cast<u32x2 const*>(a_lds + (uint32_t) (kt * TK + j * 32)) : st.a[ALDS ? 0 : j];
-            a[2 * j] = (int) v[0];
-            a[2 * j + 1] = (int) v[1];
-        }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+            {
+                u32x2 const v = ALDS ? *reinterpret_cast<u32x2 const*>(a_lds + (uint32_t) (kt * TK + j * 32))
+                                     : st.a[ALDS ? 0 : j][mt];
+                a[mt][2 * j] = (int) v[0];
+                a[mt][2 * j + 1] = (int) v[1];
+            }
         convert_and_multiply(st, kt, a, std::false_type{});
     };
 
@@ -277,22 +290,24 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 
     // ---- cross-wavefront reduction (fixed order) and epilogue: out = T(alpha * sum + bias) ----
     fp8_saturation_off();
-    constexpr int SLOTS = NS * 4;
+    constexpr int SLOTS = NS * MT * 4;
     __shared__ float red[WAVES][SLOTS][64];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            if (kg * 4 + r < p.m)
-                red[wave][s * 4 + r][lane] = acc[s][r];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (mt * 16 + kg * 4 + r < p.m)
+                    red[wave][(s * MT + mt) * 4 + r][lane] = acc[s][mt][r];
     __syncthreads();
 
     uint16_t* out16 = static_cast<uint16_t*>(p.out);
     for (int e = threadIdx.x; e < SLOTS * 64; e += WAVES * 64)
     {
         int const slot = e >> 6, ln = e & 63;
-        int const s = slot >> 2, r = slot & 3;
-        int const row = (ln >> 4) * 4 + r;
+        int const s = (slot >> 2) / MT, mt = (slot >> 2) % MT, r = slot & 3;
+        int const row = mt * 16 + (ln >> 4) * 4 + r;
         if (row >= p.m || strip0 + s >= p.strips)
             continue;
         float sum = 0.f;
@@ -336,7 +351,7 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
         return {env.stream_shape[0], env.stream_shape[1], env.stream_shape[2], env.stream_shape[3]};
     // measured on MI355X.  Activations that fit the LDS staging area: one strip per wavefront
     // and 8-way split K (two strips on very wide matrices, deeper prefetch on long K).
-    if (act_lds_bytes(m, k) <= kMaxActLds)
+    if (m <= 16 && act_lds_bytes(m, k) <= kMaxActLds)
     {
         // the group scales join the activations in LDS from K = 8192 on (2-4 % there; on K = 4096 the
         // staging pass costs more than the loads it saves)
@@ -350,6 +365,10 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
     // on very wide matrices with more than 8 rows; narrow matrices keep one strip (swept over every
     // instantiated shape on the Llama-3-8B / 70B layer shapes, M = 8 and 16)
     int const lds = scale_lds_bytes(k_tiles, 4, true) <= kMaxStagedLds ? 3 : 0;
+    // 17..32 rows (two 16-row tiles per wavefront): the activation loads weigh twice as much, so wider
+    // workgroups earlier (70B qkv, 640 strips, M = 32: 48.9 / 35.7 / 23.3 us with 1 / 2 / 4 strips)
+    if (m > 16)
+        return strips > 512 ? W4a8Shape{4, 8, 2, lds} : (strips >= 256 ? W4a8Shape{2, 8, 2, lds} : W4a8Shape{1, 8, 2, lds});
     if (strips > 1024)
         return m > 8 ? W4a8Shape{4, 8, 2, lds} : W4a8Shape{2, 8, 2, lds};
     if (strips >= 512 || (strips >= 384 && m > 4))
@@ -357,10 +376,10 @@ W4a8Shape pick_shape(int m, int k, int strips, int k_tiles)
     return {1, 8, 2, lds};
 }
 
-template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM>
+template <int ODT, bool ZERO, int NS, int WAVES, int PF, int LDSM, int MT = 1>
 int launch_variant(StreamParams sp, hipStream_t stream)
 {
-    auto kernel = stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF, LDSM>;
+    auto kernel = stream_w4a8_kernel<ODT, ZERO, NS, WAVES, PF, LDSM, MT>;
     size_t lds = 0;
     if constexpr (LDSM != 0)
     {
@@ -378,7 +397,7 @@ int launch_variant(StreamParams sp, hipStream_t stream)
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
-    note_launch("stream w4a8 ns=%d waves=%d pf=%d lds=%d", NS, WAVES, PF, LDSM);
+    note_launch("stream w4a8 mt=%d ns=%d waves=%d pf=%d lds=%d", MT, NS, WAVES, PF, LDSM);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, sp);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
@@ -390,6 +409,21 @@ template <int ODT, bool ZERO>
 int launch_shaped(StreamParams const& sp, hipStream_t s)
 {
     W4a8Shape const sh = pick_shape(sp.m, sp.k, sp.strips, sp.k_tiles);
+    if (sp.m > 16)
+    {
+        // 17..32 rows: two 16-row tiles per wavefront, activations from registers
+#define WOQ_SHAPE2(NS_, WAVES_, PF_, LDS_)                                                                             \
+    if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                                   \
+        return launch_variant<ODT, ZERO, NS_, WAVES_, PF_, LDS_, 2>(sp, s);
+        WOQ_SHAPE2(1, 8, 2, 0)
+        WOQ_SHAPE2(2, 8, 2, 0)
+        WOQ_SHAPE2(1, 8, 2, 3)
+        WOQ_SHAPE2(2, 8, 2, 3)
+        WOQ_SHAPE2(4, 8, 2, 3)
+#undef WOQ_SHAPE2
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 stream shape ns=%d waves=%d pf=%d lds=%d is not instantiated for 17..32 rows",
+            sh.ns, sh.waves, sh.pf, sh.lds);
+    }
 #define WOQ_SHAPE(NS_, WAVES_, PF_, LDS_)                                                                              \
     if (sh.ns == NS_ && sh.waves == WAVES_ && sh.pf == PF_ && sh.lds == LDS_)                                   \
         return launch_variant<ODT, ZERO, NS_, WAVES_, PF_, LDS_>(sp, s);

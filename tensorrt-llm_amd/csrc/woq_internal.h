@@ -325,7 +325,8 @@ int raise_lds_once(std::atomic<uint64_t>& raised, void const* kernel, int bytes)
 
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
 constexpr int kStreamMaxM = 128;
-constexpr int kStreamW4a8MaxM = 16;
+constexpr int kStreamW4a8MaxM = 32;     // rows the W4A8 streaming kernel covers (two 16-row tiles per wavefront above 16)
+constexpr int kStreamW4a8AutoMaxM = 16; // rows up to which the built-in rule takes it
 // most LDS a streaming workgroup stages its operands in (activations, group scales and zeros, row
 // sums): what the CU's 160 KiB leave next to the static reduction buffer of the epilogue
 // (`slots` = strips per wavefront x 16-row tiles, 256 floats per slot and wavefront)

@@ -210,7 +210,50 @@ def test_w4a8_streaming_one_hot_rows_recover_e4m3_weight(pkg, oracle, dev):
         assert (out == oracle.round_f16(w8[rows])).all()
 
 
-def test_w4a8_streaming_kernel_refuses_more_than_16_rows(pkg, oracle, dev):
-    prob = oracle.make_w4a8_problem(17, 256, 64, seed=1, out_dtype="bf16")
+def test_w4a8_streaming_kernel_refuses_more_than_32_rows(pkg, oracle, dev):
+    prob = oracle.make_w4a8_problem(33, 256, 64, seed=1, out_dtype="bf16")
     with pytest.raises(RuntimeError, match="unsupported m"):
-        _run(pkg, oracle, dev, prob, 17, 256, 64, "bf16", direct_fp8=True, regime=STREAM)
+        _run(pkg, oracle, dev, prob, 33, 256, 64, "bf16", direct_fp8=True, regime=STREAM)
+
+
+@pytest.mark.parametrize("out_dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("M,K,N", [(17, 1024, 384), (32, 2176, 1040), (24, 4096, 4112), (31, 512, 10240 + 16),
+                                   (20, 8192, 48), (32, 256, 16)])
+def test_w4a8_streaming_two_row_tiles(pkg, oracle, dev, out_dtype, M, K, N):
+    """17 ... 32 rows on the streaming kernel (two 16-row tiles per wavefront, activations from registers;
+    one, two and four strips per wavefront by the built-in rule, a last column group that is only partly
+    there, fewer tile rows than wavefronts): same oracle, same bar, with and without zeros and bias; what
+    AUTO picks here; the GEMM kernel on the same inputs agrees to float32 summation order."""
+    prob = oracle.make_w4a8_problem(M, K, N, seed=M + N, out_dtype=out_dtype)
+    rng = np.random.default_rng(M)
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+    for z, b in ((None, None), (zeros, bias)):
+        out, ref = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=z, bias=b, regime=STREAM)
+        assert "stream w4a8 mt=2" in _launch(pkg), _launch(pkg)
+        assert _perr(oracle, out, ref, prob) < TOL, (M, K, N, z is not None)
+        gemm, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=z, bias=b, regime=GEMM)
+        assert oracle.max_rel_err(gemm, out) < 2e-3
+    auto, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=zeros, bias=bias)
+    expect_stream = not (M > 24 and K >= 2 * N)
+    assert ("stream w4a8 mt=2" in _launch(pkg)) == expect_stream, _launch(pkg)
+    if expect_stream:
+        assert (auto == out).all()
+
+
+def test_w4a8_streaming_two_row_tiles_one_hot_rows(pkg, oracle, dev):
+    """One-hot activation rows through the two-tile variant: row r of the output is row k_r of the
+    e4m3-rounded dequantized weight, bit for bit - with and without zero-points."""
+    M, K, N = 32, 1024, 528
+    rng = np.random.default_rng(9)
+    q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    s = oracle.round_f16(np.exp(rng.uniform(-2, 3, (K // 128, N))).astype(np.float32))
+    zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+    rows = rng.choice(K, size=M, replace=False)
+    act = np.zeros((M, K), np.float32)
+    act[np.arange(M), rows] = 1.0
+    prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+    for z in (None, zeros):
+        out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=STREAM)
+        w8 = oracle.dequantize(q, s, z, 128, "fp8")
+        assert (out == oracle.round_f16(w8[rows])).all()
