@@ -129,7 +129,7 @@ def _cases():
         for group in (128, 64):
             out += [("c4", s, "w4", group, "bf16", m) for m in (1, 2, 4, 8, 16, 32, 64, 128, 256)]
     for s in ("70b_qkv", "70b_o_proj", "70b_gate_up", "70b_down"):
-        out += [("c5", s, "w4a8", 128, "bf16", m) for m in (1, 16, 256, 4096)]
+        out += [("c5", s, "w4a8", 128, "bf16", m) for m in (1, 16, 32, 256, 4096)]
     # fp16: one case per regime and kernel family (streaming, deferred-scale, exact-dequantize, fp8)
     out += [("fp16", "8b_qkv", "w4", 128, "fp16", m) for m in (1, 16, 48, 4096)]
     out += [("fp16", "70b_o_proj", "w4", 64, "fp16", m) for m in (4, 128)]
@@ -182,9 +182,9 @@ def test_full_size_one_hot_rows_return_weight_rows(pkg, dev, name, kind, group, 
 
 
 @pytest.mark.parametrize("name", ["70b_qkv", "70b_o_proj", "70b_gate_up", "70b_down"])
-@pytest.mark.parametrize("m", [16, 256])
+@pytest.mark.parametrize("m", [16, 24, 256])
 def test_full_size_w4a8_one_hot_rows_return_e4m3_weight_rows(pkg, dev, name, m):
-    """W4A8 (streaming kernel at 16 rows, fp8 GEMM at 256): one-hot rows are exact in e4m3, so row r
+    """W4A8 (streaming kernel at 16 rows and, with two row tiles per wavefront, at 24; fp8 GEMM at 256): one-hot rows are exact in e4m3, so row r
     of the output is alpha * (row k_r of the e4m3-rounded dequantized weight), rounded once to bf16 -
     bit for bit, at the full layer shapes."""
     L = layer(pkg, dev, name, "w4a8")
