@@ -316,8 +316,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         // the conversion pipeline's head: the stages that the first matrix instructions expect done
         constexpr int PER0 = UNITS / (RT * NS);
         ConvState cs;
+        constexpr bool PIPELINED = RT >= 8; // (64-row tiles measured 2-8 % faster without the stage pipeline, 128-row tiles 3-6 % slower)
 #pragma unroll
-        for (int lead = 0; lead < 3; ++lead)
+        for (int lead = 0; PIPELINED && lead < 3; ++lead)
 #pragma unroll
             for (int stage = 0; stage < 3 - lead; ++stage)
 #pragma unroll
@@ -366,15 +367,28 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 // FMAs of those converted behind t - 2, and so on (PER units per instruction)
                 constexpr int PER = UNITS / (RT * NS);
                 int const t = rt * NS + s;
+                if constexpr (PIPELINED)
+                {
 #pragma unroll
-                for (int stage = 3; stage >= 0; --stage)
+                    for (int stage = 3; stage >= 0; --stage)
+#pragma unroll
+                        for (int x = 0; x < PER; ++x)
+                        {
+                            int const cu = (t + 3 - stage) * PER + x;
+                            if (cu < UNITS)
+                                conv_stage(cs, b_make, st_conv, cu, stage);
+                        }
+                }
+                else
+                {
+                    // fewer row tiles: several units per matrix instruction, independent of each other -
+                    // each goes through its four stages here
 #pragma unroll
                     for (int x = 0; x < PER; ++x)
-                    {
-                        int const cu = (t + 3 - stage) * PER + x;
-                        if (cu < UNITS)
-                            conv_stage(cs, b_make, st_conv, cu, stage);
-                    }
+#pragma unroll
+                        for (int stage = 0; stage < 4; ++stage)
+                            conv_stage(cs, b_make, st_conv, t * PER + x, stage);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
