@@ -103,9 +103,10 @@ typedef enum woq_regime
  *   out              [m, n]            out_dtype
  *   n                LOGICAL number of output columns (the reference plugins receive the packed
  *                    column count and multiply it back: `real_n`)
- *   group_size       0 (per-channel, the WeightOnlyQuantMatmul plugin), 64, 128, or - with fp16 / bf16
- *                    activations - any larger multiple of 64 (what the reference's Hopper kernels accept,
- *                    launchers/fpA_intB_launcher_sm90.inl:191-198); above 128 the last group may be
+ *   group_size       0 (per-channel, the WeightOnlyQuantMatmul plugin), 64, 128, or any larger multiple
+ *                    of 64 (W4A8: 128 and any larger multiple of 128) - what the reference's Hopper
+ *                    kernels accept, a multiple of their K tile
+ *                    (launchers/fpA_intB_launcher_sm90.inl:191-198); above 128 the last group may be
  *                    shorter: scales / zeros then hold ceil(k / group_size) rows
  *   alpha            used only with FP8_ALPHA; otherwise must be 1 or is ignored as in the reference
  *   workspace        device scratch of at least woq_workspace_bytes(...) bytes (may be NULL when
@@ -150,10 +151,19 @@ int woq_matmul_check(const woq_matmul_args* args);
  * call that would need more scratch than that returns WOQ_ERR_WORKSPACE and launches nothing.
  * All calls on one GPU share that GPU's array: calls that may overlap there (different streams)
  * race; order them, or use woq_matmul with separate workspaces.  Every element of the scratch a
- * call reads was written by that call, so nothing is cleared between calls. */
+ * call reads was written by that call, so nothing is cleared between calls.
+ * Set-up that is not stream work - looking up the array's device address (hipGetSymbolAddress), reading
+ * the WOQ_* environment, raising a kernel's dynamic-LDS limit (hipFuncSetAttribute, once per kernel
+ * variant and device) - happens on first use: call woq_static_init() on each device before the first
+ * woq_matmul_static there, and, before capturing a call into a HIP graph, run that same call (same
+ * shape and flags, hence the same kernel variant) once outside capture. */
 #define WOQ_STATIC_SCRATCH_BYTES (32u << 20)
 int woq_matmul_static(const woq_matmul_args* args, void* stream);
 size_t woq_static_scratch_bytes(void);
+/* Resolves the scratch array's address on the CURRENT device and reads the environment overrides, so that
+ * woq_matmul_static itself makes no non-stream runtime call for them.  Idempotent; WOQ_OK or
+ * WOQ_ERR_RUNTIME.  (woq_matmul_static still resolves the address by itself if this was not called.) */
+int woq_static_init(void);
 
 /* Device scratch that is enough for every woq_matmul call of this n, k, quant_algo with AT MOST m
  * rows (pass the largest m, as the reference passes its profile's maxM): a region for smoothed
@@ -337,21 +347,6 @@ int woq_rmsnorm_prequant(void* out, const void* x, const void* gamma, const void
  * with fp16 scales (the W4A8 B operand). */
 int woq_dequantize(void* out, const void* weight, const void* scales, const void* zeros, int32_t k, int32_t n,
     int32_t group_size, int32_t quant_type, int32_t dtype, void* stream);
-
-/* ---- measurement probes (no counterpart in the reference) -------------------------------------- */
-
-/* What the hardware allows, measured with the same harness as the kernels (bench.py --mode ceilings).
- * woq_probe_read: a plain streaming read of `bytes` of device memory (every wavefront reads
- * kib_per_wave contiguous KiB, loads_in_flight of 1, 2, 4 or 8 16-byte loads per lane outstanding);
- * `sink` is 4 KiB of device memory.  woq_probe_empty: a kernel that does nothing.  woq_probe_mfma:
- * nothing but matrix instructions (kind 0: v_mfma_f32_16x16x32_bf16, 1: v_mfma_f32_16x16x128_f8f6f4
- * on e4m3, 2: v_mfma_f32_32x32x16_bf16) on `workgroups` x 4 wavefronts, multiplying the same operand registers every time
- * (random_operands 0: least switching activity) or four pseudo-random operand pairs in turn (1: what
- * the power management sustains under real data); returns the floating-point operations of the
- * launch (negative on a bad argument). */
-int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream);
-int woq_probe_empty(void* sink, void* stream);
-double woq_probe_mfma(int kind, int random_operands, int iters, int workgroups, void* sink, void* stream);
 
 /* ---- misc ------------------------------------------------------------------------------------ */
 

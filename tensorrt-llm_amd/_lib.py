@@ -64,6 +64,7 @@ def _load():
         "woq_matmul_check": (ctypes.c_int, [ctypes.POINTER(MatmulArgs)]),
         "woq_matmul_static": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), vp]),
         "woq_static_scratch_bytes": (sz, []),
+        "woq_static_init": (ctypes.c_int, []),
         "woq_grouped_matmul": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs), vp]),
         "woq_grouped_matmul_check": (ctypes.c_int, [ctypes.POINTER(GroupedMatmulArgs)]),
         "woq_workspace_bytes": (sz, [i32, i32, i32, i32, i32]),
@@ -85,23 +86,27 @@ def _load():
         "woq_describe_tactic": (ctypes.c_int, [ctypes.POINTER(MatmulArgs), ctypes.c_char_p, sz]),
         "woq_export_tactics": (sz, [ctypes.c_char_p, sz]),
         "woq_import_tactics": (ctypes.c_int, [ctypes.c_char_p]),
-        "woq_probe_read": (ctypes.c_int, [vp, sz, i32, i32, vp, vp]),
-        "woq_probe_empty": (ctypes.c_int, [vp, vp]),
-        "woq_probe_mfma": (ctypes.c_double, [i32, i32, i32, i32, vp, vp]),
         "woq_reload_env": (None, []),
         "woq_last_error": (ctypes.c_char_p, []),
         "woq_last_launch": (ctypes.c_char_p, []),
         "woq_abi_version": (ctypes.c_int, []),
         "woq_layout_version": (ctypes.c_int, []),
     }
-    for name, (res, args) in sig.items():
-        fn = getattr(lib, name)  # AttributeError here = header and library disagree
-        fn.restype = res
-        fn.argtypes = args
-    return lib, tuple(sig)
+    # measurement probes (csrc/woq_probes.h): in the library, outside the drop-in boundary
+    probes = {
+        "woq_probe_read": (ctypes.c_int, [vp, sz, i32, i32, vp, vp]),
+        "woq_probe_empty": (ctypes.c_int, [vp, vp]),
+        "woq_probe_mfma": (ctypes.c_double, [i32, i32, i32, i32, vp, vp]),
+    }
+    for table in (sig, probes):
+        for name, (res, args) in table.items():
+            fn = getattr(lib, name)  # AttributeError here = header and library disagree
+            fn.restype = res
+            fn.argtypes = args
+    return lib, tuple(sig), tuple(probes)
 
 
-lib, EXPORTED = _load()
+lib, EXPORTED, PROBES = _load()
 
 
 def check(status: int) -> None:

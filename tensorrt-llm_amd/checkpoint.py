@@ -1,4 +1,4 @@
-"""Checkpoint front-end: GPTQ / AutoAWQ tensors -> the operands of the groupwise matmul.
+"""Checkpoint front-end: float / GPTQ / AutoAWQ / ModelOpt tensors -> the operands of the two matmul ops.
 
 Counterpart of `postprocess_weight_only_groupwise` and its helpers
 (tensorrt_llm/quantization/functional.py:832-868, 903-1037), which the reference's weights loader
@@ -16,6 +16,8 @@ calls per tensor.  Same arithmetic, same argument conventions:
     byte, signed nibbles), `weight_scale` [N, K/g], `input_quantizer._pre_quant_scale` [K]; for W4A8
     also the per-tensor `activation_scaling_factor` and `weights_scaling_factor_2`, folded by the
     loader (tensorrt_llm/models/modeling_utils.py:1626-1682): `postprocess_modelopt_awq`, `fold_w4a8`.
+  * float weights of per-channel layers (W8A16 / W4A16): `postprocess_weight_only`
+    (functional.py:875-901: transpose, TP split, padding, symmetric quantization, bias).
   * q / k / v (or gate / up) tensors that arrive separately are concatenated along N first
     (functional.py:932-944): `concat_gptq_parts`, and list arguments of `postprocess_modelopt_awq`.
 
@@ -166,12 +168,71 @@ def fold_w4a8(weights_scaling_factor: torch.Tensor, prequant_scaling_factor: tor
     restores the magnitude in the epilogue.  Returns the four tensors under the reference's names."""
     act_sf = torch.as_tensor(activation_scaling_factor)
     wsf2 = torch.as_tensor(weights_scaling_factor_2)
+    # the reference divides IN PLACE (`weights[name] /= ...`): whatever the type and shape of the per-tensor
+    # factors (the layers declare them float32 of shape (1,), quantization/layers.py), the quotient is
+    # formed in the promoted type and rounded back to the tensor's own dtype, which the tensor keeps
+    scales = weights_scaling_factor.clone()
+    scales /= wsf2
+    pqs = prequant_scaling_factor.clone()
+    pqs /= act_sf
     return {
-        "weights_scaling_factor": (weights_scaling_factor / wsf2).to(torch.float16).contiguous(),
-        "prequant_scaling_factor": (prequant_scaling_factor / act_sf).contiguous(),
+        "weights_scaling_factor": scales.to(torch.float16).contiguous(),
+        "prequant_scaling_factor": pqs.contiguous(),
         "alpha": (act_sf.to(torch.float32) * wsf2.to(torch.float32)).reshape(1),
         "activation_scaling_factor": act_sf,
     }
+
+
+def postprocess_weight_only(weight: torch.Tensor, quant_type: torch.dtype = torch.int8, *, bias: torch.Tensor | None = None,
+                            tp_split=None, padded_shape=None):
+    """Per-channel loader hook: a float weight of one linear layer -> {"weight", "per_channel_scale"}
+    (+ "bias"), the operands of `weight_only_quant_matmul` (W8A16 with quant_type torch.int8, W4A16 with
+    torch.quint4x2).  Counterpart of `postprocess_weight_only`
+    (tensorrt_llm/quantization/functional.py:875-901), in its order of operations:
+
+      * `weight` [out_features, in_features] (or [E, out, in]) as checkpoints store it is transposed to the
+        op's [K, N];
+      * `tp_split` = (dim, size, rank) cuts the logical [K, N] weight (dim 1: column-parallel, 0:
+        row-parallel).  With `padded_shape` = the layer's (in_features, out_features) AFTER padding
+        (see padded_features) the cut is the reference's `torch.split(v, padded size, dim)[rank]`: ranks
+        own runs of the padded per-rank size, the last one what is left, and each piece is padded with
+        zeros up to the padded shape; without it the weight is cut into `size` equal parts;
+      * `symmetric_quantize_last_axis_of_batched_matrix` (one scale per output column: amax / 2^(bits-1),
+        round half away from zero) quantizes the piece and lays it out for the kernels;
+      * the bias follows the columns of a column-parallel layer (split and padded the same way) and is
+        passed through otherwise."""
+    if quant_type not in (torch.int8, torch.quint4x2):
+        raise ValueError("quant_type must be torch.int8 or torch.quint4x2")
+    if weight.dim() not in (2, 3) or not weight.is_floating_point():
+        raise ValueError("a float weight [out_features, in_features] (or [E, out, in]) is required")
+    v = weight.transpose(-1, -2)
+    tp_dim = None
+    if tp_split is not None:
+        tp_dim, tp_size, tp_rank = tp_split
+        if tp_dim not in (0, 1) or not 0 <= tp_rank < tp_size:
+            raise ValueError("tp_split is (dim 0 | 1, size, rank)")
+        axis = tp_dim + (v.dim() - 2)
+        if padded_shape is not None:
+            pieces = torch.split(v, padded_shape[tp_dim], axis)
+            if tp_rank >= len(pieces):
+                raise ValueError("rank %d owns nothing: %d pieces of %d" % (tp_rank, len(pieces), padded_shape[tp_dim]))
+            v = pieces[tp_rank]
+        else:
+            v = v.chunk(tp_size, axis)[tp_rank]
+    if padded_shape is not None:
+        v = pad_like(v, tuple(v.shape[:-2]) + tuple(padded_shape))
+    processed, scales = ops.symmetric_quantize_last_axis_of_batched_matrix(v.contiguous(), quant_type)
+    out = {"weight": processed, "per_channel_scale": scales}
+    if bias is not None:
+        if tp_dim == 1:
+            if padded_shape is not None:
+                bias = torch.split(bias, padded_shape[1], -1)[tp_rank]
+            else:
+                bias = bias.chunk(tp_size, -1)[tp_rank]
+        if padded_shape is not None:
+            bias = pad_like(bias, tuple(bias.shape[:-1]) + (padded_shape[1],))
+        out["bias"] = bias.contiguous()
+    return out
 
 
 def postprocess_modelopt_awq(weight, weight_scale, pre_quant_scale, dtype=torch.float16, *, group_size: int = 128,

@@ -394,8 +394,11 @@ int validate(woq_matmul_args const* a, MatmulProblem& p)
     // ("The group size must a multiple of <K tile>", launchers/fpA_intB_launcher_sm90.inl:191-198)
     if (a->group_size < 0 || a->group_size % 64)
         return fail(WOQ_ERR_UNSUPPORTED, "group_size must be 0 (per-channel) or a multiple of 64 (got %d)", a->group_size);
-    if (w4a8 && a->group_size != 128)
-        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 supports group_size 128 only (got %d)", a->group_size);
+    // e4m3 activations: 128 as the reference's pre-Hopper launcher (fpA_intB_gemm_template.h:136-142) and
+    // every further multiple of 128 as its Hopper one (launchers/fpA_intB_launcher_sm90.inl:190-198,
+    // tests/quantization/test_weight_only_groupwise_quant_matmul.py:429-455)
+    if (w4a8 && (a->group_size < 128 || a->group_size % 128))
+        return fail(WOQ_ERR_UNSUPPORTED, "W4A8 supports group sizes that are multiples of 128 only (got %d)", a->group_size);
     // m == 0 is a no-op (weightOnlyQuantMatmulPlugin.cpp:303): empty tensors may carry null pointers
     if (a->m > 0 && (!a->act || !a->weight || !a->out))
         return fail(WOQ_ERR_INVALID_ARGUMENT, "act, weight and out must not be NULL");
@@ -704,6 +707,13 @@ int static_scratch_ptr(void** out)
 extern "C" size_t woq_static_scratch_bytes(void)
 {
     return WOQ_STATIC_SCRATCH_BYTES;
+}
+
+extern "C" int woq_static_init(void)
+{
+    (void) env_overrides(); // read (and allocate, on the host) once, here rather than inside a first call
+    void* ptr = nullptr;
+    return static_scratch_ptr(&ptr);
 }
 
 extern "C" int woq_matmul_static(const woq_matmul_args* args, void* stream)

@@ -4,7 +4,9 @@
 // with half scales, cpp/tensorrt_llm/kernels/cutlass_kernels/fpA_intB_gemm/fpA_intB_gemm_template.h,
 // selected by weightOnlyGroupwiseQuantMatmulPlugin.cpp:203-276): the int4 weight is dequantized
 // with fp16 scales/zeros and rounded to e4m3, the MMA accumulates fp8 x fp8 products in float32,
-// and the epilogue applies alpha and the bias: out = T(alpha * acc + bias).  Group size 128 only.
+// and the epilogue applies alpha and the bias: out = T(alpha * acc + bias).  Group sizes: 128 and its
+// multiples (the reference's pre-Hopper launcher takes 128 only, fpA_intB_gemm_template.h:136-142; its
+// Hopper launcher any multiple of the K tile, launchers/fpA_intB_launcher_sm90.inl:190-198).
 //
 // Same skeleton as the 16-bit prefill kernel (gemm_kernel.h): output tile 16*RT rows x 256
 // columns, 4 wavefronts side by side along N with 64 columns each; packed weights go global ->
@@ -84,7 +86,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
     constexpr uint32_t kOob = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K);
-    uint32_t const sz_bytes = (uint32_t) (K / 128) * (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes = (uint32_t) p.scale_rows * (uint32_t) p.n * 2u;
+    uint32_t const magic = p.group_magic; // groups above 128: table row of a tile row (w4a8_scale_row)
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) p.k_tiles * 1024u);
@@ -158,7 +161,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         else
         {
             int const s = (i - NS) % NS;
-            uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + x.sc_lane[s]) | past;
+            uint32_t const off = (w4a8_scale_row((uint32_t) kt, magic) * (uint32_t) p.n * 2u + x.sc_lane[s]) | past;
             if (i < 2 * NS)
                 st.s[s] = buffer_load_u16(sc_rsrc, off);
             else
@@ -600,6 +603,8 @@ int launch_gemm_w4a8(MatmulProblem const& p, void* stream)
     gp.k = p.k;
     gp.k_tiles = (p.k + 127) / 128;
     gp.strips = p.n / kTileN;
+    gp.scale_rows = (p.k + p.group_size - 1) / p.group_size;
+    gp.group_magic = w4a8_scale_row_magic(p.group_size);
     gp.tiles_m = (p.m + plan.rt * 16 - 1) / (plan.rt * 16);
     gp.tiles_n = (p.n + kGemmBN - 1) / kGemmBN;
     gp.k_splits = plan.k_splits;

@@ -8,6 +8,7 @@
 //                    constant or with pseudo-random operands
 #include <hip/hip_runtime.h>
 
+#include "../woq_probes.h"
 #include "device_common.h"
 
 namespace woq
@@ -139,6 +140,8 @@ extern "C" int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, i
 {
     if (!src || !sink || kib_per_wave <= 0 || bytes < (size_t) kib_per_wave * 1024)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: src, sink and a buffer of at least one wavefront's share");
+    if (loads_in_flight != 1 && loads_in_flight != 2 && loads_in_flight != 4 && loads_in_flight != 8)
+        return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: loads_in_flight must be 1, 2, 4 or 8");
     if (kib_per_wave % loads_in_flight)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: kib_per_wave must be a multiple of loads_in_flight");
     size_t const waves = bytes / ((size_t) kib_per_wave * 1024);

@@ -59,10 +59,11 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 
     constexpr uint32_t kPast = 0x80000000u;
     auto const act_rsrc = make_rsrc(p.act, (uint32_t) p.m * (uint32_t) K);
-    uint32_t const sz_bytes = (uint32_t) (K / TK) * (uint32_t) p.n * 2u;
+    uint32_t const sz_bytes = (uint32_t) p.scale_rows * (uint32_t) p.n * 2u;
     auto const sc_rsrc = make_rsrc(p.scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? p.zeros : p.scales, sz_bytes);
     auto const w_rsrc = make_rsrc(p.weight, (uint32_t) p.strips * (uint32_t) KT * 1024u);
+    uint32_t const magic = p.group_magic; // groups above 128: table row of a tile row (w4a8_scale_row)
 
     // strips past the end of N (last group only) are clamped for loads and skipped at the store
     uint32_t wlane[NS], sc_lane[NS];
@@ -116,7 +117,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
 #pragma unroll
             for (int s = 0; s < NS; ++s)
             {
-                uint32_t const off = ((uint32_t) kt * (uint32_t) p.n * 2u + sc_lane[s]) | past;
+                uint32_t const off = (w4a8_scale_row((uint32_t) kt, magic) * (uint32_t) p.n * 2u + sc_lane[s]) | past;
                 st.s[s] = buffer_load_u16(sc_rsrc, off);
                 if constexpr (ZERO)
                     st.z[s] = buffer_load_u16(zr_rsrc, off);
@@ -208,7 +209,10 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             int const kt = idx / (NS * 2), ch = idx - kt * (NS * 2);
             int const strip = strip0 + (ch >> 1) < p.strips ? strip0 + (ch >> 1) : p.strips - 1;
             at = (uint32_t) kt * SC_ROW + (uint32_t) ch * 16u;
-            return idx < sc_chunks ? ((uint32_t) kt * (uint32_t) p.n + (uint32_t) (strip * 16 + (ch & 1) * 8)) * 2u : kPast;
+            // (the staged copy keeps one row per tile row: tile rows of one group hold the same values)
+            return idx < sc_chunks
+                ? (w4a8_scale_row((uint32_t) kt, magic) * (uint32_t) p.n + (uint32_t) (strip * 16 + (ch & 1) * 8)) * 2u
+                : kPast;
         };
         u32x4 av[UA], sv[UA], zv[UA];
         uint32_t a_at[UA], s_at[UA];
@@ -458,8 +462,9 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream)
     if (p.m > kStreamW4a8MaxM)
         return fail(WOQ_ERR_UNSUPPORTED, "unsupported m: the W4A8 streaming kernel covers m <= %d (got %d)",
             kStreamW4a8MaxM, p.m);
-    if (p.act_dtype != WOQ_FP8_E4M3 || p.group_size != 128 || p.k % 128)
-        return fail(WOQ_ERR_INVALID_ARGUMENT, "W4A8 streaming kernel: e4m3 activations, group 128, k %% 128 == 0");
+    if (p.act_dtype != WOQ_FP8_E4M3 || p.group_size < 128 || p.group_size % 128 || p.k % 128)
+        return fail(WOQ_ERR_INVALID_ARGUMENT,
+            "W4A8 streaming kernel: e4m3 activations, group size a multiple of 128, k %% 128 == 0");
     StreamParams sp;
     sp.act = p.act;
     sp.pqs = nullptr;
@@ -474,6 +479,8 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream)
     sp.k = p.k;
     sp.k_tiles = p.k / 128;
     sp.strips = p.n / kTileN;
+    sp.scale_rows = (p.k + p.group_size - 1) / p.group_size;
+    sp.group_magic = w4a8_scale_row_magic(p.group_size);
     sp.groups = sp.groups_per_xcd = 0;
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;

@@ -120,6 +120,22 @@ __device__ __forceinline__ T after_mode_change(T v)
     return v;
 }
 
+// Row of the [ceil(k / group_size), n] scale / zero tables that the 128-row tile row kt reads.  Groups
+// are multiples of 128 (the reference's Hopper kernels take any multiple of their K tile for e4m3
+// activations, launchers/fpA_intB_launcher_sm90.inl:190-198; the last group may be shorter): `magic` is 0
+// for groups of 128 (row = tile row) and ceil(2^32 / (group_size / 128)) otherwise, an exact division by
+// multiplication for every tile row that can occur.
+__device__ __forceinline__ uint32_t w4a8_scale_row(uint32_t kt, uint32_t magic)
+{
+    return magic ? __umulhi(kt, magic) : kt;
+}
+
+inline uint32_t w4a8_scale_row_magic(int group_size)
+{
+    uint64_t const d = (uint64_t) group_size / 128;
+    return d <= 1 ? 0u : (uint32_t) ((((uint64_t) 1 << 32) + d - 1) / d);
+}
+
 typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 

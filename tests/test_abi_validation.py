@@ -34,6 +34,10 @@ def test_valid_combinations(pkg):
     assert status(pkg, group_size=0, quant_algo=L.ALGO_INT8_WEIGHT, act_dtype=L.FP16, out_dtype=L.FP16)[0] == 0
     assert status(pkg, m=0)[0] == 0                                     # m == 0 is a no-op, not an error
     assert status(pkg, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, alpha=0.5)[0] == 0
+    # e4m3 activations: multiples of 128 above 128 as the reference's Hopper kernels, shorter last group too
+    assert status(pkg, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, group_size=256)[0] == 0
+    assert status(pkg, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, k=1024, group_size=384)[0] == 0
+    assert status(pkg, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, k=128, group_size=256)[0] == 0
 
 
 @pytest.mark.parametrize("kw,code,text", [
@@ -41,7 +45,7 @@ def test_valid_combinations(pkg):
     (dict(act=None), -1, "NULL"),
     (dict(group_size=32), -3, "group_size"),
     (dict(group_size=96), -3, "multiple of 64"),
-    (dict(quant_algo=8, act_dtype=2, group_size=256), -3, "128"),
+    (dict(quant_algo=8, act_dtype=2, group_size=192), -3, "multiples of 128"),
     (dict(k=96), -2, "multiple of 64"),
     (dict(k=576, group_size=128), -2, "group_size"),
     (dict(n=250), -2, "multiple of 16"),

@@ -220,6 +220,133 @@ def test_w4a8_fold_is_the_loaders_and_the_oracles(pkg, oracle):
     assert f["alpha"].item() == np.float32(prob["alpha"])
 
 
+def test_w4a8_fold_keeps_dtypes_with_the_layers_factor_shapes(pkg):
+    """The layers declare alpha, activation_scaling_factor and weights_scaling_factor_2 as float32 of shape
+    (1,) (quantization/layers.py).  The reference divides in place, so a bf16 model's smoothing vector stays
+    bf16 and its group scales are rounded to bf16 before they become float16: quotient in float32, one
+    rounding to the tensor's own type."""
+    wsf = torch.tensor([[0.3, 1.7], [2.9, 0.011]], dtype=torch.bfloat16)
+    pqs = torch.tensor([[1.3, 0.7, 2.9]], dtype=torch.bfloat16)
+    act_sf, wsf2 = torch.tensor([0.3], dtype=torch.float32), torch.tensor([0.7], dtype=torch.float32)
+    f = pkg.checkpoint.fold_w4a8(wsf, pqs, act_sf, wsf2)
+    assert f["prequant_scaling_factor"].dtype == torch.bfloat16 and f["prequant_scaling_factor"].shape == (1, 3)
+    assert f["weights_scaling_factor"].dtype == torch.float16 and f["alpha"].dtype == torch.float32
+    assert f["alpha"].shape == (1,) and f["alpha"].item() == (act_sf * wsf2).item()
+    assert torch.equal(f["prequant_scaling_factor"], (pqs.float() / 0.3).to(torch.bfloat16))
+    assert torch.equal(f["weights_scaling_factor"], (wsf.float() / 0.7).to(torch.bfloat16).to(torch.float16))
+    # not the same as dividing by the factor rounded to bf16 first, nor as skipping the bf16 rounding
+    assert not torch.equal(f["weights_scaling_factor"], (wsf.float() / 0.7).to(torch.float16))
+    assert torch.equal(wsf, torch.tensor([[0.3, 1.7], [2.9, 0.011]], dtype=torch.bfloat16))  # inputs untouched
+    # fp16 model: same rule
+    f = pkg.checkpoint.fold_w4a8(wsf.to(torch.float16), pqs.to(torch.float16), act_sf, wsf2)
+    assert f["prequant_scaling_factor"].dtype == torch.float16
+
+
+# ---- per-channel layers from float weights ----------------------------------------------------------
+
+
+@pytest.mark.parametrize("quant_type,bits", [(torch.int8, 8), (torch.quint4x2, 4)])
+def test_postprocess_weight_only_quantizes_like_the_oracle(pkg, oracle, quant_type, bits):
+    """[out, in] float weight -> transposed, quantized per output column (amax / 2^(bits-1), half away from
+    zero: the oracle's symmetric_quantize), laid out for the kernels."""
+    N, K = 96, 128
+    rng = np.random.default_rng(31)
+    w = torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(torch.float16)
+    out = pkg.checkpoint.postprocess_weight_only(w, quant_type)
+    q, scale = oracle.symmetric_quantize(w.float().numpy().T.copy(), bits, "fp16")
+    assert (_decode(pkg, out["weight"], K, bits) == q).all()
+    assert out["per_channel_scale"].dtype == torch.float16
+    assert (out["per_channel_scale"].float().numpy() == scale).all()
+
+
+def test_postprocess_weight_only_tp_split_padding_and_bias(pkg, oracle):
+    """The reference's padded layers (functional.py:883-886, 896-899): a column-parallel layer with 100
+    output features on 2 ranks pads to 64 per rank; ranks own runs of 64 columns of the transposed weight
+    (rank 1: the remaining 36, padded with zeros); the bias is cut and padded with them.  Row-parallel
+    layers cut K and keep the bias."""
+    C = pkg.checkpoint
+    N, K = 100, 100
+    rng = np.random.default_rng(32)
+    w = torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(torch.bfloat16)
+    bias = torch.arange(N, dtype=torch.float32).to(torch.bfloat16)
+    k_pad, n_pad = C.padded_features(K, N, 0, tp_size=2)  # 128, 128 in total: 64 columns per rank
+    assert (k_pad, n_pad) == (128, 128)
+    wt = w.float().numpy().T  # [K, N]
+    for rank, cols in ((0, slice(0, 64)), (1, slice(64, 100))):
+        out = C.postprocess_weight_only(w, torch.int8, bias=bias, tp_split=(1, 2, rank), padded_shape=(k_pad, n_pad // 2))
+        piece = np.zeros((k_pad, 64), np.float32)
+        piece[:K, :cols.stop - cols.start] = wt[:, cols]
+        q, scale = oracle.symmetric_quantize(piece, 8, "bf16")
+        assert (_decode(pkg, out["weight"], k_pad, 8) == q).all()
+        assert (out["per_channel_scale"].float().numpy() == scale).all()
+        want_bias = torch.zeros(64, dtype=torch.bfloat16)
+        want_bias[:cols.stop - cols.start] = bias[cols]
+        assert torch.equal(out["bias"], want_bias)
+    # row-parallel, unpadded: equal parts of K, bias passed through
+    out = C.postprocess_weight_only(w[:, :64].contiguous(), torch.quint4x2, bias=bias, tp_split=(0, 2, 1))
+    q, scale = oracle.symmetric_quantize(wt[32:64].copy(), 4, "bf16")
+    assert (_decode(pkg, out["weight"], 32, 4)[:32] == q).all() and torch.equal(out["bias"], bias)
+    with pytest.raises(ValueError):
+        C.postprocess_weight_only(w.to(torch.int8), torch.int8)
+    # a batch of experts [E, out, in] keeps its leading dimension
+    e = C.postprocess_weight_only(torch.stack([w[:64, :64], w[:64, 36:]]).contiguous(), torch.int8)
+    assert e["per_channel_scale"].shape == (2, 64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("quant_type,bits,M", [(torch.int8, 8, 1), (torch.quint4x2, 4, 40)])
+def test_postprocess_weight_only_layer_runs_through_the_matmul(pkg, oracle, dev, quant_type, bits, M):
+    """Float checkpoint weight -> per-channel hook -> GPU matmul == the oracle's dequantize-then-matmul on
+    the oracle's own quantization of the same weight."""
+    N, K = 512, 1024
+    rng = np.random.default_rng(33)
+    w = torch.from_numpy((rng.standard_normal((N, K)) * 0.02).astype(np.float32)).to(torch.float16)
+    t = pkg.checkpoint.postprocess_weight_only(w, quant_type)
+    act = oracle.round_f16(rng.standard_normal((M, K)).astype(np.float32))
+    F = pkg.functional
+    out = F.weight_only_quant_matmul(torch.from_numpy(act).to(torch.float16).to(dev), t["weight"].to(dev),
+                                     t["per_channel_scale"].to(dev), F.INT8 if bits == 8 else F.INT4, "float16")
+    torch.cuda.synchronize()
+    q, scale = oracle.symmetric_quantize(w.float().numpy().T.copy(), bits, "fp16")
+    ref = oracle.woq_matmul_ref(act, q, scale, group_size=0, act_dtype="fp16")
+    assert oracle.max_rel_err(out.float().cpu().numpy(), ref) < 1e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [4, 200])
+def test_modelopt_w4a8_layer_runs_through_the_matmul(pkg, oracle, dev, M):
+    """A ModelOpt-style W4A8 layer (int8 [N/2, K] weight, [N, K/g] scales, smoothing vector, the two per-tensor
+    factors as float32 tensors of shape (1,)) -> postprocess_modelopt_awq -> woq_matmul with 16-bit activations
+    and the smoothing vector == the oracle on the operands of its own benchmark generator, which folds the same
+    factors independently."""
+    K, N, g = 512, 384, 128
+    seed = 50 + M
+    prob = oracle.make_w4a8_problem(M, K, N, seed=seed, out_dtype="bf16")
+    # the unfolded tensors, as the generator defines them
+    q, scale = oracle.make_w4_groupwise_sym(K, N, g, seed, "fp32")
+    rng = np.random.default_rng(seed + 7)
+    smooth = oracle.round_to(rng.uniform(0.5, 2.0, size=(K,)).astype(np.float32), "bf16")
+    act = oracle.make_activations(M, K, seed + 13, "bf16")
+    act_sf = np.float32(np.abs(act * smooth).max() / 448.0)
+    wsf2 = np.float32(np.abs(q.astype(np.float32).reshape(K // g, g, N) * scale[:, None, :]).max() / 448.0)
+    assert (q == prob["q"]).all()
+    t = pkg.checkpoint.postprocess_modelopt_awq(
+        _modelopt_pack(q), torch.from_numpy(scale.T.copy()), torch.from_numpy(smooth), torch.float32, group_size=g,
+        activation_scaling_factor=torch.tensor([act_sf]), weights_scaling_factor_2=torch.tensor([wsf2]))
+    assert (t["weights_scaling_factor"].float().numpy() == prob["scales"]).all()
+    pqs = t["prequant_scaling_factor"].to(torch.bfloat16).reshape(-1)
+    assert (pqs.float().numpy() == prob["pre_quant_scale"]).all()
+    F = pkg.functional
+    out = F.weight_only_groupwise_quant_matmul(
+        torch.from_numpy(prob["act"]).to(torch.bfloat16).to(dev), pqs.to(dev), t["weight"].to(dev),
+        t["weights_scaling_factor"].to(dev), None, None, t["alpha"], F.PRE_QUANT_SCALE | F.FP8_ALPHA, g, "bfloat16")
+    torch.cuda.synchronize()
+    ref = oracle.woq_matmul_ref(prob["act"], prob["q"], prob["scales"], None, None, prob["pre_quant_scale"],
+                                prob["alpha"], g, "bf16", w4a8=True)
+    assert abs(float(t["alpha"]) - prob["alpha"]) <= 1e-7 * prob["alpha"]
+    assert oracle.max_rel_err(out.float().cpu().numpy(), ref) < 1e-2
+
+
 # ---- TensorRT-LLM checkpoints (reference-layout weights) ---------------------------------------------
 
 import json

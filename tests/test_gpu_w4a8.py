@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, direct_fp8=False, regime=0):
+def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, direct_fp8=False, regime=0, group=128):
     F = pkg.functional
     w = preprocess(pkg, oracle, prob["q"], 4, torch.float8_e4m3fn).to(dev)
     scales = to_dev(prob["scales"], "fp16", dev)
@@ -22,21 +22,21 @@ def _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=None, bias=None, dire
     if direct_fp8:
         a8 = oracle.apply_per_channel_scale(prob["act"], prob["pre_quant_scale"], out_dtype, "fp8")
         act = torch.from_numpy(a8).to(dev).to(torch.float8_e4m3fn)
-        out = F.woq_matmul_raw(act, None, w, scales, z, b, n=N, k=K, group_size=128, quant_algo=algo,
+        out = F.woq_matmul_raw(act, None, w, scales, z, b, n=N, k=K, group_size=group, quant_algo=algo,
                                alpha=prob["alpha"], out_dtype=TORCH_DT[out_dtype], regime=regime)
-        ref = oracle.woq_matmul_ref(a8, prob["q"], prob["scales"], zeros, bias, None, prob["alpha"], 128, out_dtype,
+        ref = oracle.woq_matmul_ref(a8, prob["q"], prob["scales"], zeros, bias, None, prob["alpha"], group, out_dtype,
                                     w4a8=True)
     else:
         algo |= F.PRE_QUANT_SCALE
         out = F.woq_matmul_raw(to_dev(prob["act"], out_dtype, dev), to_dev(prob["pre_quant_scale"], out_dtype, dev), w,
-                               scales, z, b, n=N, k=K, group_size=128, quant_algo=algo, alpha=prob["alpha"],
+                               scales, z, b, n=N, k=K, group_size=group, quant_algo=algo, alpha=prob["alpha"],
                                out_dtype=TORCH_DT[out_dtype], regime=regime)
         ref = oracle.woq_matmul_ref(prob["act"], prob["q"], prob["scales"], zeros, bias, prob["pre_quant_scale"],
-                                    prob["alpha"], 128, out_dtype, w4a8=True)
+                                    prob["alpha"], group, out_dtype, w4a8=True)
     torch.cuda.synchronize()
     # floor of the per-column norm: the expected output magnitude of each column for these operands
     a8 = oracle.apply_per_channel_scale(prob["act"], prob["pre_quant_scale"], out_dtype, "fp8")
-    prob["_col_floor"] = oracle.column_magnitude(a8, oracle.dequantize(prob["q"], prob["scales"], zeros, 128, "fp8"),
+    prob["_col_floor"] = oracle.column_magnitude(a8, oracle.dequantize(prob["q"], prob["scales"], zeros, group, "fp8"),
                                                  prob["alpha"])
     return out.float().cpu().numpy(), ref
 
@@ -257,3 +257,63 @@ def test_w4a8_streaming_two_row_tiles_one_hot_rows(pkg, oracle, dev):
         out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=STREAM)
         w8 = oracle.dequantize(q, s, z, 128, "fp8")
         assert (out == oracle.round_f16(w8[rows])).all()
+
+
+# the reference's own grid for e4m3 activations with group sizes above 128
+# (tests/quantization/test_weight_only_groupwise_quant_matmul.py:429-455: m, n, k, dtype, pre-quant scale,
+# zeros, bias, group size - a group may be longer than K, or leave a shorter last group)
+_FLEX_GRID = [(32, 1024, 128, "fp16", True, True, 128), (32, 1024, 128, "fp16", True, True, 256),
+              (32, 1024, 256, "fp16", True, False, 384), (32, 1024, 256, "bf16", True, True, 384),
+              (32, 2048, 1024, "fp16", False, True, 512), (64, 2048, 2048, "bf16", False, False, 640),
+              (64, 2048, 2048, "fp16", False, False, 640),
+              # beyond the reference's grid: decode rows, long K with a shorter last group, staged scales
+              (1, 512, 8192, "bf16", True, True, 384), (7, 272, 8192 + 128, "fp16", True, False, 640),
+              (16, 4112, 4096, "bf16", False, True, 256), (300, 528, 2304, "bf16", True, True, 512)]
+
+
+@pytest.mark.parametrize("m,n,k,dtype,has_zero,has_bias,group", _FLEX_GRID)
+def test_w4a8_flexible_group_sizes(pkg, oracle, dev, m, n, k, dtype, has_zero, has_bias, group):
+    """Group sizes that are multiples of 128 (what the reference's Hopper launcher accepts for e4m3
+    activations, launchers/fpA_intB_launcher_sm90.inl:190-198) in both regimes and as AUTO picks, 16-bit
+    activations with the smoothing vector as in the reference's test: the tables hold ceil(k / group) rows."""
+    rng = np.random.default_rng(m * 7 + n + k + group)
+    rows = -(-k // group)
+    q = rng.integers(-8, 8, size=(k, n)).astype(np.int8)
+    s = oracle.round_f16(np.exp(rng.uniform(-3, 0, (rows, n))).astype(np.float32))
+    zeros = oracle.round_f16((rng.standard_normal((rows, n)) * 2).astype(np.float32)) if has_zero else None
+    bias = oracle.round_to(rng.standard_normal(n).astype(np.float32), dtype) if has_bias else None
+    prob = dict(q=q, scales=s, alpha=0.37,
+                act=oracle.round_to(rng.standard_normal((m, k)).astype(np.float32), dtype),
+                pre_quant_scale=oracle.round_to(rng.uniform(0.5, 2.0, k).astype(np.float32), dtype))
+    regimes = [0, GEMM] + ([STREAM] if m <= 32 else [])
+    outs = {}
+    for regime in regimes:
+        for direct in (False, True):
+            out, ref = _run(pkg, oracle, dev, prob, m, k, n, dtype, zeros=zeros, bias=bias, direct_fp8=direct,
+                            regime=regime, group=group)
+            assert _perr(oracle, out, ref, prob) < TOL, (regime, direct, _launch(pkg))
+            outs[regime, direct] = out
+        # the smoothing pass in front of the kernel and fp8 activations handed over directly: the same bits
+        assert (outs[regime, False] == outs[regime, True]).all()
+
+
+def test_w4a8_flexible_groups_one_hot_rows(pkg, oracle, dev):
+    """One-hot rows return the e4m3-rounded dequantized weight rows bit for bit with groups of 384 (rows of
+    different groups inside one 128-row tile row never occur, rows of one group span three): every
+    tile row reads its group's table row, in both kernels."""
+    M, K, N, G = 32, 1280, 272, 384
+    rng = np.random.default_rng(12)
+    q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+    rows_g = -(-K // G)
+    s = oracle.round_f16(np.exp(rng.uniform(-2, 3, (rows_g, N))).astype(np.float32))
+    zeros = oracle.round_f16((rng.standard_normal((rows_g, N)) * 20).astype(np.float32))
+    rows = np.concatenate([[0, 127, 128, 383, 384, 767, 768, 1151, 1152, 1279],
+                           rng.choice(K, size=M - 10, replace=False)])
+    act = np.zeros((M, K), np.float32)
+    act[np.arange(M), rows] = 1.0
+    prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+    for regime in (STREAM, GEMM):
+        for z in (None, zeros):
+            out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=regime, group=G)
+            w8 = oracle.dequantize(q, s, z, G, "fp8")
+            assert (out == oracle.round_f16(w8[rows])).all(), (regime, z is not None)

@@ -20,6 +20,12 @@ def test_library_exports_every_declared_symbol(pkg):
     for name in sorted(declared):
         assert hasattr(lib, name), "libwoq.so does not export %s" % name
     assert declared == set(pkg._lib.EXPORTED), "python binding and header disagree"
+    # the measurement probes live in an internal header: in the library, not in the boundary
+    probes = open(os.path.join(ROOT, "tensorrt-llm_amd", "csrc", "woq_probes.h")).read()
+    probes = set(re.findall(r"\b(woq_[a-z0-9_]+)\s*\(", re.sub(r"/\*.*?\*/", "", probes, flags=re.S)))
+    assert probes == set(pkg._lib.PROBES) and not (probes & declared)
+    for name in sorted(probes):
+        assert hasattr(lib, name), "libwoq.so does not export %s" % name
     assert lib.woq_abi_version() == 1 and lib.woq_layout_version() == 1
 
 

@@ -82,3 +82,46 @@ def test_static_scratch_rejects_what_does_not_fit(pkg, dev):
                         out_dtype=L.BF16, regime=L.REGIME_GEMM, workspace=None, workspace_bytes=0)
     assert lib.woq_matmul_static(ctypes.byref(args), None) == -4  # WOQ_ERR_WORKSPACE
     assert b"static scratch" in lib.woq_last_error()
+
+
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph(pkg, oracle, dev):
+    """After woq_static_init() and one call outside capture, a static call with `out=` given leaves the
+    device's free memory where it was, and the same call captured into a HIP graph replays to the eager
+    bits every time (eager work of the library between the replays; the input changes between them)."""
+    assert pkg._lib.lib.woq_static_init() == 0
+    assert pkg._lib.lib.woq_static_init() == 0  # idempotent
+    o = _operands(pkg, oracle, dev, 96, 4096, 512, 4, 128, "bf16", 5, True)
+    other = _operands(pkg, oracle, dev, 40, 2048, 256, 4, 128, "bf16", 6, True)
+    F = pkg.functional
+    out = torch.empty((96, o["n"]), dtype=o["dtype"], device=dev)
+
+    def static_call():
+        F.woq_matmul_raw(o["act"], o["pqs"], o["w"], o["scales"], o["zeros"], o["bias"], n=o["n"], k=o["k"],
+                         group_size=o["group"], quant_algo=o["algo"], out_dtype=o["dtype"], regime=GEMM, out=out,
+                         static_scratch=True)
+
+    static_call()  # first use of this kernel variant: outside capture
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    for _ in range(3):
+        static_call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            static_call()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    acts = [o["act"].clone(), (o["act"] * 0.5).contiguous(), o["act"].flip(0).contiguous()]
+    for a in acts:
+        o["act"].copy_(a)
+        want = _call(pkg, o, False, GEMM)
+        _call(pkg, other, True, GEMM)  # eager work on the same scratch between the replays
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
