@@ -192,7 +192,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
     // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
     // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
-    int const act_rows = ALDS ? (p.m < 16 ? p.m : 16) : 0;
+    int const act_rows = ALDS ? (SLOTS == 16 ? 1 : (p.m < 16 ? p.m : 16)) : 0;
     int const sc_rows = SCLDS ? (int) scale_row<GROUP>((uint32_t) (KT * TK - 1), p.group_magic) + 1 : 0;
     constexpr uint32_t SC_ROW = NS * 32u;
     char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
@@ -492,7 +492,8 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         int const act_chunks = act_rows * chunks_per_row;
         auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
         {
-            int const row = act_rows == 1 ? 0 : idx / chunks_per_row;
+            // (group slots for a single row: the row is known at compile time, no division in the prologue)
+            int const row = (SLOTS == 16 || act_rows == 1) ? 0 : idx / chunks_per_row;
             ch = (uint32_t) (idx - row * chunks_per_row);
             lds_at = (uint32_t) row * lds_row + ch * 16u;
             sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;

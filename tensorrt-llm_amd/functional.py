@@ -54,8 +54,22 @@ def woq_matmul_raw(act, pre_quant_scale, weight, scales, zeros, bias, *, n: int,
     if act.shape[-1] != k:
         raise RuntimeError("activation has %d input features, weight expects %d" % (act.shape[-1], k))
     m = act.numel() // k if k else 0
+    # the C ABI receives untyped pointers: a tensor of another element type would be read as the expected
+    # one without any error.  16-bit activations and the smoothing vector are of the output type; scales
+    # and zeros too, except for W4A8, whose kernels read float16 values whatever the output type (the
+    # reference stores those bits under the activation type's name: a 2-byte tensor of either type passes)
+    w4a8 = bool(quant_algo & FP8_ALPHA)
+    if act.dtype != torch.float8_e4m3fn and act.dtype != out_dtype:
+        raise RuntimeError("activation dtype %s does not match the output dtype %s" % (act.dtype, out_dtype))
+    scale_types = (torch.float16, out_dtype) if w4a8 else (out_dtype,)
+    for name, t, allowed in (("pre_quant_scale", pre_quant_scale, (out_dtype,)), ("scales", scales, scale_types),
+                             ("zeros", zeros, scale_types), ("bias", bias, (out_dtype,))):
+        if t is not None and t.dtype not in allowed:
+            raise RuntimeError("%s has dtype %s, the op expects %s" % (name, t.dtype, " or ".join(map(str, allowed))))
     if out is None:
         out = torch.empty(act.shape[:-1] + (n,), dtype=out_dtype, device=act.device)
+    elif out.dtype != out_dtype:
+        raise RuntimeError("out has dtype %s, expected %s" % (out.dtype, out_dtype))
     need = 0 if static_scratch else lib.woq_workspace_bytes(m, n, k, quant_algo, _WOQ_DT[act.dtype])
     if need and workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=act.device)

@@ -221,3 +221,36 @@ def test_rmsnorm_prequant_validation(pkg):
     assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 4, 64, L.FP8_E4M3, L.BF16, None) == -1
     assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 4, 64, L.BF16, L.FP16, None) == -1
     assert f(0x3000, 0x1000, 0x2000, None, None, 1e-5, 0, 64, L.BF16, L.FP8_E4M3, None) == 0  # m == 0: nothing to do
+
+
+@pytest.mark.gpu
+def test_python_wrapper_refuses_operands_of_another_dtype(pkg, dev):
+    """The C ABI takes untyped pointers, so the wrapper checks element types: a float32 smoothing vector
+    (what an unguarded W4A8 fold returns), bf16 scales next to fp16 activations or a float32 bias would
+    otherwise be read as 16-bit values without any error."""
+    import torch
+    F = pkg.functional
+    K, N = 256, 64
+    a = torch.zeros(2, K, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(K, N // 2, dtype=torch.int8, device=dev)
+    s = torch.ones(K // 128, N, dtype=torch.bfloat16, device=dev)
+    kw = dict(n=N, k=K, group_size=128)
+    F.woq_matmul_raw(a, None, w, s, None, None, quant_algo=0, **kw)
+    with pytest.raises(RuntimeError, match="scales has dtype"):
+        F.woq_matmul_raw(a, None, w, s.to(torch.float16), None, None, quant_algo=0, **kw)
+    with pytest.raises(RuntimeError, match="pre_quant_scale has dtype"):
+        F.woq_matmul_raw(a, torch.ones(K, device=dev), w, s, None, None, quant_algo=F.PRE_QUANT_SCALE, **kw)
+    with pytest.raises(RuntimeError, match="bias has dtype"):
+        F.woq_matmul_raw(a, None, w, s, None, torch.ones(N, device=dev), quant_algo=F.BIAS, **kw)
+    with pytest.raises(RuntimeError, match="zeros has dtype"):
+        F.woq_matmul_raw(a, None, w, s, s.float(), None, quant_algo=F.ZERO, **kw)
+    with pytest.raises(RuntimeError, match="activation dtype"):
+        F.woq_matmul_raw(a.to(torch.float16), None, w, s, None, None, quant_algo=0, out_dtype=torch.bfloat16, **kw)
+    # W4A8: float16 scales whatever the output type, or the same bits under the output type's name
+    a8 = torch.zeros(2, K, dtype=torch.float8_e4m3fn, device=dev)
+    h = torch.ones(K // 128, N, dtype=torch.float16, device=dev)
+    for sc in (h, h.view(torch.bfloat16)):
+        F.woq_matmul_raw(a8, None, w, sc, None, None, quant_algo=F.FP8_ALPHA, out_dtype=torch.bfloat16, **kw)
+    with pytest.raises(RuntimeError, match="scales has dtype"):
+        F.woq_matmul_raw(a8, None, w, h.float(), None, None, quant_algo=F.FP8_ALPHA, out_dtype=torch.bfloat16, **kw)
+    torch.cuda.synchronize()

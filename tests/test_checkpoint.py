@@ -283,9 +283,10 @@ def test_postprocess_weight_only_tp_split_padding_and_bias(pkg, oracle):
         want_bias[:cols.stop - cols.start] = bias[cols]
         assert torch.equal(out["bias"], want_bias)
     # row-parallel, unpadded: equal parts of K, bias passed through
-    out = C.postprocess_weight_only(w[:, :64].contiguous(), torch.quint4x2, bias=bias, tp_split=(0, 2, 1))
-    q, scale = oracle.symmetric_quantize(wt[32:64].copy(), 4, "bf16")
-    assert (_decode(pkg, out["weight"], 32, 4)[:32] == q).all() and torch.equal(out["bias"], bias)
+    out = C.postprocess_weight_only(w[:96, :64].contiguous(), torch.quint4x2, bias=bias[:96], tp_split=(0, 2, 1))
+    q, scale = oracle.symmetric_quantize(wt[32:64, :96].copy(), 4, "bf16")
+    assert (_decode(pkg, out["weight"], 32, 4)[:32] == q).all() and torch.equal(out["bias"], bias[:96])
+    assert (out["per_channel_scale"].float().numpy() == scale).all()
     with pytest.raises(ValueError):
         C.postprocess_weight_only(w.to(torch.int8), torch.int8)
     # a batch of experts [E, out, in] keeps its leading dimension

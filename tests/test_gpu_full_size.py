@@ -228,3 +228,69 @@ def test_full_size_regimes_agree(pkg, dev):
     act = activations(dev, L, 16, "regimes")
     a, b = run(pkg, L, act, 1).float(), run(pkg, L, act, 2).float()
     assert ((a - b).abs().max() / a.abs().max()).item() < TOL
+
+
+def test_full_size_config1_literally(pkg, dev):
+    """Benchmark configuration 1 as written: M = 1, K = N = 4096, fp16 activations ~ N(0, 1), weights float32
+    ~ N(0, 0.02) quantized symmetrically to int8 with one fp16 scale per output column, absmax / 127."""
+    k = n = 4096
+    g = torch.Generator(device=dev).manual_seed(_seed("c1", k, n))
+    w = torch.randn((k, n), generator=g, device=dev) * 0.02
+    scale = (w.abs().amax(0) / 127.0).to(torch.float16)
+    q = torch.round(w / scale.float()).clamp(-127, 127).to(torch.int8)
+    act = torch.randn((1, k), generator=g, device=dev).to(torch.float16)
+    F = pkg.functional
+    wq = pkg.ops.preprocess_weights_for_mixed_gemm(q.cpu().contiguous(), torch.int8, torch.float16).to(dev)
+    out = F.weight_only_quant_matmul(act, wq, scale, F.INT8, "float16")
+    torch.cuda.synchronize()
+    assert "stream" in (pkg._lib.lib.woq_last_launch() or b"").decode()
+    deq = (q.double() * scale.double()[None, :]).to(torch.float16)  # one rounding of the exact product
+    ref = act.float() @ deq.float()
+    err = (out.float() - ref).abs()
+    assert (err.max() / ref.abs().max()).item() < TOL
+    floor = ((act.float() ** 2) @ (deq.float() ** 2)).sqrt()
+    assert (err / torch.maximum(ref.abs(), floor)).max().item() < TOL
+
+
+@pytest.mark.parametrize("name", ["70b_down", "70b_gate_up"])
+@pytest.mark.parametrize("m", [1, 256, 4096])
+def test_full_size_w4a8_smoothing_leg(pkg, dev, name, m):
+    """Configuration 5 with its smoothing vector: bf16 activations ~ N(0, 1) and a per-input-channel vector
+    ~ U(0.5, 2) (per-tensor scaled into the e4m3 range) go through PRE_QUANT_SCALE | FP8_ALPHA - the smoothing
+    pass writes m * k bytes of e4m3 activations to the front of the workspace, the fp8 kernels (and their
+    split-K slabs) work behind it.  Reference on the GPU: (bf16(act * pqs) -> e4m3).float() @ deq.float() *
+    alpha.  Handing the same e4m3 activations over directly gives the same bits; so does woq_matmul_static
+    where its scratch is large enough, which otherwise says so and launches nothing."""
+    L = layer(pkg, dev, name, "w4a8")
+    F = pkg.functional
+    k, n = L["k"], L["n"]
+    g = torch.Generator(device=dev).manual_seed(_seed("c5-smooth", name, m))
+    act = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
+    pqs = torch.rand((k,), generator=g, device=dev) * 1.5 + 0.5
+    pqs = (pqs * (440.0 / (act.float() * pqs).abs().max())).to(torch.bfloat16)
+    smoothed = (act.float() * pqs.float()).to(torch.bfloat16)  # the product of two bf16 values, rounded once
+    assert smoothed.float().abs().max().item() < 464.0          # below the first value that e4m3 cannot hold
+    a8 = smoothed.float().to(torch.float8_e4m3fn)
+    algo = L["algo"] | F.PRE_QUANT_SCALE
+    args = dict(n=n, k=k, group_size=128, quant_algo=algo, alpha=L["alpha"], out_dtype=torch.bfloat16)
+    out = F.woq_matmul_raw(act, pqs, L["weight"], L["scales"], None, None, **args)
+    torch.cuda.synchronize()
+    direct = run(pkg, L, a8)
+    assert torch.equal(out, direct)
+    ref = (a8.float() @ L["deq"].float()) * L["alpha"]
+    err = (out.float() - ref).abs()
+    assert (err.max() / ref.abs().max()).item() < TOL
+    floor = ((a8.float() ** 2) @ (L["deq"].float() ** 2)).mean(dim=0).sqrt() * abs(L["alpha"])
+    assert (err.max(dim=0).values / torch.maximum(ref.abs().max(dim=0).values, floor)).max().item() < TOL
+    # the entry point that allocates nothing: same bits, or a clear refusal when m * k bytes (plus the
+    # split-K slabs) exceed its scratch
+    lib = pkg._lib.lib
+    need = lib.woq_workspace_bytes(m, n, k, algo, pkg._lib.BF16)
+    fits = m * k <= lib.woq_static_scratch_bytes()
+    if fits and need <= lib.woq_static_scratch_bytes():
+        got = F.woq_matmul_raw(act, pqs, L["weight"], L["scales"], None, None, static_scratch=True, **args)
+        torch.cuda.synchronize()
+        assert torch.equal(got, out)
+    elif not fits:
+        with pytest.raises(RuntimeError, match="static scratch"):
+            F.woq_matmul_raw(act, pqs, L["weight"], L["scales"], None, None, static_scratch=True, **args)

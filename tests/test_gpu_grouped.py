@@ -17,7 +17,7 @@ def grouped_problem(oracle, rows, K, N, bits, group, dtype, zero, bias, seed):
     E, total = len(rows), int(sum(rows))
     lo = -(1 << (bits - 1))
     q = rng.integers(lo, -lo, size=(E, K, N)).astype(np.int8)
-    gshape = (E, K // group, N) if group else (E, N)
+    gshape = (E, -(-K // group), N) if group else (E, N)  # a group size above 128 may leave a shorter last group
     p = dict(rows=rows, q=q, bits=bits, group=group, dtype=dtype, K=K, N=N,
              scales=oracle.round_to(rng.uniform(0.002, 0.02, gshape).astype(np.float32) * (16.0 / (1 << bits)), dtype),
              zeros=oracle.round_to((rng.standard_normal(gshape) * 0.02).astype(np.float32), dtype) if zero else None,
@@ -167,3 +167,20 @@ def test_grouped_rejections(pkg, oracle, dev):
         F.woq_grouped_matmul_raw(act.reshape(2, 2, 256), w, sc, None, None,
                                  torch.tensor([2, 4], dtype=torch.int64, device=dev), n=64, k=256, group_size=128,
                                  quant_algo=0)
+
+
+@pytest.mark.parametrize("group,K", [(192, 1024), (256, 1024), (320, 768)])
+@pytest.mark.parametrize("zero", [False, True])
+@pytest.mark.parametrize("rows,regime", [([3, 0, 16, 1], STREAM), ([20, 3, 0, 50, 33], GEMM), ([300, 0, 270], GEMM)])
+def test_grouped_flexible_group_sizes(pkg, oracle, dev, woq_env, group, K, zero, rows, regime):
+    """Group sizes that are multiples of 64 above 128 through the grouped entry: every expert's table has
+    ceil(k / group) rows (1024 / 192 and 768 / 320 leave a shorter last group), so the per-expert scale and
+    zero offsets follow that row count.  Streaming passes, the deferred-scale and the exact-dequantize tiled
+    kernels."""
+    p = grouped_problem(oracle, rows, K, 272, 4, group, "bf16", zero, True, seed=group + sum(rows))
+    ref = reference(oracle, p)
+    for kernel in (("exact", "skinny") if regime == GEMM and sum(rows) < 200 else (None,)):
+        woq_env(WOQ_GEMM_KERNEL=kernel)
+        out = run_grouped(pkg, oracle, dev, p, regime=regime)
+        assert np.isfinite(out).all()
+        assert oracle.max_rel_err(out, ref) < TOL, kernel
