@@ -27,7 +27,10 @@ COMMON = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-command-line-argum
           "-ffp-contract=off"]
 # Per-file additions.  The skinny-M kernel reads its MFMA results with VALU instructions every
 # group: keep those accumulators in the architectural VGPRs instead of copying them out of AGPRs.
-PER_FILE = {"skinny_": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+# The single-row decode kernel takes what its first requests need as scalar arguments and has them preloaded
+# into SGPRs at wavefront start (no scalar loads from the argument buffer in front of the first address).
+PER_FILE = {"skinny_": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+            "stream_row": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
 
 
 def sources():

@@ -224,6 +224,37 @@ bool pick_wide_shape(int m, int n, int k, int group, int bits, WideShape& out)
     return false;
 }
 
+// The single-row streaming kernel (one workgroup per strip, short-lived wavefronts) for this problem, and
+// its launch shape: wavefronts per workgroup and tiles (1 KiB, 128 rows of K) per wavefront and pass.
+// WOQ_ROW_SHAPE="waves,tiles" forces it, "0" switches it off.
+bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& tiles)
+{
+    (void) n;
+    if (m != 1 || bits != 4 || (group != 64 && group != 128))
+        return false;
+    if (Tactic const* t = current_tactic())
+        if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)
+            return false; // a tuned launch shape of the strip-group kernel
+    EnvOverrides const& env = env_overrides();
+    if (env.row_mode == 0 || env.has_stream_shape || env.wide_mode == 1)
+        return false;
+    if (env.row_mode == 1)
+    {
+        waves = env.row_shape[0], tiles = env.row_shape[1];
+        return true;
+    }
+    // Measured on MI355X (one row, int4 with group scales and zeros, against the strip-group and wide
+    // kernels): 4096 x 6144 5.69 -> 4.74 us, 4096 x 4096 4.64 -> 3.91, 4096 x 28672 13.74 -> 12.85,
+    // 14336 x 4096 8.43 -> 8.28, 8192 x 10240 11.15 -> 10.97, 8192 x 8192 9.34 -> 8.93, 8192 x 57344
+    // 45.79 -> 44.34, 28672 x 8192 26.90 -> 24.61.  Launch shape: one pass over K where a workgroup of
+    // at most sixteen wavefronts x eight tiles reaches that far (few wavefronts with eight tiles each up to
+    // K = 4096, eight up to 8192, sixteen up to 16384), else passes of four wavefronts x eight tiles.
+    int const k_tiles = (k + 127) / 128;
+    tiles = 8;
+    waves = k_tiles <= 32 ? 4 : (k_tiles <= 64 ? 8 : (k_tiles <= 128 ? 16 : 4));
+    return true;
+}
+
 // bytes of float32 slabs a streaming launch of m rows splitting K into `slices` needs
 static size_t stream_slab_bytes(int m, int n, int slices)
 {
@@ -314,6 +345,8 @@ EnvOverrides read_env()
             == 4;
     if (char const* e = std::getenv("WOQ_WIDE_SHAPE"))
         o.wide_mode = std::sscanf(e, "%d,%d,%d", &o.wide_shape[0], &o.wide_shape[1], &o.wide_shape[2]) == 3 ? 1 : 0;
+    if (char const* e = std::getenv("WOQ_ROW_SHAPE"))
+        o.row_mode = std::sscanf(e, "%d,%d", &o.row_shape[0], &o.row_shape[1]) == 2 ? 1 : 0;
     if (char const* e = std::getenv("WOQ_STREAM_SLOTS"))
         o.slots_off = e[0] == '0';
     if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))

@@ -192,7 +192,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
     char const* a_lds = reinterpret_cast<char const*>(act_lds) + (uint32_t) a_row * lds_row + (uint32_t) kg * 16u;
     // staged scales: one row of NS*16 values per group of K (rows past the end of K hold zeros),
     // strip slot s at columns s*16 ..; the zeros follow in the same arrangement
-    int const act_rows = ALDS ? (SLOTS == 16 ? 1 : (p.m < 16 ? p.m : 16)) : 0;
+    int const act_rows = ALDS ? (p.m < 16 ? p.m : 16) : 0;
     int const sc_rows = SCLDS ? (int) scale_row<GROUP>((uint32_t) (KT * TK - 1), p.group_magic) + 1 : 0;
     constexpr uint32_t SC_ROW = NS * 32u;
     char* const sc_lds = reinterpret_cast<char*>(act_lds) + (uint32_t) act_rows * lds_row;
@@ -492,8 +492,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         int const act_chunks = act_rows * chunks_per_row;
         auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
         {
-            // (group slots for a single row: the row is known at compile time, no division in the prologue)
-            int const row = (SLOTS == 16 || act_rows == 1) ? 0 : idx / chunks_per_row;
+            int const row = act_rows == 1 ? 0 : idx / chunks_per_row;
             ch = (uint32_t) (idx - row * chunks_per_row);
             lds_at = (uint32_t) row * lds_row + ch * 16u;
             sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;
@@ -1055,6 +1054,10 @@ int launch_stream_grouped(StreamParams const& sp, hipStream_t s)
 template <int DT, int BITS>
 bool try_launch_stream_wide(MatmulProblem const& p, StreamParams const& sp, hipStream_t s, int& rc);
 
+// the single-row kernel (stream_row.hip) and the rule that picks it and its launch shape (api.cpp)
+int launch_stream_row(StreamParams const& sp, int dtype, int group, bool pqs, bool zero, int waves, int tpw, void* stream);
+bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& tiles);
+
 template <int DT, int BITS>
 int launch_stream_typed(MatmulProblem const& p, void* stream)
 {
@@ -1090,6 +1093,16 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
     int const mt = p.m <= 16 ? 1 : (p.m <= 32 ? 2 : (p.m <= 64 ? 4 : 8));
     bool const pqs = p.pre_quant_scale != nullptr;
     bool const zero = p.zeros != nullptr;
+    if (mt == 1 && !p.num_experts)
+    {
+        int waves = 0, tiles = 0;
+        if (pick_row_shape(p.m, p.n, p.k, p.group_size, BITS, waves, tiles))
+        {
+            int const rc = launch_stream_row(sp, DT, p.group_size, pqs, zero, waves, tiles, stream);
+            if (rc != WOQ_ERR_UNSUPPORTED)
+                return rc;
+        }
+    }
     if (mt == 1)
     {
         // wide matrices at decode: the kernel whose wavefronts own whole columns, where the rule picks it

@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_wide_kernel(StreamParams p)
 
     // LDS: rows of (smoothed) activations, the row sums of every group (16 floats per group), zeros,
     // then WAVES scale windows
-    int const rows = R == 1 ? 1 : p.m;
+    int const rows = p.m;
     uint32_t const lds_row = (uint32_t) KT * TK * 2u + 16u;
     char* const lds = reinterpret_cast<char*>(wide_lds);
     char* const sum_lds = lds + (uint32_t) rows * lds_row;
@@ -131,7 +131,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_wide_kernel(StreamParams p)
     int const act_chunks = rows * chunks_per_row;
     auto act_offset = [&](int idx, uint32_t& lds_at, uint32_t& ch, uint32_t& sum_at)
     {
-        int const row = R == 1 ? 0 : idx / chunks_per_row; // (one row: no division in the prologue)
+        int const row = rows == 1 ? 0 : idx / chunks_per_row;
         ch = (uint32_t) (idx - row * chunks_per_row);
         lds_at = (uint32_t) row * lds_row + ch * 16u;
         sum_at = ch / (SEG / 8) * 64u + (uint32_t) row * 4u;
@@ -366,11 +366,6 @@ int launch_stream_wide_shaped(StreamParams const& sp, WideShape sh, hipStream_t 
         return launch_stream_wide_variant<DT, BITS, GROUP, PQS, ZERO, NS_, WAVES_, PF_, 16>(sp, s);
     WOQ_WIDE(2, 4, 4)
     WOQ_WIDE(1, 4, 4)
-    WOQ_WIDE(1, 7, 4)
-    WOQ_WIDE(1, 7, 6)
-    WOQ_WIDE(1, 7, 8)
-    WOQ_WIDE(2, 7, 4)
-    WOQ_WIDE(2, 7, 2)
 #undef WOQ_WIDE
     return fail(WOQ_ERR_UNSUPPORTED, "wide stream shape ns=%d waves=%d pf=%d is not instantiated", sh.ns, sh.waves,
         sh.pf);

@@ -148,8 +148,10 @@ def test_stream_every_launch_shape(pkg, oracle, dev, woq_env, shape, M):
 
 
 @pytest.mark.parametrize("N", [6144, 16384])
-def test_stream_wide_n_default_heuristic(pkg, oracle, dev, N):
-    """Wide outputs take the multi-strip launch shapes of the heuristic."""
+def test_stream_wide_n_default_heuristic(pkg, oracle, dev, woq_env, N):
+    """Wide outputs take the multi-strip launch shapes of the heuristic (strip-group kernel: the single-row
+    kernel is switched off)."""
+    woq_env(WOQ_ROW_SHAPE="0")
     p = random_problem(oracle, 1, 512, N, 4, 128, "bf16", zero=True, seed=N)
     err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
     assert err < TOL, err
@@ -226,24 +228,78 @@ def test_wide_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, bits, group
         assert err < TOL, (shape, zero, bias, pqs, err)
 
 
-def test_wide_decode_kernel_is_what_wide_single_row_problems_run_on(pkg, oracle, dev, woq_env):
-    """One row, K <= 4096, at least 1536 column strips: the built-in rule takes the wide kernel (switching it
-    off changes the float32 summation order, hence some output bits, while both stay within the bar), and
-    a one-hot activation returns the dequantized weight row through it."""
+def test_wide_decode_kernel_is_what_wide_single_row_int8_problems_run_on(pkg, oracle, dev, woq_env):
+    """One row, int8 weights with group scales, K <= 4096, at least 1536 column strips: the built-in rule takes
+    the wide kernel (switching it off changes the float32 summation order, hence some output bits, while both
+    stay within the bar), and a one-hot activation returns the dequantized weight row through it.  (int4
+    weights with group scales of 64 / 128 run on the single-row kernel.)"""
     K, N = 512, 24576 + 48
-    p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=77)
+    p = random_problem(oracle, 1, K, N, 8, 64, "bf16", zero=True, seed=77)
     auto = run_product(pkg, oracle, dev, p, 0)
+    assert "stream wide" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, auto, p) < TOL
     woq_env(WOQ_WIDE_SHAPE="0")
     other = run_product(pkg, oracle, dev, p, 0)
+    assert "stream mt=1" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, other, p) < TOL
     assert (auto != other).any()
     woq_env(WOQ_WIDE_SHAPE=None)
     p["act"] = np.zeros((1, K), np.float32)
     p["act"][0, 300] = 1.0
     out = run_product(pkg, oracle, dev, p, 0)
-    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")[300]
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 64, "bf16")[300]
     assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()
+
+
+@pytest.mark.parametrize("shape", ["8,4", "16,4", "8,8", "16,8", "4,8"])
+@pytest.mark.parametrize("group,dtype,K,N", [(128, "bf16", 2176, 272), (64, "fp16", 1408, 1040), (128, "fp16", 128, 16),
+                                             (64, "bf16", 4160, 528), (128, "bf16", 14336, 48)])
+def test_row_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, K, N):
+    """The single-row kernel (one workgroup per strip, every wavefront a few consecutive tiles, no staging
+    pass), forced through WOQ_ROW_SHAPE: K that needs several passes of the workgroup or leaves wavefronts
+    without tiles, a last tile that is only half inside K, groups that end inside a wavefront's quad of rows;
+    every optional input."""
+    woq_env(WOQ_ROW_SHAPE=shape)
+    for zero, bias, pqs in [(True, True, True), (False, False, False), (True, False, False), (False, True, True)]:
+        p = random_problem(oracle, 1, K, N, 4, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N)
+        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+        assert "stream row" in _last_launch(pkg), _last_launch(pkg)
+        assert err < TOL, (shape, zero, bias, pqs, err)
+
+
+def test_row_decode_kernel_is_what_single_row_int4_problems_run_on(pkg, oracle, dev, woq_env):
+    """One row, int4 with group scales of 64 or 128: the built-in rule takes the single-row kernel, with one
+    pass over K where sixteen wavefronts x eight tiles reach that far; int8 weights, more rows, per-channel
+    scales or larger groups do not.  Every one-hot activation returns the dequantized weight row through it;
+    switched off, the strip-group kernel meets the same bar."""
+    K, N = 4096, 272
+    p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=78)
+    auto = run_product(pkg, oracle, dev, p, 0)
+    assert "stream row waves=4 tpw=8 passes=1" in _last_launch(pkg), _last_launch(pkg)
+    assert parity_err(oracle, auto, p) < TOL
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")
+    for k_hot in (0, 127, 128, 2049, 4095):
+        p["act"] = np.zeros((1, K), np.float32)
+        p["act"][0, k_hot] = 1.0
+        out = run_product(pkg, oracle, dev, p, 0)
+        assert (np.abs(out[0] - w[k_hot]) <= np.abs(w[k_hot]) * 2.0 ** -7 + 2.5e-7).all(), k_hot
+    woq_env(WOQ_ROW_SHAPE="0")
+    p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=78)
+    other = run_product(pkg, oracle, dev, p, 0)
+    assert "stream mt=1" in _last_launch(pkg), _last_launch(pkg)
+    assert parity_err(oracle, other, p) < TOL
+    woq_env(WOQ_ROW_SHAPE=None)
+    for K2, group, want in ((8192, 64, "waves=8 tpw=8 passes=1"), (14336, 128, "waves=16 tpw=8 passes=1"),
+                            (28672, 128, "waves=4 tpw=8 passes=7"), (128, 64, "waves=4 tpw=8 passes=1")):
+        q = random_problem(oracle, 1, K2, 48, 4, group, "fp16", zero=True, bias=True, pqs=True, seed=K2)
+        assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL
+        assert "stream row " + want in _last_launch(pkg), (K2, _last_launch(pkg))
+    for kw in (dict(M=2), dict(bits=8, group=64), dict(group=0), dict(group=256)):
+        a = dict(M=1, K=K, N=N, bits=4, group=128)
+        a.update(kw)
+        q = random_problem(oracle, a["M"], a["K"], a["N"], a["bits"], a["group"], "bf16", seed=79)
+        assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL
+        assert "stream row" not in _last_launch(pkg), (kw, _last_launch(pkg))
 
 
 def _last_launch(pkg):
@@ -253,10 +309,12 @@ def _last_launch(pkg):
 @pytest.mark.parametrize("M,bits,group,dtype,K,N", [(1, 4, 128, "bf16", 512, 9216), (1, 4, 64, "fp16", 384, 12288 - 16),
                                                     (2, 4, 128, "bf16", 256, 8208), (4, 8, 64, "bf16", 256, 10240),
                                                     (1, 8, 0, "fp16", 320, 12288), (3, 4, 0, "bf16", 512, 9232)])
-def test_stream_three_strips_per_workgroup(pkg, oracle, dev, M, bits, group, dtype, K, N):
+def test_stream_three_strips_per_workgroup(pkg, oracle, dev, woq_env, M, bits, group, dtype, K, N):
     """513 ... 768 column strips and few rows: the built-in rule gives a workgroup three strips (a last
     workgroup with one or two, N that is not a multiple of 48); every optional input; one-hot rows return
-    the dequantized weight."""
+    the dequantized weight.  (The single-row kernel, which would take the one-row int4 cases, is switched
+    off: this is the strip-group kernel's test.)"""
+    woq_env(WOQ_ROW_SHAPE="0")
     for zero, bias, pqs in [(group != 0, True, True), (False, False, False)]:
         p = random_problem(oracle, M, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + M)
         out = run_product(pkg, oracle, dev, p, 0)
@@ -274,10 +332,11 @@ def test_stream_three_strips_per_workgroup(pkg, oracle, dev, M, bits, group, dty
 
 
 @pytest.mark.parametrize("M,K,group", [(1, 14336, 128), (3, 14336, 64), (1, 20480, 128), (2, 16384 + 64, 64)])
-def test_stream_staged_chunks_beyond_the_first_batch(pkg, oracle, dev, M, K, group):
+def test_stream_staged_chunks_beyond_the_first_batch(pkg, oracle, dev, woq_env, M, K, group):
     """Activations of more than two (and more than four) 16-byte chunks per thread and group tables of more
     than one: the chunks a thread keeps across the weight prefetch, the batched loop behind it, a ragged
-    last batch."""
+    last batch (strip-group kernel: the single-row kernel is switched off)."""
+    woq_env(WOQ_ROW_SHAPE="0")
     p = random_problem(oracle, M, K, 272, 4, group, "bf16", zero=True, bias=True, pqs=True, seed=K + M)
     out = run_product(pkg, oracle, dev, p, 0)
     assert "stream" in _last_launch(pkg), _last_launch(pkg)
