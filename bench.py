@@ -39,11 +39,12 @@ CACHE_BYTES = 256 << 20  # last-level (Infinity) cache; rotation must exceed it
 TRAFFIC_PROFILE = "profiles/stream_gemv_gate_up_m1_hbm_traffic.md"
 
 
-def recorded_traffic_bytes():
+def recorded_traffic_bytes(launched):
     """HBM bytes per launch of the dominant kernel as the tracked rocprofv3 --pmc summary records them
     (FETCH_SIZE / WRITE_SIZE runs calibrated with a 256 MiB copy; the line `traffic_bytes_per_launch: N`
     of TRAFFIC_PROFILE).  Counters cannot be read from inside this process; None when the summary is
-    missing or does not name the kernel this library now launches for the shape."""
+    missing or was taken on another kernel or launch shape than `launched`, which is what the library
+    reports (woq_last_launch) for the launch this run timed (the summary's line `launch: ...`)."""
     import os
     import re
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), TRAFFIC_PROFILE)
@@ -52,14 +53,15 @@ def recorded_traffic_bytes():
     except OSError:
         return None
     m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", text, re.M)
-    k = re.search(r"^kernel:\s*(\S+)", text, re.M)
-    if not m or not k or k.group(1) != DOMINANT_KERNEL:
+    k = re.search(r"^launch:\s*(.+?)\s*$", text, re.M)
+    if not m or not k or k.group(1) != launched:
         return None
     return int(m.group(1))
 
 
-# the kernel the library launches for gate_up at M = 1 (named in the rocprof summaries)
-DOMINANT_KERNEL = "stream_wide_kernel<1,4,128,false,true,2,4,4,16>"
+def last_launch(pkg):
+    """What the library launched for this thread's last matmul call (kernel family and launch shape)."""
+    return (pkg._lib.lib.woq_last_launch() or b"").decode()
 
 
 def algorithmic_bytes(m, k, n, bits=4, group=GROUP, n_sz=2, act_bytes=2):
@@ -191,6 +193,7 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
     reps = max(steps, 50)
     _, dom_s, dom_launches = time_graph(
         lambda: [launch(pkg, acts[gk], layers[gi][r % len(layers[gi])], outs[gi]) for r in range(reps)], reps)
+    dom_launch = last_launch(pkg)  # the kernel and launch shape the timed launches ran on
     dom_bytes = algorithmic_bytes(m, gk, gn)
     dom_dur = dom_s / dom_launches
     per_shape = {}
@@ -199,7 +202,7 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
             lambda: [launch(pkg, acts[k], layers[i][r % len(layers[i])], outs[i]) for r in range(reps)], reps)
         per_shape[name] = dict(us=round(s_s / s_l * 1e6, 3), gbs=round(algorithmic_bytes(m, k, n) / (s_s / s_l) / 1e9, 1))
     return dict(host_s=host_s, ev_s=ev_s, per_step_bytes=per_step_bytes, copies=copies, dom_dur=dom_dur,
-                dom_bytes=dom_bytes, per_shape=per_shape, layers=layers, acts=acts)
+                dom_bytes=dom_bytes, dom_launch=dom_launch, per_shape=per_shape, layers=layers, acts=acts)
 
 
 def bench_cpu_baseline(layers, acts, m=1, budget_s=15.0):
@@ -254,6 +257,7 @@ def bench_gemm(pkg, dev, m=4096, reps=40):
         torch.cuda.synchronize()
         # the launches replay from a HIP graph, once untimed first; the fastest of three timed replays
         _, sec, launches = time_graph(lambda: [launch(pkg, act, layer, out) for _ in range(reps)], reps, repeats=3)
+        launched = last_launch(pkg)
         sec /= launches
         tf = 2.0 * m * n * k / sec / 1e12
         # context, not a baseline: the vendor library's plain bf16 x bf16 GEMM (no dequantize) of the
@@ -269,7 +273,7 @@ def bench_gemm(pkg, dev, m=4096, reps=40):
                     # the M = 4096 half of the metric in the shape of `roofline`
                     roofline={"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_BF16_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                              "kernel": "gemm_kernel<bf16,int4,g128,zeros,RT=16,persistent> on gate_up K=%d N=%d M=%d" % (k, n, m),
+                              "kernel": "%s (bf16 x int4 g128 + zeros) on gate_up K=%d N=%d M=%d" % (launched, k, n, m),
                               "flop_per_launch": 2.0 * m * n * k, "us_per_launch": round(sec * 1e6, 1)})
     except Exception as e:  # the decode line is still valid without the prefill extra
         return dict(error=str(e)[:200])
@@ -376,6 +380,8 @@ def run_for_counters(pkg, dev, mode, reps=20):
         print(json.dumps({"mode": mode, "kernel": "GEMM regime on gate_up K=4096 N=28672 M=%d" % m,
                           "flop_per_launch": 2.0 * m * n * k, "launches": reps}))
         return
+    if mode == "dominant70b":  # the same GEMV on the Llama-3-70B gate_up
+        _, k, n = SHAPES_70B[2]
     copies = max(2, -(-3 * CACHE_BYTES // (k * n // 2)))
     layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
     act = torch.randn((1, k), device=dev).to(torch.bfloat16)
@@ -383,7 +389,7 @@ def run_for_counters(pkg, dev, mode, reps=20):
     for r in range(reps):
         launch(pkg, act, layers[r % copies], out)
     torch.cuda.synchronize()
-    print(json.dumps({"mode": "dominant", "kernel": DOMINANT_KERNEL + " on gate_up K=4096 N=28672 M=1",
+    print(json.dumps({"mode": mode, "kernel": last_launch(pkg) + " on gate_up K=%d N=%d M=1" % (k, n),
                       "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n), "launches": reps}))
 
 
@@ -561,7 +567,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
-    ap.add_argument("--mode", choices=["bench", "dominant", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
+    ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
@@ -602,9 +608,9 @@ def main():
                                "bf16 scales+zeros, decode GEMV M=1; %d rotating weight copies" % r["copies"],
                    "m": 1, "group_size": GROUP, "weight_bits": 4},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic_bytes(),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": recorded_traffic_bytes(r["dom_launch"]),
                      "traffic_source": TRAFFIC_PROFILE,
-                     "kernel": DOMINANT_KERNEL + " on gate_up K=4096 N=28672",
+                     "kernel": r["dom_launch"] + " (bf16 x int4 g128 + zeros) on gate_up K=4096 N=28672",
                      "bytes_per_launch": r["dom_bytes"], "us_per_launch": round(r["dom_dur"] * 1e6, 3)},
         "per_shape": r["per_shape"],
         "event_ms_per_step": round(r["ev_s"] / args.steps * 1e3, 5),

@@ -230,7 +230,7 @@ bool pick_wide_shape(int m, int n, int k, int group, int bits, WideShape& out)
 bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& tiles)
 {
     (void) n;
-    if (m != 1 || bits != 4 || (group != 64 && group != 128))
+    if (m < 1 || m > 4 || bits != 4 || (group != 64 && group != 128))
         return false;
     if (Tactic const* t = current_tactic())
         if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)
@@ -243,15 +243,39 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
         waves = env.row_shape[0], tiles = env.row_shape[1];
         return true;
     }
-    // Measured on MI355X (one row, int4 with group scales and zeros, against the strip-group and wide
-    // kernels): 4096 x 6144 5.69 -> 4.74 us, 4096 x 4096 4.64 -> 3.91, 4096 x 28672 13.74 -> 12.85,
+    // Measured on MI355X (int4 with group scales and zeros, against the strip-group and wide kernels).
+    // One row: 4096 x 6144 5.69 -> 4.74 us, 4096 x 4096 4.64 -> 3.91, 4096 x 28672 13.74 -> 12.85,
     // 14336 x 4096 8.43 -> 8.28, 8192 x 10240 11.15 -> 10.97, 8192 x 8192 9.34 -> 8.93, 8192 x 57344
     // 45.79 -> 44.34, 28672 x 8192 26.90 -> 24.61.  Launch shape: one pass over K where a workgroup of
     // at most sixteen wavefronts x eight tiles reaches that far (few wavefronts with eight tiles each up to
     // K = 4096, eight up to 8192, sixteen up to 16384), else passes of four wavefronts x eight tiles.
+    // Two rows (two rows of the M-tile per group, so at most eight groups per wavefront): 4096 x 6144
+    // 5.89 -> 5.17, 4096 x 4096 4.58 -> 4.31, 4096 x 28672 14.06 -> 13.49, 14336 x 4096 10.02 -> 8.51,
+    // 28672 x 8192 27.63 -> 24.67; nothing to gain at K = 8192.  Three and four rows (four groups per
+    // wavefront): the narrow matrices only - 4096 x 6144 6.33 -> 5.84, 4096 x 4096 5.25 -> 4.51, 14336 x 4096
+    // 12.14 -> 10.07; the wide ones and K >= 8192 with 512 strips or more are 5-15 % slower than on the
+    // strip-group kernel, which shares each activation fragment among more strips.
     int const k_tiles = (k + 127) / 128;
-    tiles = 8;
-    waves = k_tiles <= 32 ? 4 : (k_tiles <= 64 ? 8 : (k_tiles <= 128 ? 16 : 4));
+    int const strips = n / 16;
+    int const segs = 128 / group;
+    if (m == 1)
+    {
+        tiles = 8;
+        waves = k_tiles <= 32 ? 4 : (k_tiles <= 64 ? 8 : (k_tiles <= 128 ? 16 : 4));
+        return true;
+    }
+    if (m == 2)
+    {
+        if (k_tiles > 32 && k_tiles <= 64 && strips < 2048)
+            return false;
+        tiles = 4;
+        waves = k_tiles <= 128 ? 8 : 4;
+        return true;
+    }
+    if (strips > 512 || k_tiles > 128 || (k_tiles > 32 && k_tiles <= 64))
+        return false;
+    tiles = 4 / segs;
+    waves = segs == 1 ? 8 : 16;
     return true;
 }
 

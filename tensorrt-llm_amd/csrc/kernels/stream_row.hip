@@ -1,4 +1,4 @@
-// Single-row decode (M = 1, int4 weights, group scales): short-lived wavefronts in address order.
+// Decode of one to four rows (int4 weights, group scales): short-lived wavefronts in address order.
 //
 // Counterpart of the reference's small-M kernel at batch 1
 // (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernel.h:57-118) in purpose only.  What HBM rewards on
@@ -8,9 +8,10 @@
 // strip with all its loads issued at once, and there is no staging pass and no barrier before the
 // arithmetic - every wavefront fetches the few activations and scales it needs itself:
 //   * lane (kg, c) of the 16x16x32 matrix instruction supplies row c of the A operand.  Row c carries the
-//     activations of the wavefront's c-th group of K (c < ROWS = groups per wavefront, at most 16) and
-//     nothing else, so one instruction multiplies every group's activations with one group's weights;
-//     D_g = A x W_g is kept per group g and only its row g is used: no masking, no zero operands;
+//     activations of activation row c % R of the wavefront's (c / R)-th group of K (R = 1, 2 or 4 rows of
+//     the problem; groups per wavefront x R <= 16) and nothing else, so one instruction multiplies every
+//     group's activations with one group's weights; D_g = A x W_g is kept per group g and only its rows
+//     g * R .. g * R + R - 1 are used: no masking, no zero operands;
 //   * A x ones gives the activation sum S_g of every group in the same register layout;
 //   * register r of lane (kg, c) is row kg * 4 + r: that lane loads the scale and zero of groups
 //     kg * 4 + r for its column c (2-byte loads, 32 contiguous bytes per group and strip) and forms
@@ -43,6 +44,8 @@ struct RowTail
 {
     void const* pqs;
     void const* bias;
+    float alpha;
+    int m;
     unsigned long long* trace; // WOQ_TIMELINE builds only
 };
 
@@ -50,17 +53,20 @@ struct RowTail
 // the wavefront finds them in SGPRs when it starts (kernel-argument preloading; this file is compiled with
 // -amdgpu-kernarg-preload-count=16, of which the hardware's sixteen user SGPRs leave fourteen): a by-value
 // struct is fetched with scalar loads from the argument buffer instead, 0.2-0.3 us per dependent batch,
-// before the first address can be formed.
-template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int TPW, bool MULTI>
+// before the first address can be formed.  `act_bytes` = m * k * 2: rows of the M-tile past m start
+// outside the descriptor, read zeros and cost no traffic.
+template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int TPW, bool MULTI, int R>
 __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weight, void const* act, void const* scales,
-    void const* zeros, int k_tiles, int strips, int groups_per_xcd, int n, int k, float alpha, void* out, RowTail tail)
+    void const* zeros, int k_tiles, int strips, int groups_per_xcd, int n, int k, int act_bytes, void* out, RowTail tail)
 {
     using E = Elem<DT>;
     constexpr int TK = 128;
     constexpr int SEGS = TK / GROUP, SEG_SLABS = GROUP / 32;
-    constexpr int ROWS = TPW * SEGS; // groups of K per wavefront and pass = rows of the M-tile in use
+    constexpr int GROUPS = TPW * SEGS; // groups of K per wavefront and pass
+    constexpr int ROWS = GROUPS * R;   // rows of the M-tile in use
     static_assert(GROUP == 64 || GROUP == 128, "group scales of 64 or 128 rows");
-    static_assert(ROWS == 4 || ROWS == 8 || ROWS == 16, "whole quads of MFMA rows");
+    static_assert(R == 1 || R == 2 || R == 4, "one, two or four activation rows");
+    static_assert(ROWS <= 16, "the M-tile has 16 rows");
     constexpr float OFF = Offset<DT, 4>::value;
     constexpr uint32_t kOob = 0x80000000u;
 
@@ -79,7 +85,9 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
     uint32_t const wlane = ((uint32_t) strip * (uint32_t) KT * 64u + (uint32_t) lane) * 16u;
     int const c = lane & 15, kg = lane >> 4;
     int const groups_k = k / GROUP;
-    auto const act_rsrc = make_rsrc(act, (uint32_t) k * 2u);
+    auto const act_rsrc = make_rsrc(act, (uint32_t) act_bytes);
+    // this lane's activations: row c % R of the problem, group c / R of the pass
+    uint32_t const a_lane = (uint32_t) (c % R) * (uint32_t) k * 2u + (uint32_t) (kg * 8) * 2u;
 
     // One pass of the workgroup covers WAVES * TPW tiles of K; wavefront w takes the TPW consecutive tiles
     // w * TPW .. of it.  MULTI (K longer than one pass): the passes follow one another, each with all its
@@ -95,11 +103,11 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
     // multiplied as it arrives) and the weights: needed first, requested before anything else is worked out
     auto fetch_operands = [&](Stage& st, int kt0)
     {
-        int const g_mine = kt0 * SEGS + c; // the group whose activations this lane holds
+        int const g_mine = kt0 * SEGS + c / R; // the group whose activations this lane holds
         bool const a_ok = c < ROWS && g_mine < groups_k;
 #pragma unroll
         for (int js = 0; js < SEG_SLABS; ++js)
-            st.a[js] = buffer_load_x4(act_rsrc, a_ok ? (uint32_t) (g_mine * GROUP + js * 32 + kg * 8) * 2u : kOob);
+            st.a[js] = buffer_load_x4(act_rsrc, a_ok ? a_lane + (uint32_t) (g_mine * GROUP + js * 32) * 2u : kOob);
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
             st.w[i] = buffer_load_x4(w_rsrc, kt0 + i < KT ? wlane + (uint32_t) (kt0 + i) * 1024u : kOob);
@@ -118,25 +126,26 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
     u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
     NibbleConsts const nib = nibble_consts<DT>();
     f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
-    // what the end of a pass needs: the scale and zero of groups kg * 4 + r for this lane's column (and the
-    // smoothing factors of the lane's activations)
+    // what the end of a pass needs: register r of lane (kg, c) is row kg * 4 + r of the M-tile, i.e. group
+    // (kg * 4 + r) / R - the lane loads that group's scale and zero for its column c (and the smoothing
+    // factors of the lane's activations)
     auto fetch_scales = [&](Stage& st, int kt0)
     {
         int const g0 = kt0 * SEGS;
         if constexpr (PQS)
         {
-            int const g_mine = g0 + c;
+            int const g_mine = g0 + c / R;
             bool const a_ok = c < ROWS && g_mine < groups_k;
 #pragma unroll
             for (int js = 0; js < SEG_SLABS; ++js)
                 st.pq[js] = buffer_load_x4(pqs_rsrc, a_ok ? (uint32_t) (g_mine * GROUP + js * 32 + kg * 8) * 2u : kOob);
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+        for (int r = 0; r < 4; r += R)
         {
-            int const row = kg * 4 + r;
-            bool const ok = row < ROWS && g0 + row < groups_k;
-            uint32_t const off = ok ? (uint32_t) (g0 + row) * (uint32_t) n * 2u + sc_lane : kOob;
+            int const gl = (kg * 4 + r) / R;
+            bool const ok = gl < GROUPS && g0 + gl < groups_k;
+            uint32_t const off = ok ? (uint32_t) (g0 + gl) * (uint32_t) n * 2u + sc_lane : kOob;
             st.s[r] = buffer_load_u16(sc_rsrc, off);
             st.z[r] = ZERO ? buffer_load_u16(zr_rsrc, off) : (uint16_t) 0;
         }
@@ -145,7 +154,10 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
     __builtin_amdgcn_sched_barrier(0);
     WOQ_TR(2);
 
-    float total = 0.f; // this lane's share of output column c
+    float total[R]; // this lane's share of output column c, per activation row
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+        total[i] = 0.f;
     auto compute = [&](Stage& st)
     {
         // ---- products: D_g = A x W_g for every group g of the pass, S = A x ones ----
@@ -171,21 +183,24 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
                 for (int js = 0; js < SEG_SLABS; ++js)
                     acc[i][seg] = E::mma(st.a[js], expand_int4<DT>(st.w[i][seg * SEG_SLABS + js], nib), acc[i][seg]);
             }
-        // ---- row kg * 4 + r of D_(kg * 4 + r), scaled ----
+        // ---- row kg * 4 + r of D_g, g = (kg * 4 + r) / R, scaled ----
 #pragma unroll
         for (int r = 0; r < 4; ++r)
         {
             float P = 0.f;
 #pragma unroll
-            for (int q = 0; q < ROWS / 4; ++q)
+            for (int q = 0; q < 4; ++q)
             {
-                int const g = q * 4 + r;
-                float const v = acc[g / SEGS][g % SEGS][r];
-                P = kg == q ? v : P;
+                int const g = (q * 4 + r) / R;
+                if (g < GROUPS)
+                {
+                    float const v = acc[g / SEGS][g % SEGS][r];
+                    P = kg == q ? v : P;
+                }
             }
-            float const sc = E::from_bits(st.s[r]);
-            float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits(st.z[r]) : 0.f);
-            total = __builtin_fmaf(sc, P, __builtin_fmaf(cc, acc_s[r], total));
+            float const sc = E::from_bits(st.s[r - r % R]);
+            float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits(st.z[r - r % R]) : 0.f);
+            total[r % R] = __builtin_fmaf(sc, P, __builtin_fmaf(cc, acc_s[r], total[r % R]));
         }
     };
     compute(st[0]);
@@ -204,25 +219,31 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
 
     // ---- rows (lanes kg) of a wavefront, then the wavefronts, in fixed order ----
     WOQ_TR(6);
-    total += __shfl_xor(total, 16);
-    total += __shfl_xor(total, 32);
-    __shared__ float red[WAVES][16];
-    if (kg == 0)
-        red[wave][c] = total;
+    __shared__ float red[WAVES][R][16];
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+    {
+        total[i] += __shfl_xor(total[i], 16);
+        total[i] += __shfl_xor(total[i], 32);
+        if (kg == 0)
+            red[wave][i][c] = total[i];
+    }
     WOQ_TR(7);
     __syncthreads();
     WOQ_TR(8);
-    if (threadIdx.x < 16)
+    if (threadIdx.x < 16 * R)
     {
+        int const row = threadIdx.x >> 4;
         float sum = 0.f;
 #pragma unroll
         for (int w2 = 0; w2 < WAVES; ++w2)
-            sum += red[w2][c];
+            sum += red[w2][row][c];
         int const ocol = strip * 16 + c;
-        float v = alpha * sum;
+        float v = tail.alpha * sum;
         if (tail.bias)
             v += E::load(tail.bias, ocol);
-        static_cast<uint16_t*>(out)[ocol] = E::store(v);
+        if (row < tail.m)
+            static_cast<uint16_t*>(out)[(size_t) row * n + ocol] = E::store(v);
     }
 #ifdef WOQ_TIMELINE
     WOQ_TR(9);
@@ -237,67 +258,90 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_kernel(void const* weig
 
 namespace
 {
-template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int TPW>
+template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int TPW, int R>
 int launch_row_variant(StreamParams sp, hipStream_t stream)
 {
-    bool const multi = sp.k_tiles > WAVES * TPW; // K longer than one pass of the workgroup
-    sp.groups = sp.strips; // one workgroup per strip
-    sp.groups_per_xcd = (sp.groups + 7) / 8;
-    dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
-    note_launch("stream row waves=%d tpw=%d passes=%d", WAVES, TPW, (sp.k_tiles + WAVES * TPW - 1) / (WAVES * TPW));
-    RowTail tail{sp.pqs, sp.bias, nullptr};
-#ifdef WOQ_TIMELINE
-    if (char const* e = std::getenv("WOQ_TRACE_PTR"))
-        tail.trace = reinterpret_cast<unsigned long long*>(std::strtoull(e, nullptr, 16));
-#endif
-    if (multi)
-        hipLaunchKernelGGL((stream_row_kernel<DT, GROUP, PQS, ZERO, WAVES, TPW, true>), grid, block, 0, stream, sp.weight,
-            sp.act, sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, sp.alpha, sp.out, tail);
+    if constexpr (TPW * (128 / GROUP) * R > 16)
+        return fail(WOQ_ERR_UNSUPPORTED, "row stream shape: %d tiles of %d groups x %d rows do not fit the 16 MFMA rows", TPW,
+            128 / GROUP, R);
     else
-        hipLaunchKernelGGL((stream_row_kernel<DT, GROUP, PQS, ZERO, WAVES, TPW, false>), grid, block, 0, stream, sp.weight,
-            sp.act, sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, sp.alpha, sp.out, tail);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess)
-        return fail(WOQ_ERR_RUNTIME, "row stream kernel launch failed: %s", hipGetErrorString(err));
-    return WOQ_OK;
+    {
+        bool const multi = sp.k_tiles > WAVES * TPW; // K longer than one pass of the workgroup
+        sp.groups = sp.strips;                       // one workgroup per strip
+        sp.groups_per_xcd = (sp.groups + 7) / 8;
+        dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+        note_launch("stream row waves=%d tpw=%d passes=%d rows=%d", WAVES, TPW, (sp.k_tiles + WAVES * TPW - 1) / (WAVES * TPW),
+            R);
+        RowTail tail{sp.pqs, sp.bias, sp.alpha, sp.m, nullptr};
+#ifdef WOQ_TIMELINE
+        if (char const* e = std::getenv("WOQ_TRACE_PTR"))
+            tail.trace = reinterpret_cast<unsigned long long*>(std::strtoull(e, nullptr, 16));
+#endif
+        int const act_bytes = sp.m * sp.k * 2;
+        if (multi)
+            hipLaunchKernelGGL((stream_row_kernel<DT, GROUP, PQS, ZERO, WAVES, TPW, true, R>), grid, block, 0, stream,
+                sp.weight, sp.act, sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes,
+                sp.out, tail);
+        else
+            hipLaunchKernelGGL((stream_row_kernel<DT, GROUP, PQS, ZERO, WAVES, TPW, false, R>), grid, block, 0, stream,
+                sp.weight, sp.act, sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes,
+                sp.out, tail);
+        hipError_t err = hipGetLastError();
+        if (err != hipSuccess)
+            return fail(WOQ_ERR_RUNTIME, "row stream kernel launch failed: %s", hipGetErrorString(err));
+        return WOQ_OK;
+    }
 }
 
-template <int DT, int GROUP, bool PQS, bool ZERO>
+template <int DT, int GROUP, bool PQS, bool ZERO, int R>
 int launch_row_shaped(StreamParams const& sp, int waves, int tpw, hipStream_t s)
 {
 #define WOQ_ROW(WAVES_, TPW_)                                                                                          \
     if (waves == WAVES_ && tpw == TPW_)                                                                                \
-        return launch_row_variant<DT, GROUP, PQS, ZERO, WAVES_, TPW_>(sp, s);
-    WOQ_ROW(8, 4)
-    WOQ_ROW(16, 4)
+        return launch_row_variant<DT, GROUP, PQS, ZERO, WAVES_, TPW_, R>(sp, s);
+    WOQ_ROW(4, 8)
     WOQ_ROW(8, 8)
     WOQ_ROW(16, 8)
-    WOQ_ROW(4, 8)
+    WOQ_ROW(4, 4)
+    WOQ_ROW(8, 4)
+    WOQ_ROW(16, 2)
 #undef WOQ_ROW
     return fail(WOQ_ERR_UNSUPPORTED, "row stream shape waves=%d tpw=%d is not instantiated", waves, tpw);
 }
 
-template <int DT, int GROUP>
+template <int DT, int GROUP, int R>
 int launch_row_flags(StreamParams const& sp, bool pqs, bool zero, int waves, int tpw, hipStream_t s)
 {
     if (pqs)
-        return zero ? launch_row_shaped<DT, GROUP, true, true>(sp, waves, tpw, s)
-                    : launch_row_shaped<DT, GROUP, true, false>(sp, waves, tpw, s);
-    return zero ? launch_row_shaped<DT, GROUP, false, true>(sp, waves, tpw, s)
-                : launch_row_shaped<DT, GROUP, false, false>(sp, waves, tpw, s);
+        return zero ? launch_row_shaped<DT, GROUP, true, true, R>(sp, waves, tpw, s)
+                    : launch_row_shaped<DT, GROUP, true, false, R>(sp, waves, tpw, s);
+    return zero ? launch_row_shaped<DT, GROUP, false, true, R>(sp, waves, tpw, s)
+                : launch_row_shaped<DT, GROUP, false, false, R>(sp, waves, tpw, s);
+}
+
+template <int DT, int GROUP>
+int launch_row_rows(StreamParams const& sp, bool pqs, bool zero, int waves, int tpw, hipStream_t s)
+{
+    if (sp.m == 1)
+        return launch_row_flags<DT, GROUP, 1>(sp, pqs, zero, waves, tpw, s);
+    if (sp.m == 2)
+        return launch_row_flags<DT, GROUP, 2>(sp, pqs, zero, waves, tpw, s);
+    return launch_row_flags<DT, GROUP, 4>(sp, pqs, zero, waves, tpw, s);
 }
 } // namespace
 
 int launch_stream_row(StreamParams const& sp, int dtype, int group, bool pqs, bool zero, int waves, int tpw, void* stream)
 {
     auto s = static_cast<hipStream_t>(stream);
-    if (sp.m != 1 || (group != 64 && group != 128) || sp.k % group)
-        return fail(WOQ_ERR_UNSUPPORTED, "row stream kernel: one row, int4, group size 64 or 128");
+    if (sp.m < 1 || sp.m > 4 || (group != 64 && group != 128) || sp.k % group)
+        return fail(WOQ_ERR_UNSUPPORTED, "row stream kernel: one to four rows, int4, group size 64 or 128");
+    if ((uint64_t) sp.m * (uint64_t) sp.n * 2 >= ((uint64_t) 1 << 31))
+        return fail(WOQ_ERR_UNSUPPORTED, "row stream kernel: output beyond 2 GiB");
     if (dtype == WOQ_BF16)
-        return group == 64 ? launch_row_flags<WOQ_BF16, 64>(sp, pqs, zero, waves, tpw, s)
-                           : launch_row_flags<WOQ_BF16, 128>(sp, pqs, zero, waves, tpw, s);
-    return group == 64 ? launch_row_flags<WOQ_FP16, 64>(sp, pqs, zero, waves, tpw, s)
-                       : launch_row_flags<WOQ_FP16, 128>(sp, pqs, zero, waves, tpw, s);
+        return group == 64 ? launch_row_rows<WOQ_BF16, 64>(sp, pqs, zero, waves, tpw, s)
+                           : launch_row_rows<WOQ_BF16, 128>(sp, pqs, zero, waves, tpw, s);
+    return group == 64 ? launch_row_rows<WOQ_FP16, 64>(sp, pqs, zero, waves, tpw, s)
+                       : launch_row_rows<WOQ_FP16, 128>(sp, pqs, zero, waves, tpw, s);
 }
 
 } // namespace woq

@@ -176,6 +176,7 @@ def test_stream_narrow_n_long_k_stages_beyond_64k(pkg, oracle, dev, woq_env, M, 
     """Few column groups and a long K (a down projection at M = 2..4): the activations are staged in
     LDS although they take 57 / 115 KiB (by the heuristic up to 3 rows, since one workgroup per CU
     covers the problem anyway; forced for 4)."""
+    woq_env(WOQ_ROW_SHAPE="0")  # the strip-group kernel's test: the row kernel would take these
     if forced:
         woq_env(WOQ_STREAM_SHAPE="1,8,4,1")
     p = random_problem(oracle, M, 14336, 256, 4, 128, "bf16", zero=True, bias=True, seed=M)
@@ -251,50 +252,61 @@ def test_wide_decode_kernel_is_what_wide_single_row_int8_problems_run_on(pkg, or
     assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()
 
 
-@pytest.mark.parametrize("shape", ["8,4", "16,4", "8,8", "16,8", "4,8"])
+@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,2"])
 @pytest.mark.parametrize("group,dtype,K,N", [(128, "bf16", 2176, 272), (64, "fp16", 1408, 1040), (128, "fp16", 128, 16),
                                              (64, "bf16", 4160, 528), (128, "bf16", 14336, 48)])
 def test_row_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, K, N):
-    """The single-row kernel (one workgroup per strip, every wavefront a few consecutive tiles, no staging
-    pass), forced through WOQ_ROW_SHAPE: K that needs several passes of the workgroup or leaves wavefronts
-    without tiles, a last tile that is only half inside K, groups that end inside a wavefront's quad of rows;
-    every optional input."""
+    """The row kernel (one workgroup per strip, every wavefront a few consecutive tiles, no staging pass),
+    forced through WOQ_ROW_SHAPE for one to four rows: K that needs several passes of the workgroup or leaves
+    wavefronts without tiles, a last tile that is only half inside K, groups that end inside a wavefront's
+    rows; every optional input.  (A shape whose groups x rows exceed the 16 MFMA rows is refused and the call
+    falls through to the strip-group kernel.)"""
     woq_env(WOQ_ROW_SHAPE=shape)
-    for zero, bias, pqs in [(True, True, True), (False, False, False), (True, False, False), (False, True, True)]:
-        p = random_problem(oracle, 1, K, N, 4, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N)
-        err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
-        assert "stream row" in _last_launch(pkg), _last_launch(pkg)
-        assert err < TOL, (shape, zero, bias, pqs, err)
+    tiles = int(shape.split(",")[1])
+    for M in (1, 2, 3, 4):
+        fits = tiles * (128 // group) * (1 if M == 1 else (2 if M == 2 else 4)) <= 16
+        for zero, bias, pqs in [(True, True, True), (False, False, False), (True, False, False), (False, True, True)]:
+            p = random_problem(oracle, M, K, N, 4, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + M)
+            err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+            assert ("stream row" in _last_launch(pkg)) == fits, (M, _last_launch(pkg))
+            assert err < TOL, (shape, M, zero, bias, pqs, err)
 
 
-def test_row_decode_kernel_is_what_single_row_int4_problems_run_on(pkg, oracle, dev, woq_env):
-    """One row, int4 with group scales of 64 or 128: the built-in rule takes the single-row kernel, with one
-    pass over K where sixteen wavefronts x eight tiles reach that far; int8 weights, more rows, per-channel
-    scales or larger groups do not.  Every one-hot activation returns the dequantized weight row through it;
-    switched off, the strip-group kernel meets the same bar."""
+def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev, woq_env):
+    """One row, int4 with group scales of 64 or 128: the built-in rule takes the row kernel, with one pass over
+    K where sixteen wavefronts x eight tiles reach that far; two rows except at K = 8192 on narrow matrices;
+    three and four rows on narrow matrices with K up to 4096 or beyond 8192.  int8 weights, more rows,
+    per-channel scales or larger groups do not.  Every one-hot activation returns the dequantized weight row
+    through it; switched off, the strip-group kernel meets the same bar."""
     K, N = 4096, 272
     p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=78)
     auto = run_product(pkg, oracle, dev, p, 0)
-    assert "stream row waves=4 tpw=8 passes=1" in _last_launch(pkg), _last_launch(pkg)
+    assert "stream row waves=4 tpw=8 passes=1 rows=1" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, auto, p) < TOL
     w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")
-    for k_hot in (0, 127, 128, 2049, 4095):
-        p["act"] = np.zeros((1, K), np.float32)
-        p["act"][0, k_hot] = 1.0
+    for M in (1, 2, 4):
+        hot = [(997 * r + 127) % K for r in range(M)]
+        p = random_problem(oracle, M, K, N, 4, 128, "bf16", zero=True, seed=78)
+        p["act"] = np.zeros((M, K), np.float32)
+        p["act"][np.arange(M), hot] = 1.0
         out = run_product(pkg, oracle, dev, p, 0)
-        assert (np.abs(out[0] - w[k_hot]) <= np.abs(w[k_hot]) * 2.0 ** -7 + 2.5e-7).all(), k_hot
+        assert "stream row" in _last_launch(pkg), _last_launch(pkg)
+        assert (np.abs(out - w[hot]) <= np.abs(w[hot]) * 2.0 ** -7 + 2.5e-7).all(), M
     woq_env(WOQ_ROW_SHAPE="0")
     p = random_problem(oracle, 1, K, N, 4, 128, "bf16", zero=True, seed=78)
     other = run_product(pkg, oracle, dev, p, 0)
     assert "stream mt=1" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, other, p) < TOL
     woq_env(WOQ_ROW_SHAPE=None)
-    for K2, group, want in ((8192, 64, "waves=8 tpw=8 passes=1"), (14336, 128, "waves=16 tpw=8 passes=1"),
-                            (28672, 128, "waves=4 tpw=8 passes=7"), (128, 64, "waves=4 tpw=8 passes=1")):
-        q = random_problem(oracle, 1, K2, 48, 4, group, "fp16", zero=True, bias=True, pqs=True, seed=K2)
+    for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=8 passes=1 rows=1"), (1, 14336, 128, "waves=16 tpw=8 passes=1 rows=1"),
+                               (1, 28672, 128, "waves=4 tpw=8 passes=7 rows=1"), (1, 128, 64, "waves=4 tpw=8 passes=1 rows=1"),
+                               (2, 4096, 128, "waves=8 tpw=4 passes=1 rows=2"), (2, 28672, 64, "waves=4 tpw=4 passes=14 rows=2"),
+                               (3, 4096, 128, "waves=8 tpw=4 passes=1 rows=4"), (4, 14336, 64, "waves=16 tpw=2 passes=4 rows=4")):
+        q = random_problem(oracle, M, K2, 48, 4, group, "fp16", zero=True, bias=True, pqs=True, seed=K2 + M)
         assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL
-        assert "stream row " + want in _last_launch(pkg), (K2, _last_launch(pkg))
-    for kw in (dict(M=2), dict(bits=8, group=64), dict(group=0), dict(group=256)):
+        assert "stream row " + want in _last_launch(pkg), (M, K2, _last_launch(pkg))
+    for kw in (dict(M=5), dict(M=2, K=8192), dict(M=4, K=8192), dict(M=4, N=513 * 16), dict(bits=8, group=64),
+               dict(group=0), dict(group=256)):
         a = dict(M=1, K=K, N=N, bits=4, group=128)
         a.update(kw)
         q = random_problem(oracle, a["M"], a["K"], a["N"], a["bits"], a["group"], "bf16", seed=79)
