@@ -313,7 +313,7 @@ def bench_w4a8(pkg, dev, m=4096, reps=40):
         return dict(error=str(e)[:200])
 
 
-def run_for_counters(pkg, dev, mode, reps=20):
+def run_for_counters(pkg, dev, mode, reps=20, shape=None):
     """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
     dominant kernel (gate_up GEMV, rotating weight copies); `gemm<M>` launches the GEMM regime on
     gate_up at M rows (256-row tiles at 4096, 64-row tiles at 128); `copy` runs a plain device-to-device
@@ -371,14 +371,20 @@ def run_for_counters(pkg, dev, mode, reps=20):
         return
     if mode.startswith("gemm"):
         m = int(mode[4:] or 4096)
-        layer = make_layer(pkg, dev, k, n, 2002)
+        if shape:  # another layer shape than the 8B gate_up: "70b_qkv", "8b_down", ...
+            k, n = dict([("8b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_8B]
+                        + [("70b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_70B])[shape]
+        # weights rotate over copies beyond the last-level cache while they matter (M <= 256), as in the sweeps
+        copies = min(copies_beyond_cache(k * n // 2), 64) if m <= 256 else 1
+        layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
         act = torch.randn((m, k), device=dev).to(torch.bfloat16)
         out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
         for r in range(reps):
-            launch(pkg, act, layer, out)
+            launch(pkg, act, layers[r % copies], out)
         torch.cuda.synchronize()
-        print(json.dumps({"mode": mode, "kernel": "GEMM regime on gate_up K=4096 N=28672 M=%d" % m,
-                          "flop_per_launch": 2.0 * m * n * k, "launches": reps}))
+        print(json.dumps({"mode": mode, "kernel": "%s on %s K=%d N=%d M=%d" % (last_launch(pkg), shape or "8b_gate_up", k, n, m),
+                          "flop_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": algorithmic_bytes(m, k, n),
+                          "launches": reps}))
         return
     if mode == "dominant70b":  # the same GEMV on the Llama-3-70B gate_up
         _, k, n = SHAPES_70B[2]
@@ -567,6 +573,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
+    ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
     ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
@@ -594,7 +601,7 @@ def main():
         run_ceilings(pkg, dev)
         return
     if args.mode != "bench":
-        run_for_counters(pkg, dev, args.mode)
+        run_for_counters(pkg, dev, args.mode, shape=args.shape)
         return
     r = bench_decode(pkg, dev, args.steps, args.warmup)
     sec_per_step = r["host_s"] / args.steps

@@ -22,15 +22,16 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 # packed-fp32 ops are switched off for all device code (compiler-generated v_pk_*_f32 forms have
 # produced wrong results on this hardware pool)
-DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Kernels whose arguments are plain scalars find the first fourteen dwords of them in SGPRs when a wavefront
+# starts (kernel-argument preloading) instead of fetching them with scalar loads, 0.2-0.3 us per dependent
+# batch; kernels that take a struct by value are unaffected.
+DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
           "-ffp-contract=off"]
 # Per-file additions.  The skinny-M kernel reads its MFMA results with VALU instructions every
 # group: keep those accumulators in the architectural VGPRs instead of copying them out of AGPRs.
-# The single-row decode kernel takes what its first requests need as scalar arguments and has them preloaded
-# into SGPRs at wavefront start (no scalar loads from the argument buffer in front of the first address).
-PER_FILE = {"skinny_": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-            "stream_row": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
+PER_FILE = {"skinny_": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources():

@@ -279,6 +279,37 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
     return true;
 }
 
+// The W4A8 row kernel (stream_row_w4a8.hip) for this problem and its launch shape; WOQ_ROW_SHAPE as above.
+bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles)
+{
+    (void) n;
+    if (m < 1 || m > 4)
+        return false;
+    EnvOverrides const& env = env_overrides();
+    if (env.row_mode == 0 || env.has_stream_shape)
+        return false;
+    if (env.row_mode == 1)
+    {
+        waves = env.row_shape[0], tiles = env.row_shape[1];
+        return true;
+    }
+    // Measured on MI355X against the strip-group W4A8 kernel (both convert through the table): with K up to
+    // 4096 eight wavefronts x four tiles (4096 x 28672 at one row 15.9 -> 14.3 us, 4096 x 4096 5.08 -> 4.86);
+    // with K up to 8192 and at most 1024 strips sixteen x four (8192 x 8192 10.4 -> 9.7 us, at four rows
+    // 11.6 -> 10.8; 8192 x 10240 at four rows 14.6 -> 13.4).  The conversion, not the memory system, bounds
+    // this kernel (about 80 VALU instructions per KiB of weights), so the wide and long matrices, where the
+    // strip-group kernel's deeper pipeline keeps more of it under the loads, stay there.
+    int const k_tiles = (k + 127) / 128;
+    if (k_tiles <= 32)
+        waves = 8;
+    else if (k_tiles <= 64 && n <= 1024 * 16)
+        waves = 16;
+    else
+        return false;
+    tiles = 4;
+    return true;
+}
+
 // bytes of float32 slabs a streaming launch of m rows splitting K into `slices` needs
 static size_t stream_slab_bytes(int m, int n, int slices)
 {

@@ -135,11 +135,23 @@ __global__ void __launch_bounds__(256) gemm_finish_partial(
     size_t const i = ((size_t) blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= count)
         return;
+    // eight slabs are requested at a time (a loop of one dependent load after another paid a memory round
+    // trip per slab: 4-5 us for the 6-12 slabs of a skinny problem), then added in slab order; a request
+    // past the last slab re-reads that slab and is not added
     f32x4 sum = *reinterpret_cast<f32x4 const*>(partial + i);
-    for (int y = 1; y < splits; ++y)
+    for (int y = 1; y < splits; y += 8)
     {
-        f32x4 const v = *reinterpret_cast<f32x4 const*>(partial + (size_t) y * count + i);
-        sum[0] += v[0], sum[1] += v[1], sum[2] += v[2], sum[3] += v[3];
+        f32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+        {
+            int const yy = y + u < splits ? y + u : splits - 1;
+            v[u] = *reinterpret_cast<f32x4 const*>(partial + (size_t) yy * count + i);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (y + u < splits)
+                sum[0] += v[u][0], sum[1] += v[u][1], sum[2] += v[u][2], sum[3] += v[u][3];
     }
     int const col = (int) (i % n);
     f32x4 b = {0.f, 0.f, 0.f, 0.f};

@@ -140,24 +140,44 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             return st.z[s];
     };
 
-    NibbleConsts const nib = nibble_consts<WOQ_FP16>();
+    [[maybe_unused]] NibbleConsts const nib = nibble_consts<WOQ_FP16>();
+    [[maybe_unused]] float qf[4];
+    fp8_table_lane_values(kg, qf);
+    [[maybe_unused]] Fp8LookupConsts const lk = fp8_lookup_consts();
     // Saturation to +-448 is part of the conversion: the wavefront runs with the conversion instruction's
     // own saturating mode switched on (fp8_saturation_on below), as the tiled kernel does, so no clamp and
     // no test for scales that could reach the limit is needed.
-    auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 const (&a)[MT], auto clamp_tag)
+    auto convert_and_multiply = [&](Stage const& st, int kt, i32x8 const (&a)[MT])
     {
-        constexpr bool CLAMP = decltype(clamp_tag)::value;
 #pragma unroll
         for (int s = 0; s < NS; ++s)
         {
             float const sc = EH::from_bits(scale_bits(st, kt, s));
             float const zr = ZERO ? EH::from_bits(zero_bits(st, kt, s)) : 0.f;
             i32x8 b;
+            if constexpr (MT == 1)
+            {
+                // the sixteen possible results of this (group, column), then every weight a table look-up
+                // (70B gate_up at M = 1: 54.3 -> 51.1 us, at M = 16 56.4 -> 52.6; with two row tiles the
+                // reordering of twice the A operand makes it 4 % slower than the arithmetic form)
+                Fp8Table const table = build_fp8_table(sc, zr, qf);
 #pragma unroll
-            for (int j = 0; j < SLABS; ++j)
+                for (int j = 0; j < SLABS; ++j)
+                {
+                    uint32_t b0, b1;
+                    fp8_lookup8(st.w[s][j], table, lk, b0, b1);
+                    b[2 * j] = (int) b0;
+                    b[2 * j + 1] = (int) b1;
+                }
+            }
+            else
+            {
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    b[2 * j + h] = (int) dequant4_fp8<ZERO, CLAMP>(st.w[s][j], h, sc, zr, nib);
+                for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        b[2 * j + h] = (int) dequant4_fp8<ZERO, false>(st.w[s][j], h, sc, zr, nib);
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 acc[s][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[mt], b, acc[s][mt], 0, 0, 0, 0, 0, 0);
@@ -173,10 +193,13 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
             {
                 u32x2 const v = ALDS ? *reinterpret_cast<u32x2 const*>(a_lds + (uint32_t) (kt * TK + j * 32))
                                      : st.a[ALDS ? 0 : j][mt];
-                a[mt][2 * j] = (int) v[0];
-                a[mt][2 * j + 1] = (int) v[1];
+                uint32_t a0 = v[0], a1 = v[1];
+                if constexpr (MT == 1) // the lane's eight k-values in the order the weight look-up delivers them
+                    fp8_a_order(v[0], v[1], a0, a1);
+                a[mt][2 * j] = (int) a0;
+                a[mt][2 * j + 1] = (int) a1;
             }
-        convert_and_multiply(st, kt, a, std::false_type{});
+        convert_and_multiply(st, kt, a);
     };
 
     // tile rows of this wavefront: kt = wave + it * WAVES.  Every load tolerates kt >= KT, so
@@ -457,6 +480,9 @@ int launch_shaped(StreamParams const& sp, hipStream_t s)
 
 } // namespace
 
+int launch_stream_row_w4a8(StreamParams const& sp, int out_dtype, int waves, int tpw, void* stream);
+bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles);
+
 int launch_stream_w4a8(MatmulProblem const& p, void* stream)
 {
     if (p.m > kStreamW4a8MaxM)
@@ -484,6 +510,16 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream)
     sp.groups = sp.groups_per_xcd = 0;
     auto s = static_cast<hipStream_t>(stream);
     bool const zero = p.zeros != nullptr;
+    {
+        // one to four rows: the row kernel (stream_row_w4a8.hip), where the rule (or WOQ_ROW_SHAPE) picks it
+        int waves = 0, tiles = 0;
+        if (pick_row_w4a8_shape(p.m, p.n, p.k, waves, tiles))
+        {
+            int const rc = launch_stream_row_w4a8(sp, p.out_dtype, waves, tiles, stream);
+            if (rc != WOQ_ERR_UNSUPPORTED)
+                return rc;
+        }
+    }
     if (p.out_dtype == WOQ_BF16)
         return zero ? launch_shaped<WOQ_BF16, true>(sp, s) : launch_shaped<WOQ_BF16, false>(sp, s);
     return zero ? launch_shaped<WOQ_FP16, true>(sp, s) : launch_shaped<WOQ_FP16, false>(sp, s);

@@ -96,6 +96,79 @@ __device__ __forceinline__ uint32_t dequant4_fp8(uint32_t w, int h, float s, flo
     return (uint32_t) r;
 }
 
+// ---- table form of the same dequantize (the decode kernels) ----------------------------------------
+// A (group, column) has only sixteen possible results e4m3(fma(u - 8, s, z)), u = 0 .. 15 the stored
+// nibble.  The four lanes (kg = 0 .. 3) that hold one column of a tile each convert four of them - the
+// same FMA and the same saturating conversion instruction as dequant4_fp8, so the bytes are identical -
+// and exchange their quarters; every weight is then a byte looked up with v_perm_b32: 13 instructions
+// per eight weights instead of 17-22, plus 12 per tile for the table.  Requires fp8_saturation_on().
+struct Fp8Table
+{
+    uint32_t t[4]; // entries 4 i .. 4 i + 3 in dword i, entry u in byte u % 4
+};
+
+// qf[i] = float(4 kg + i - 8): the signed values of the lane's four table entries
+__device__ __forceinline__ void fp8_table_lane_values(int kg, float (&qf)[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        qf[i] = (float) (4 * kg + i - 8);
+}
+
+__device__ __forceinline__ Fp8Table build_fp8_table(float s, float z, float const (&qf)[4])
+{
+    float const v0 = __builtin_fmaf(qf[0], s, z), v1 = __builtin_fmaf(qf[1], s, z);
+    float const v2 = __builtin_fmaf(qf[2], s, z), v3 = __builtin_fmaf(qf[3], s, z);
+    int d = __builtin_amdgcn_cvt_pk_fp8_f32(v0, v1, 0, false);
+    d = __builtin_amdgcn_cvt_pk_fp8_f32(v2, v3, d, true);
+    // all-gather over the four rows of sixteen lanes: D = the lane's own quarter, D_r that of row r
+    auto const r = __builtin_amdgcn_permlane16_swap((uint32_t) d, (uint32_t) d, false, false); // [D0 D0 D2 D2], [D1 D1 D3 D3]
+    auto const e = __builtin_amdgcn_permlane32_swap(r[0], r[0], false, false);                   // D0 everywhere, D2 everywhere
+    auto const o = __builtin_amdgcn_permlane32_swap(r[1], r[1], false, false);                   // D1 everywhere, D3 everywhere
+    return Fp8Table{{e[0], o[0], e[1], o[1]}};
+}
+
+// Constants of the look-up as values the compiler cannot see through: with literals it emits v_and + v_or
+// (a VOP3 encoding carries no 32-bit literal on gfx9); with the mask in an SGPR and the byte numbers in a
+// VGPR it selects the fused v_and_or_b32 (as NibbleConsts does for the 16-bit kernels).
+struct Fp8LookupConsts
+{
+    uint32_t low3;  // 0x07070707, SGPR
+    uint32_t bit2;  // 0x04040404, SGPR
+    uint32_t bytes; // 0x03020100, VGPR
+};
+
+__device__ __forceinline__ Fp8LookupConsts fp8_lookup_consts()
+{
+    Fp8LookupConsts k{0x07070707u, 0x04040404u, 0x03020100u};
+    asm volatile("" : "+s"(k.low3));
+    asm volatile("" : "+s"(k.bit2));
+    asm volatile("" : "+v"(k.bytes));
+    return k;
+}
+
+// The eight weights of slab dword `w` (element e in nibble e even ? e / 2 : 4 + e / 2) -> two operand
+// dwords in the order the nibbles sit in: bytes [e0, e4, e1, e5] and [e2, e6, e3, e7].  The A operand
+// has to present its eight k-values in the same order (fp8_a_order).
+__device__ __forceinline__ void fp8_lookup8(uint32_t w, Fp8Table const& T, Fp8LookupConsts const& k, uint32_t& b0, uint32_t& b1)
+{
+    uint32_t const sel_e = w & k.low3, sel_o = (w >> 4) & k.low3; // entry % 8 of the low / high nibbles
+    uint32_t const lo_e = __builtin_amdgcn_perm(T.t[1], T.t[0], sel_e), hi_e = __builtin_amdgcn_perm(T.t[3], T.t[2], sel_e);
+    uint32_t const lo_o = __builtin_amdgcn_perm(T.t[1], T.t[0], sel_o), hi_o = __builtin_amdgcn_perm(T.t[3], T.t[2], sel_o);
+    // bit 3 of each nibble picks the upper half of the table: byte j from lo (selector j) or hi (4 + j)
+    uint32_t const pick_e = ((w >> 1) & k.bit2) | k.bytes;
+    uint32_t const pick_o = ((w >> 5) & k.bit2) | k.bytes;
+    b0 = __builtin_amdgcn_perm(hi_e, lo_e, pick_e);
+    b1 = __builtin_amdgcn_perm(hi_o, lo_o, pick_o);
+}
+
+// eight consecutive k-values (bytes a0 .. a7 in v0, v1) in the order fp8_lookup8 delivers the weights
+__device__ __forceinline__ void fp8_a_order(uint32_t v0, uint32_t v1, uint32_t& a0, uint32_t& a1)
+{
+    a0 = __builtin_amdgcn_perm(v1, v0, 0x05010400u); // [a0, a4, a1, a5]
+    a1 = __builtin_amdgcn_perm(v1, v0, 0x07030602u); // [a2, a6, a3, a7]
+}
+
 // MODE.FP16_OVFL (bit 23 of the wavefront's MODE register) makes v_cvt_pk_fp8_f32 saturate finite
 // overflow to +-448 instead of producing NaN - the rounding the W4A8 dequantize is defined with.
 // The bit also makes fp16 results clamp instead of overflowing to infinity, so it is switched off

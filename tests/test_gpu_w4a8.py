@@ -317,3 +317,58 @@ def test_w4a8_flexible_groups_one_hot_rows(pkg, oracle, dev):
             out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, regime=regime, group=G)
             w8 = oracle.dequantize(q, s, z, G, "fp8")
             assert (out == oracle.round_f16(w8[rows])).all(), (regime, z is not None)
+
+
+@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,4"])
+@pytest.mark.parametrize("K,N", [(2176, 272), (128, 16), (8192, 48), (14336, 32)])
+def test_w4a8_row_kernel_forced(pkg, oracle, dev, woq_env, shape, K, N):
+    """The W4A8 row kernel (one workgroup per strip, no staging pass, weights converted through the table of
+    their (group, column)), forced through WOQ_ROW_SHAPE for one to four rows: several passes over K, wavefronts
+    without tiles, with and without zeros; 16-bit activations through the smoothing pass and e4m3 activations
+    handed over directly give the same bits.  A shape whose tiles x rows exceed the 16 MFMA rows is refused
+    and the call runs on the strip-group kernel."""
+    tiles = int(shape.split(",")[1])
+    for M in (1, 2, 3, 4):
+        fits = tiles * (1 if M == 1 else (2 if M == 2 else 4)) <= 16
+        prob = oracle.make_w4a8_problem(M, K, N, seed=K + N + M, out_dtype="bf16")
+        rng = np.random.default_rng(M + K)
+        zeros = oracle.round_f16((rng.standard_normal((K // 128, N)) * 20).astype(np.float32))
+        bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+        for z, b in ((None, None), (zeros, bias)):
+            woq_env(WOQ_ROW_SHAPE=shape)
+            out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, regime=STREAM)
+            assert ("stream row w4a8" in _launch(pkg)) == fits, (M, _launch(pkg))
+            assert _perr(oracle, out, ref, prob) < TOL, (shape, M, z is not None)
+            direct, _ = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, direct_fp8=True, regime=STREAM)
+            assert (direct == out).all()
+            woq_env(WOQ_ROW_SHAPE="0")
+            other, _ = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, regime=STREAM)
+            assert "stream w4a8" in _launch(pkg), _launch(pkg)
+            assert oracle.max_rel_err(other, out) < 2e-3
+
+
+def test_w4a8_row_kernel_rule_and_exact_rows(pkg, oracle, dev):
+    """One to four rows with K up to 4096, or up to 8192 on at most 1024 strips, run on the row kernel; one-hot
+    rows and saturating scales come back as the e4m3-rounded dequantized weight rows, bit for bit (the table is
+    built with the arithmetic form's own FMA and saturating conversion), also with groups of 256."""
+    rng = np.random.default_rng(31)
+    for M, K, N, G, want in ((1, 4096, 272, 128, "waves=8 tpw=4 passes=1 rows=1"), (4, 1024, 64, 128, "waves=8 tpw=4 passes=1 rows=4"),
+                             (2, 8192, 48, 256, "waves=16 tpw=4 passes=1 rows=2"), (3, 8192, 16400, 128, None),
+                             (1, 14336, 32, 128, None), (5, 1024, 64, 128, None)):
+        rows_g = -(-K // G)
+        q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+        s = oracle.round_f16(np.exp(rng.uniform(-2, 4.5, (rows_g, N))).astype(np.float32))  # up to 90: saturates
+        zeros = oracle.round_f16((rng.standard_normal((rows_g, N)) * 100).astype(np.float32))
+        hot = rng.choice(K, size=M, replace=False)
+        act = np.zeros((M, K), np.float32)
+        act[np.arange(M), hot] = 1.0
+        prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+        for z in (None, zeros):
+            out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, group=G)
+            if want is None:
+                assert "stream row w4a8" not in _launch(pkg), (M, K, N, _launch(pkg))
+            else:
+                assert "stream row w4a8 " + want in _launch(pkg), (M, K, N, _launch(pkg))
+            w8 = oracle.dequantize(q, s, z, G, "fp8")
+            assert np.abs(w8).max() == 448.0
+            assert (out == oracle.round_f16(w8[hot])).all(), (M, K, N, z is not None)
