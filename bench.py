@@ -139,20 +139,38 @@ def launch(pkg, act, layer, out, regime=0):
                      regime=regime, workspace=workspace_for(pkg, act.shape[0], layer, act.device))
 
 
-def time_graph(fn_body, launches, repeats=1):
-    """Captures fn_body() (which issues `launches` kernels) in a HIP graph, replays it once
-    untimed, then times one replay with HIP events on the replay stream and with the host clock
-    (`repeats` > 1: the fastest of that many timed replays, for short cases that would otherwise
-    be measured while the clocks still ramp up)."""
+SETTLE_S = 0.08  # untimed replays before a timed one; see time_graph
+
+
+def time_graph(fn_body, launches, repeats=1, settle_s=SETTLE_S, first=None):
+    """Captures fn_body() (which issues `launches` kernels) in a HIP graph, replays it untimed until
+    `settle_s` seconds have passed, then times one replay with HIP events on the replay stream and with
+    the host clock (`repeats` > 1: the median of that many timed replays).
+
+    Why the untimed replays: when load starts on an idle GPU, the first millisecond runs at full clocks,
+    then the power management pulls the clocks down (kernels take up to 1.5x as long) and lets them come
+    back over the next 20-40 ms, after which the time per launch stays flat for seconds.  A timed replay
+    without the settling phase lands somewhere on that curve.  `first`, a dict, receives the event time
+    of the very first replay ("first_replay_s"), the figure a measurement without settling would give."""
     stream = torch.cuda.Stream()
     stream.wait_stream(torch.cuda.current_stream())
-    best = None
+    timed = []
     with torch.cuda.stream(stream):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
             fn_body()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
         graph.replay()
+        e1.record(stream)
         torch.cuda.synchronize()
+        if first is not None:
+            first["first_replay_s"] = e0.elapsed_time(e1) * 1e-3
+        t_settle = time.perf_counter()
+        while time.perf_counter() - t_settle < settle_s:
+            graph.replay()
+            graph.replay()
+            torch.cuda.synchronize()
         for _ in range(repeats):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
@@ -161,10 +179,9 @@ def time_graph(fn_body, launches, repeats=1):
             e1.record(stream)
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-            cur = ((t1 - t0), e0.elapsed_time(e1) * 1e-3, launches)
-            if best is None or cur[1] < best[1]:
-                best = cur
-    return best
+            timed.append(((t1 - t0), e0.elapsed_time(e1) * 1e-3, launches))
+    timed.sort(key=lambda t: t[1])
+    return timed[len(timed) // 2]
 
 
 def bench_decode(pkg, dev, steps, warmup, m=1):
@@ -185,7 +202,8 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
     for s in range(warmup):
         step(s)
     torch.cuda.synchronize()
-    host_s, ev_s, _ = time_graph(lambda: [step(s) for s in range(steps)], steps * len(SHAPES_8B))
+    first = {}
+    host_s, ev_s, _ = time_graph(lambda: [step(s) for s in range(steps)], steps * len(SHAPES_8B), first=first)
 
     # dominant kernel on its own: the gate_up GEMV
     gi = 2
@@ -201,7 +219,7 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
         _, s_s, s_l = time_graph(
             lambda: [launch(pkg, acts[k], layers[i][r % len(layers[i])], outs[i]) for r in range(reps)], reps)
         per_shape[name] = dict(us=round(s_s / s_l * 1e6, 3), gbs=round(algorithmic_bytes(m, k, n) / (s_s / s_l) / 1e9, 1))
-    return dict(host_s=host_s, ev_s=ev_s, per_step_bytes=per_step_bytes, copies=copies, dom_dur=dom_dur,
+    return dict(host_s=host_s, ev_s=ev_s, first_replay_s=first["first_replay_s"], per_step_bytes=per_step_bytes, copies=copies, dom_dur=dom_dur,
                 dom_bytes=dom_bytes, dom_launch=dom_launch, per_shape=per_shape, layers=layers, acts=acts)
 
 
@@ -245,8 +263,7 @@ def bench_cpu_baseline(layers, acts, m=1, budget_s=15.0):
 
 def bench_gemm(pkg, dev, m=4096, reps=40):
     """Prefill regime, largest shape (gate_up): TFLOP/s at M = 4096, as the average of `reps` launches
-    back to back (a replay of ~30 ms: bursts of a few launches run 5-9 % slower, on this kernel and on the
-    vendor library's alike, because the clocks have not settled yet)."""
+    back to back (a replay of ~30 ms, after the settling replays every timing here has)."""
     try:
         name, k, n = SHAPES_8B[2]
         layer = make_layer(pkg, dev, k, n, 3000)
@@ -255,7 +272,7 @@ def bench_gemm(pkg, dev, m=4096, reps=40):
         out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
         launch(pkg, act, layer, out)
         torch.cuda.synchronize()
-        # the launches replay from a HIP graph, once untimed first; the fastest of three timed replays
+        # the launches replay from a HIP graph; the median of three timed replays
         _, sec, launches = time_graph(lambda: [launch(pkg, act, layer, out) for _ in range(reps)], reps, repeats=3)
         launched = last_launch(pkg)
         sec /= launches
@@ -313,30 +330,41 @@ def bench_w4a8(pkg, dev, m=4096, reps=40):
         return dict(error=str(e)[:200])
 
 
-def run_for_counters(pkg, dev, mode, reps=20, shape=None):
-    """Helpers for `rocprofv3 --pmc` runs (one counter set per run): `dominant` launches only the
+def run_for_counters(pkg, dev, mode, reps=20, shape=None, replay_ms=0):
+    """Helpers for `rocprofv3` runs (one counter set per --pmc run): `dominant` launches only the
     dominant kernel (gate_up GEMV, rotating weight copies); `gemm<M>` launches the GEMM regime on
     gate_up at M rows (256-row tiles at 4096, 64-row tiles at 128); `copy` runs a plain device-to-device
     copy of a known size (256 MiB read + 256 MiB written per launch), whose FETCH_SIZE /
-    WRITE_SIZE readings calibrate the counters."""
+    WRITE_SIZE readings calibrate the counters.  Each mode issues `reps` plain launches; with
+    `replay_ms` it then replays 40 launches from a HIP graph for that long and times three more
+    replays, as the sweeps do - for kernel traces (see summarize_trace), not for counter runs."""
+    def finish(issue, line):
+        for r in range(reps):
+            issue(r)
+        torch.cuda.synchronize()
+        line["launches"] = reps
+        if replay_ms > 0:
+            first = {}
+            _, sec, launches = time_graph(lambda: [issue(r) for r in range(40)], 40, repeats=3,
+                                          settle_s=replay_ms * 1e-3, first=first)
+            line["replayed"] = {"ms": replay_ms, "launches_per_replay": 40,
+                                "us_per_launch": round(sec / launches * 1e6, 2),
+                                "first_replay_us_per_launch": round(first["first_replay_s"] / 40 * 1e6, 2)}
+        print(json.dumps(line))
+
     if mode == "copy":
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
         dst = torch.empty_like(src)
-        for _ in range(reps):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"mode": "copy", "bytes_read_per_launch": 256 << 20, "bytes_written_per_launch": 256 << 20,
-                          "launches": reps}))
+        finish(lambda r: dst.copy_(src),
+               {"mode": "copy", "bytes_read_per_launch": 256 << 20, "bytes_written_per_launch": 256 << 20})
         return
     if mode == "w4a8_decode":
         _, k, n = SHAPES_70B[2]
         copies = copies_beyond_cache(k * n // 2)
         run = w4a8_setup(pkg, dev, 1, k, n, copies=copies)
-        for r in range(reps):
-            run(r)
-        torch.cuda.synchronize()
-        print(json.dumps({"mode": mode, "kernel": "W4A8 streaming kernel on 70B gate_up K=8192 N=57344 M=1",
-                          "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n, 4, GROUP, 1, 1), "launches": reps}))
+        run(0)
+        finish(run, {"mode": mode, "kernel": last_launch(pkg) + " on 70B gate_up K=8192 N=57344 M=1",
+                     "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n, 4, GROUP, 1, 1)})
         return
     if mode == "moe_decode":
         F = pkg.functional
@@ -350,24 +378,19 @@ def run_for_counters(pkg, dev, mode, reps=20, shape=None):
         total = torch.cumsum(rows, 0).to(torch.int64).to(dev)
         act = torch.randn((int(rows.sum()), k), device=dev).to(torch.bfloat16)
         out = torch.empty((act.shape[0], n // 2), dtype=torch.bfloat16, device=dev)
-        for r in range(reps):
-            F.woq_grouped_matmul_raw(act, weight[r % copies], scales, zeros, None, total, n=n, k=k, group_size=GROUP,
-                                     quant_algo=F.ZERO, activation="swiglu", out=out)
-        torch.cuda.synchronize()
         by = experts * (k * n // 2 + (k // GROUP) * n * 4) + act.numel() * 2 + out.numel() * 2
-        print(json.dumps({"mode": mode, "kernel": "grouped streaming kernel, 8 experts K=4096 N=28672 + swiglu, "
-                                                  "32 rows (16 tokens, top-2)",
-                          "algorithmic_bytes_per_launch": by, "launches": reps}))
+        finish(lambda r: F.woq_grouped_matmul_raw(act, weight[r % copies], scales, zeros, None, total, n=n, k=k,
+                                                  group_size=GROUP, quant_algo=F.ZERO, activation="swiglu", out=out),
+               {"mode": mode, "kernel": "grouped streaming kernel, 8 experts K=4096 N=28672 + swiglu, "
+                                        "32 rows (16 tokens, top-2)", "algorithmic_bytes_per_launch": by})
         return
     _, k, n = SHAPES_8B[2]
     if mode.startswith("w4a8_") and mode[5:].isdigit():
         m = int(mode[5:])
         run = w4a8_setup(pkg, dev, m, k, n)
-        for r in range(reps):
-            run()
-        torch.cuda.synchronize()
-        print(json.dumps({"mode": mode, "kernel": "W4A8 GEMM on gate_up K=4096 N=28672 M=%d" % m,
-                          "flop_per_launch": 2.0 * m * n * k, "launches": reps}))
+        run()
+        finish(lambda r: run(), {"mode": mode, "kernel": "%s on gate_up K=4096 N=28672 M=%d" % (last_launch(pkg), m),
+                                 "flop_per_launch": 2.0 * m * n * k})
         return
     if mode.startswith("gemm"):
         m = int(mode[4:] or 4096)
@@ -379,12 +402,10 @@ def run_for_counters(pkg, dev, mode, reps=20, shape=None):
         layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
         act = torch.randn((m, k), device=dev).to(torch.bfloat16)
         out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
-        for r in range(reps):
-            launch(pkg, act, layers[r % copies], out)
-        torch.cuda.synchronize()
-        print(json.dumps({"mode": mode, "kernel": "%s on %s K=%d N=%d M=%d" % (last_launch(pkg), shape or "8b_gate_up", k, n, m),
-                          "flop_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": algorithmic_bytes(m, k, n),
-                          "launches": reps}))
+        launch(pkg, act, layers[0], out)
+        finish(lambda r: launch(pkg, act, layers[r % copies], out),
+               {"mode": mode, "kernel": "%s on %s K=%d N=%d M=%d" % (last_launch(pkg), shape or "8b_gate_up", k, n, m),
+                "flop_per_launch": 2.0 * m * n * k, "algorithmic_bytes_per_launch": algorithmic_bytes(m, k, n)})
         return
     if mode == "dominant70b":  # the same GEMV on the Llama-3-70B gate_up
         _, k, n = SHAPES_70B[2]
@@ -392,11 +413,29 @@ def run_for_counters(pkg, dev, mode, reps=20, shape=None):
     layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
     act = torch.randn((1, k), device=dev).to(torch.bfloat16)
     out = torch.empty((1, n), dtype=torch.bfloat16, device=dev)
-    for r in range(reps):
-        launch(pkg, act, layers[r % copies], out)
-    torch.cuda.synchronize()
-    print(json.dumps({"mode": mode, "kernel": last_launch(pkg) + " on gate_up K=%d N=%d M=1" % (k, n),
-                      "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n), "launches": reps}))
+    launch(pkg, act, layers[0], out)
+    finish(lambda r: launch(pkg, act, layers[r % copies], out),
+           {"mode": mode, "kernel": last_launch(pkg) + " on gate_up K=%d N=%d M=1" % (k, n),
+            "algorithmic_bytes_per_launch": algorithmic_bytes(1, k, n)})
+
+
+def summarize_trace(path):
+    """Reads a `rocprofv3 --kernel-trace --output-format csv` kernel trace and prints, per kernel, the
+    dispatch count and the durations (end - begin stamp, us): mean of all, median of the first 20
+    dispatches (a GPU that was idle just before), largest median over any 40 consecutive dispatches (the dip
+    of the clocks that follows), median of the last quarter (settled).  No GPU needed."""
+    import csv
+    import statistics as st
+    by_kernel = {}
+    for row in csv.DictReader(open(path)):
+        by_kernel.setdefault(row["Kernel_Name"], []).append((int(row["Start_Timestamp"]), int(row["End_Timestamp"])))
+    for name, stamps in sorted(by_kernel.items(), key=lambda kv: -sum(e - b for b, e in kv[1])):
+        stamps.sort()
+        d = [(e - b) / 1e3 for b, e in stamps]
+        worst = max(st.median(d[i:i + 40]) for i in range(0, max(1, len(d) - 39), 20))
+        print(json.dumps({"kernel": name[:120], "dispatches": len(d), "mean_us": round(st.mean(d), 2),
+                          "first20_median_us": round(st.median(d[:20]), 2), "worst40_median_us": round(worst, 2),
+                          "last_quarter_median_us": round(st.median(d[-max(1, len(d) // 4):]), 2)}))
 
 
 SWEEPS = {
@@ -573,6 +612,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-gemm", action="store_true", help="skip the M=4096 extra")
+    ap.add_argument("--replay-ms", type=int, default=0,
+                    help="counter / trace modes: afterwards replay the launches from a HIP graph for this long")
+    ap.add_argument("--summarize-trace", default=None, metavar="CSV",
+                    help="print per-kernel durations of a rocprofv3 kernel trace (no GPU needed) and exit")
     ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
     ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings"],
@@ -582,6 +625,9 @@ def main():
     ap.add_argument("--tuned", action="store_true",
                     help="sweep: also profile each layer's tactics and time the tuned choices")
     args = ap.parse_args()
+    if args.summarize_trace:
+        summarize_trace(args.summarize_trace)
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1): the op contains no communication, a "
                  "tensor-parallel model gives each GPU its own column or row slice of the weights")
@@ -601,7 +647,7 @@ def main():
         run_ceilings(pkg, dev)
         return
     if args.mode != "bench":
-        run_for_counters(pkg, dev, args.mode, shape=args.shape)
+        run_for_counters(pkg, dev, args.mode, shape=args.shape, replay_ms=args.replay_ms)
         return
     r = bench_decode(pkg, dev, args.steps, args.warmup)
     sec_per_step = r["host_s"] / args.steps
@@ -621,6 +667,10 @@ def main():
                      "bytes_per_launch": r["dom_bytes"], "us_per_launch": round(r["dom_dur"] * 1e6, 3)},
         "per_shape": r["per_shape"],
         "event_ms_per_step": round(r["ev_s"] / args.steps * 1e3, 5),
+        # every timed replay follows SETTLE_S of untimed replays of the same graph (the clocks of a GPU that
+        # was idle dip for 20-40 ms after load starts); the step's very first replay, by the events, for comparison
+        "settle_ms": SETTLE_S * 1e3,
+        "first_replay_ms_per_step": round(r["first_replay_s"] / args.steps * 1e3, 5),
     }
     if not args.no_gemm:
         line["gemm"] = bench_gemm(pkg, dev)
