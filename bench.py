@@ -599,10 +599,58 @@ def run_ceilings(pkg, dev):
             torch.cuda.synchronize()
             _, sec, launches = time_graph(body, 8, repeats=3)
             tf = flop[0] / (sec / launches) / 1e12
-            out.setdefault("mfma", []).append({"instruction": name, "operands": "random" if random_operands else "constant",
-                                               "tflops": round(tf, 1), "peak": peak, "frac_of_peak": round(tf / peak, 4),
-                                               "ms_per_launch": round(sec / launches * 1e3, 3)})
+            entry = {"instruction": name, "operands": "random" if random_operands else "constant",
+                     "tflops": round(tf, 1), "peak": peak, "frac_of_peak": round(tf / peak, 4),
+                     "ms_per_launch": round(sec / launches * 1e3, 3)}
+            if kind != 2:  # the 16x16 probes leave shader-clock cycles and 100 MHz ticks of one wavefront's loop
+                counts = sink.view(torch.int32)[1020:1022].tolist()
+                if counts[1] > 0:
+                    entry["shader_clock_mhz"] = round((counts[0] & 0xFFFFFFFF) / counts[1] * 100.0)
+            out.setdefault("mfma", []).append(entry)
     print(json.dumps(out))
+
+
+def run_operands(pkg, dev, m=4096, reps=20):
+    """The real prefill kernels (W4A16 g128 bf16 and W4A8 on the 8B gate_up at M = 4096) on three sets of
+    operands: the benchmark's random ones, the same weights with all-zero activations, and all-zero activations
+    with weights whose stored bytes are all equal (every nibble 8: q = 0).  The instruction stream is the same
+    in all three; what differs is the switching activity in the matrix core and with it the clock the power
+    management sustains.  One JSON line."""
+    name, k, n = SHAPES_8B[2]
+    layer = make_layer(pkg, dev, k, n, 3000)
+    flat = dict(layer)
+    flat["weight"] = torch.full_like(layer["weight"], 0x88 - 256 if layer["weight"].dtype == torch.int8 else 0x88)
+    g = torch.Generator(device=dev).manual_seed(3999)
+    act_r = torch.randn((m, k), generator=g, device=dev).to(torch.bfloat16)
+    act_0 = torch.zeros_like(act_r)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    line = {"mode": "operands", "shape": name, "m": m, "w4a16": {}, "w4a8": {}}
+    for label, act, lay in [("random", act_r, layer), ("zero_activations", act_0, layer),
+                            ("zero_activations_flat_weights", act_0, flat)]:
+        launch(pkg, act, lay, out)
+        torch.cuda.synchronize()
+        _, sec, launches = time_graph(lambda: [launch(pkg, act, lay, out) for _ in range(reps)], reps, repeats=3)
+        tf = 2.0 * m * n * k / (sec / launches) / 1e12
+        line["w4a16"][label] = {"us": round(sec / launches * 1e6, 1), "tflops": round(tf, 1),
+                                "frac_of_bf16_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)}
+    line["w4a16"]["kernel"] = last_launch(pkg)
+    F = pkg.functional
+    scales16 = layer["scales"].to(torch.float16)
+    a8_r = (torch.randn((m, k), generator=g, device=dev) * 0.5).to(torch.float8_e4m3fn)
+    a8_0 = torch.zeros_like(a8_r)
+    for label, act, lay in [("random", a8_r, layer), ("zero_activations", a8_0, layer),
+                            ("zero_activations_flat_weights", a8_0, flat)]:
+        def run():
+            F.woq_matmul_raw(act, None, lay["weight"], scales16, None, None, n=n, k=k, group_size=GROUP,
+                             quant_algo=F.FP8_ALPHA, alpha=0.5, out_dtype=torch.bfloat16, out=out)
+        run()
+        torch.cuda.synchronize()
+        _, sec, launches = time_graph(lambda: [run() for _ in range(reps)], reps, repeats=3)
+        tf = 2.0 * m * n * k / (sec / launches) / 1e12
+        line["w4a8"][label] = {"us": round(sec / launches * 1e6, 1), "tflops": round(tf, 1),
+                               "frac_of_fp8_peak": round(tf / MFMA_FP8_PEAK_TFLOPS, 4)}
+    line["w4a8"]["kernel"] = last_launch(pkg)
+    print(json.dumps(line))
 
 
 def main():
@@ -618,7 +666,7 @@ def main():
                     help="print per-kernel durations of a rocprofv3 kernel trace (no GPU needed) and exit")
     ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
     ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
-                                       "sweep", "ceilings"],
+                                       "sweep", "ceilings", "operands"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
@@ -645,6 +693,9 @@ def main():
         return
     if args.mode == "ceilings":
         run_ceilings(pkg, dev)
+        return
+    if args.mode == "operands":
+        run_operands(pkg, dev)
         return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode, shape=args.shape, replay_ms=args.replay_ms)

@@ -38,6 +38,21 @@ struct GemmParams
     void const* residual = nullptr; // [m, n_out] in the output type, added last (no split-K with it)
 };
 
+// A fragments (16 rows x 32 k of 16-bit values, 1 KiB) in LDS.  The DMA that fills a fragment writes lane l's
+// 16 bytes at position l, and lane l = 4 * row + q fetches a 16-byte chunk of `row`, so that quads read
+// 64 contiguous bytes from memory; the matrix core wants lane (kg, row) to read chunk kg of `row`.  Which
+// chunk sits at position 4 * row + q is chosen so that those reads do not collide on LDS banks: a 128-bit
+// LDS read is served in four phases of 16 lanes, and the phases are NOT runs of consecutive lanes - phase 0
+// takes lanes 0-3, 12-15, 20-23, 24-27, phase 1 lanes 4-7, 8-11, 16-19, 28-31, phases 2 and 3 the same plus
+// 32 - so the four lanes of a phase that share (row mod 4) come from row blocks 0, 3 (chunk kg) and 1, 2
+// (chunk kg + 1).  With chunk kg of a row in block b at q = kg ^ frag_swizzle(b) they land on four different
+// bank groups.  (kg ^ b, conflict-free if phases were runs of 16 lanes, measures two-way conflicts on
+// every read.)
+__device__ __forceinline__ int frag_swizzle(int row_block)
+{
+    return (4 - row_block) & 3;
+}
+
 // Strip slot s of a wavefront whose first slot is `first` (even): without a gated activation strip
 // first + s; with one, slots pair up - even slot: pair (first + s) / 2 in the value half, odd
 // slot: the same pair in the gate half, `half` strips further.  `valid`: the slot's strip exists.

@@ -160,9 +160,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     static_assert(4 % SLABS == 0 && FRAGS % 4 == 0, "fragment to wavefront mapping");
     int const dma_j = wave % SLABS;
     uint32_t dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
-                                 + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
+                                 + (uint32_t) (dma_j * 32 + (((lane & 3) ^ frag_swizzle(lane >> 4)) * 8)))
         * 2u;
-    int const dma_lane_k = dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8); // k of this lane inside a tile row
+    int const dma_lane_k = dma_j * 32 + (((lane & 3) ^ frag_swizzle(lane >> 4)) * 8); // k of this lane inside a tile row
     uint32_t const dma_piece_stride = (uint32_t) (4 / SLABS) * 16u * (uint32_t) K * 2u;
     auto dma_base = [&](int kt) -> uint32_t
     {
@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             dma_piece(buf, base, i);
     };
     // where MFMA lane (kg, c) finds its operand (row c, chunk kg) inside a fragment
-    int const a_lane_off = (c * 4 + (kg ^ ((c >> 2) & 3))) * 16;
+    int const a_lane_off = (c * 4 + (kg ^ frag_swizzle(c >> 2))) * 16;
 
     struct BStage
     {
@@ -503,7 +503,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                             }
                         }
                         dma_lane_base = ((uint32_t) (m0 + (wave / SLABS) * 16 + (lane >> 2)) * (uint32_t) K
-                                            + (uint32_t) (dma_j * 32 + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)))
+                                            + (uint32_t) (dma_j * 32 + (((lane & 3) ^ frag_swizzle(lane >> 4)) * 8)))
                             * 2u;
                     }
                     else

@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters)
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             s += acc32[i][0];
-        sink[(blockIdx.x * 256 + threadIdx.x) & 1023] = s;
+        sink[(blockIdx.x * 256 + threadIdx.x) & 511] = s;
         return;
     }
     f32x4 acc[16];
@@ -109,6 +109,9 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters)
             uint32_t const bits2 = RANDOM ? h : 0u;
             b[v][r] = KIND == 0 ? ((bits2 & 0x81FF81FFu) | 0x3C003C00u) : (bits2 & 0xB7B7B7B7u);
         }
+    // shader-clock and constant-rate (100 MHz) counters around the loop: their ratio is the clock the
+    // power management ran this wavefront at
+    uint64_t const clk0 = __builtin_readcyclecounter(), ref0 = __builtin_amdgcn_s_memrealtime();
     for (int it = 0; it < iters; ++it)
     {
 #pragma unroll
@@ -125,11 +128,17 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters)
         }
     }
     mma_drain();
+    uint64_t const clk1 = __builtin_readcyclecounter(), ref1 = __builtin_amdgcn_s_memrealtime();
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
         s += acc[i][0];
-    sink[(blockIdx.x * 256 + threadIdx.x) & 1023] = s;
+    sink[(blockIdx.x * 256 + threadIdx.x) & 511] = s;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        reinterpret_cast<uint32_t*>(sink)[1020] = (uint32_t) (clk1 - clk0);
+        reinterpret_cast<uint32_t*>(sink)[1021] = (uint32_t) (ref1 - ref0);
+    }
 }
 } // namespace
 } // namespace woq

@@ -127,14 +127,14 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
     }
 
     // A tile -> LDS, same fragment layout as the prefill kernel: fragment f = rt * SLABS + j is the
-    // 16 rows x 32 k of one MFMA; lane l = 4*r + q fetches row r's 16-byte chunk (q ^ (r>>2)), so
+    // 16 rows x 32 k of one MFMA; lane l = 4*r + q fetches row r's 16-byte chunk q ^ frag_swizzle(r>>2), so
     // quads read contiguous 64 bytes from memory and the fragment read is bank-conflict free.
     constexpr int FRAGS = RT * SLABS;
     static_assert(FRAGS % kSkinnyWaves == 0, "fragments spread evenly over the wavefronts");
     constexpr int DMA_OPS = FRAGS / kSkinnyWaves;
     auto dma_a = [&](int buf, int kt)
     {
-        int const r = lane >> 2, chunk = (lane & 3) ^ ((lane >> 4) & 3);
+        int const r = lane >> 2, chunk = (lane & 3) ^ frag_swizzle(lane >> 4);
 #pragma unroll
         for (int i = 0; i < DMA_OPS; ++i)
         {
@@ -150,7 +150,7 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
                 (int) off, 0, 0, 0);
         }
     };
-    int const a_lane_off = (c * 4 + (kg ^ ((c >> 2) & 3))) * 16;
+    int const a_lane_off = (c * 4 + (kg ^ frag_swizzle(c >> 2))) * 16;
 
     struct Stage
     {
@@ -404,6 +404,130 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         }
     };
 
+    // ---- four row tiles, int4, group scales: A fragments just in time ----------------------------
+    // With four row tiles a step uses 16 A fragments and no second set of them fits the register file, so
+    // the step above reads half of them in one burst after the barrier - eight wavefronts at once, the LDS
+    // pipe busy for about as long as the step's matrix instructions take, and nothing else running.  Here
+    // the loops are ordered (slab, row tile, strip): a fragment feeds the two strips' matrix instructions
+    // back to back and is dead afterwards, so a window of WIN fragments, refilled one per pair of
+    // mini-blocks (from the next step's tile once this step's are all requested: it has landed, see WAIT),
+    // spreads the LDS reads evenly over the step.  The sums P of both strips are live at once; a group's P
+    // is applied one mini-block before the next step's first matrix instruction overwrites it.
+    constexpr bool JIT = BITS == 4 && GROUP == 128 && RT == 4;
+    constexpr int WIN = 4;
+    u32x4 awin[WIN];
+    f32x4 pj[NS][SEGS][RT];                // P of the step in flight / pending from the previous step
+    f32x4 ps_p[SEGS][RT];                  // S that goes with the pending P
+    float sc_p[NS][SEGS], cc_p[NS][SEGS];  // s and z - OFFSET * s that go with the pending P
+#pragma unroll
+    for (int seg = 0; seg < SEGS; ++seg)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+        {
+            ps_p[seg][rt] = zero4;
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+            {
+                pj[s][seg][rt] = zero4;
+                sc_p[s][seg] = cc_p[s][seg] = 0.f;
+            }
+        }
+    // fragment f in the order of use: slab f / RT, row tile f % RT
+    auto frag_at = [&](int buf, int f) -> u32x4
+    {
+        return *reinterpret_cast<u32x4 const*>(
+            reinterpret_cast<char const*>(stage_a[buf]->a) + a_lane_off + ((f % RT) * SLABS + f / RT) * 1024);
+    };
+    auto apply_group = [&](int s, int seg, int rt)
+    {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            acc[rt][s][r] = __builtin_fmaf(
+                sc_p[s][seg], pj[s][seg][rt][r], __builtin_fmaf(cc_p[s][seg], ps_p[seg][rt][r], acc[rt][s][r]));
+    };
+    auto compute_jit = [&](int buf, int buf_next, Stage const& st)
+    {
+        char const* sc_base = reinterpret_cast<char const*>(stage_sc[buf]->sc[wave]) + c * 2;
+        uint16_t raw_s[NS][SEGS], raw_z[NS][SEGS];
+        f32x4 ps_n[SEGS][RT];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                char const* slot = sc_base + seg * (ZERO ? 512 : 256) + s * 32;
+                raw_s[s][seg] = *reinterpret_cast<uint16_t const*>(slot);
+                raw_z[s][seg] = ZERO ? *reinterpret_cast<uint16_t const*>(slot + 256) : (uint16_t) 0;
+            }
+#pragma unroll
+        for (int seg = 0; seg < SEGS; ++seg)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                ps_n[seg][rt] = sum_lds[buf][seg * RT + rt][kg];
+        __builtin_amdgcn_sched_barrier(0);
+        form_sums(buf_next);
+        __builtin_amdgcn_sched_barrier(0);
+        u32x4 b_cur[NS], b_nxt[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                b_cur[s][x] = expand_reg(st.w[s], 0, x);
+        apply_group(0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        float sc_n[NS][SEGS], cc_n[NS][SEGS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                sc_n[s][seg] = E::from_bits(raw_s[s][seg]);
+                cc_n[s][seg] = __builtin_fmaf(-OFF, sc_n[s][seg], ZERO ? E::from_bits(raw_z[s][seg]) : 0.f);
+            }
+#pragma unroll
+        for (int j = 0; j < SLABS; ++j)
+        {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+            {
+                int const f = j * RT + rt;
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    int const seg = j / SEG_SLABS;
+                    pj[s][seg][rt] = E::mma(awin[f % WIN], b_cur[s], j % SEG_SLABS == 0 ? zero4 : pj[s][seg][rt]);
+                    // the pending P that the NEXT mini-block overwrites (runs under this matrix instruction)
+                    int const t = (j * RT + rt) * NS + s + 1;
+                    int const tj = t / (RT * NS), trt = (t / NS) % RT, ts = t % NS;
+                    if (tj < SLABS && tj % SEG_SLABS == 0)
+                        apply_group(ts, tj / SEG_SLABS, trt);
+                    // one register of this strip's next operand per mini-block
+                    if (j + 1 < SLABS)
+                        b_nxt[s][rt] = expand_reg(st.w[s], j + 1, rt);
+                    if (s == NS - 1)
+                        awin[f % WIN] = f + WIN < FRAGS ? frag_at(buf, f + WIN) : frag_at(buf_next, f + WIN - FRAGS);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                b_cur[s] = b_nxt[s];
+        }
+#pragma unroll
+        for (int seg = 0; seg < SEGS; ++seg)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+            {
+                ps_p[seg][rt] = ps_n[seg][rt];
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    sc_p[s][seg] = sc_n[s][seg];
+                    cc_p[s][seg] = cc_n[s][seg];
+                }
+            }
+    };
+
     // ---- main loop --------------------------------------------------------------------------
     // Step kt: wait until everything this wavefront requested for step kt has landed, barrier (now
     // all of A(kt) is in LDS and nobody reads A(kt-1) any more), request step kt+DEPTH (its A tile
@@ -433,7 +557,13 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
         form_sums(0);
     }
     u32x4 a_set0[RT][SLABS], a_set1[RT][SLABS];
-    if constexpr (A_AHEAD && AH > 0)
+    if constexpr (JIT)
+    {
+#pragma unroll
+        for (int f = 0; f < WIN; ++f)
+            awin[f] = frag_at(0, f);
+    }
+    else if constexpr (A_AHEAD && AH > 0)
     {
         read_frags(0, a_set0);
     }
@@ -449,7 +579,12 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             fetch_b(st[(u + DEPTH) % (DEPTH + 1)], (u + DEPTH) % (DEPTH + 1), kt + u + DEPTH);
             __builtin_amdgcn_sched_barrier(0);
             if (kt + u < KT) // uniform; the requests above go on (they read zeros past the end of K)
-                compute(u, (u + 1) % (DEPTH + 1), st[u], u % 2 == 0 ? a_set0 : a_set1, u % 2 == 0 ? a_set1 : a_set0);
+            {
+                if constexpr (JIT)
+                    compute_jit(u, (u + 1) % (DEPTH + 1), st[u]);
+                else
+                    compute(u, (u + 1) % (DEPTH + 1), st[u], u % 2 == 0 ? a_set0 : a_set1, u % 2 == 0 ? a_set1 : a_set0);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -473,9 +608,22 @@ __global__ void __launch_bounds__(kSkinnyWaves * 64) __attribute__((amdgpu_waves
             acc_s[rt] = t;
         }
     }
+    if constexpr (JIT)
+    {
 #pragma unroll
-    for (int u = 0; u < UNITS; ++u)
-        apply_unit(NS - 1, u); // the last step's last strip
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    apply_group(s, seg, rt); // the last step's sums
+    }
+    else
+    {
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u)
+            apply_unit(NS - 1, u); // the last step's last strip
+    }
 
     // ---- epilogue ----------------------------------------------------------------------------
     uint16_t* out16 = static_cast<uint16_t*>(p.out);

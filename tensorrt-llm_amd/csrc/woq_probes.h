@@ -17,7 +17,9 @@ extern "C" {
  * on e4m3, 2: v_mfma_f32_32x32x16_bf16) on `workgroups` x 4 wavefronts, multiplying the same operand
  * registers every time (random_operands 0: least switching activity) or four pseudo-random operand pairs
  * in turn (1: what the power management sustains under real data); returns the floating-point
- * operations of the launch (negative on a bad argument). */
+ * operations of the launch (negative on a bad argument).  Kinds 0 and 1 also leave two 32-bit counts at
+ * sink + 4080: shader-clock cycles and ticks of the constant 100 MHz counter that the first wavefront spent
+ * in its loop (their ratio x 100 = the MHz that wavefront ran at). */
 int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream);
 int woq_probe_empty(void* sink, void* stream);
 double woq_probe_mfma(int kind, int random_operands, int iters, int workgroups, void* sink, void* stream);
