@@ -176,7 +176,8 @@ int raise_lds_once(std::atomic<uint64_t>& raised, void const* kernel, int bytes)
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess)
     {
-        uint64_t const bit = (uint64_t) 1 << (dev & 63);
+        // device ordinals from 64 on have no bit of their own: the (idempotent) call is made every time there
+        uint64_t const bit = dev < 64 ? (uint64_t) 1 << dev : 0;
         if (raised.load(std::memory_order_relaxed) & bit)
             return WOQ_OK;
         e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);

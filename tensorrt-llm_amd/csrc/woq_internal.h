@@ -321,8 +321,8 @@ bool find_tactic(woq_matmul_args const& a, Tactic& out);
 size_t tuned_split_bytes(int m, int n, int k, int quant_algo);
 
 // Raises a kernel's dynamic-LDS limit to `bytes` (hipFuncSetAttribute) on the current device, once per
-// device: `raised` holds one bit per device ordinal (ordinals from 64 on share bits, which only
-// repeats the idempotent call).  The sticky HIP error of a failed call is cleared.
+// device: `raised` holds one bit per device ordinal below 64 (for ordinals from 64 on the idempotent
+// call is simply repeated at every launch).  The sticky HIP error of a failed call is cleared.
 int raise_lds_once(std::atomic<uint64_t>& raised, void const* kernel, int bytes);
 
 // largest M the streaming kernels are instantiated for (16-bit activations; W4A8)
