@@ -610,6 +610,62 @@ def run_ceilings(pkg, dev):
     print(json.dumps(out))
 
 
+def run_timeline(pkg, dev, shape):
+    """Per-wavefront time stamps of the row decode kernel (M = 1, W4A16 g128) on one layer shape.  Needs the
+    library built with `python tensorrt-llm_amd/build.py --timeline` and selected through
+    WOQ_LIB_PATH=tensorrt-llm_amd/libwoq_timeline.so: its row kernel stamps the constant 100 MHz clock at seven
+    points of every wavefront and stores them where WOQ_TRACE_PTR (read at launch) points.  Twelve launches
+    replay from one graph after the usual settling; the stamps of launches 3-11 are reported as percentiles
+    over the wavefronts, in us after the launch's first wavefront started, medians over the launches.  The
+    stamps cost time (the same launch runs about a tenth slower than in the plain library): the figures
+    show where a wavefront waits, not what the plain kernel takes."""
+    import os
+    import numpy as np
+    k, n = dict([("8b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_8B]
+                + [("70b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_70B])[shape or "8b_gate_up"]
+    copies = copies_beyond_cache(k * n // 2, 3)
+    layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
+    act = torch.randn((1, k), device=dev).to(torch.bfloat16)
+    out = torch.empty((1, n), dtype=torch.bfloat16, device=dev)
+    launches = 12
+    waves_max = (n // 16) * 16  # one workgroup per strip, at most 16 wavefronts each
+    traces = [torch.zeros(waves_max * 10, dtype=torch.int64, device=dev) for _ in range(launches)]
+    launch(pkg, act, layers[0], out)
+    torch.cuda.synchronize()
+
+    def body():
+        for r in range(launches):
+            os.environ["WOQ_TRACE_PTR"] = hex(traces[r].data_ptr())
+            launch(pkg, act, layers[r % copies], out)
+    _, sec, _ = time_graph(body, launches, repeats=3)
+    os.environ.pop("WOQ_TRACE_PTR", None)
+    launched = last_launch(pkg)
+    if not launched.startswith("stream row") or not bool((traces[3] != 0).any()):
+        sys.exit("bench.py --mode timeline: no stamps were written - run it on a shape the row kernel serves, with "
+                 "WOQ_LIB_PATH pointing at the library built by `python tensorrt-llm_amd/build.py --timeline`")
+    stamps = {"wavefront starts": 0, "activations and weights requested": 1, "scales and zeros requested": 2,
+              "arithmetic done": 6, "sums in LDS": 7, "barrier passed": 8, "wavefront ends": 9}
+    per = {nm: [] for nm in stamps}
+    next_start, life = [], []
+    for r in range(2, launches - 1):
+        t = traces[r].cpu().numpy().reshape(-1, 10)
+        t = t[t[:, 0] != 0]
+        t0 = t[:, 0].min()
+        for nm, i in stamps.items():
+            per[nm].append([np.percentile((t[:, i] - t0) / 100.0, q) for q in (0, 10, 50, 90, 99, 100)])
+        nxt = traces[r + 1].cpu().numpy().reshape(-1, 10)
+        next_start.append((nxt[nxt[:, 0] != 0][:, 0].min() - t0) / 100.0)
+        life.append(float(np.median((t[:, 9] - t[:, 0]) / 100.0)))
+    line = {"mode": "timeline", "shape": shape or "8b_gate_up", "k": k, "n": n, "kernel": launched,
+            "us_per_launch_with_stamps": round(sec / launches * 1e6, 2), "wavefronts": int(t.shape[0]),
+            "percentiles": ["min", "p10", "p50", "p90", "p99", "max"],
+            "us_after_first_wavefront_start": {nm: [round(float(x), 2) for x in np.median(np.array(v), axis=0)]
+                                               for nm, v in per.items()},
+            "next_launch_first_wavefront_us": round(float(np.median(next_start)), 2),
+            "wavefront_life_median_us": round(float(np.median(life)), 2)}
+    print(json.dumps(line))
+
+
 def run_operands(pkg, dev, m=4096, reps=20):
     """The real prefill kernels (W4A16 g128 bf16 and W4A8 on the 8B gate_up at M = 4096) on three sets of
     operands: the benchmark's random ones, the same weights with all-zero activations, and all-zero activations
@@ -666,7 +722,7 @@ def main():
                     help="print per-kernel durations of a rocprofv3 kernel trace (no GPU needed) and exit")
     ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
     ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
-                                       "sweep", "ceilings", "operands"],
+                                       "sweep", "ceilings", "operands", "timeline"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
     ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["moe"], default="llama70b")
@@ -696,6 +752,9 @@ def main():
         return
     if args.mode == "operands":
         run_operands(pkg, dev)
+        return
+    if args.mode == "timeline":
+        run_timeline(pkg, dev, args.shape)
         return
     if args.mode != "bench":
         run_for_counters(pkg, dev, args.mode, shape=args.shape, replay_ms=args.replay_ms)

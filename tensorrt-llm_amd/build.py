@@ -96,6 +96,13 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=None)
     ap.add_argument("--changed", action="store_true", help="recompile only what changed (development)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="a second library, libwoq_timeline.so, whose row decode kernel records per-wavefront time "
+                         "stamps (-DWOQ_TIMELINE; objects in build_timeline/): for `bench.py --mode timeline`")
     a = ap.parse_args()
     _ONLY_CHANGED = a.changed
+    if a.timeline:
+        OBJ = os.path.join(HERE, "build_timeline")
+        LIB = os.path.join(HERE, "libwoq_timeline.so")
+        DEVICE_FLAGS = DEVICE_FLAGS + ["-DWOQ_TIMELINE"]
     build_lib(a.jobs)

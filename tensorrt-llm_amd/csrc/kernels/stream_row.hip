@@ -24,7 +24,8 @@ namespace woq
 {
 
 #ifdef WOQ_TIMELINE
-// per-wavefront time stamps (100 MHz constant clock) for `bench.py --mode timeline`: a build of its own
+// per-wavefront time stamps (100 MHz constant clock) for `bench.py --mode timeline`: a library of its own
+// (`build.py --timeline`), whose launcher takes the address of the stamp buffer from WOQ_TRACE_PTR
 #define WOQ_TR(i)                                                                                                      \
     do                                                                                                                 \
     {                                                                                                                  \
