@@ -280,6 +280,51 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
     return true;
 }
 
+// The multi-row streaming kernel (stream_rows.hip: up to sixteen rows, no staging pass) for this problem, and
+// its launch shape: wavefronts per workgroup, strips per workgroup, tile rows per wavefront and pass.
+// WOQ_ROWS_SHAPE="waves,ns,tiles" forces it, "0" switches it off.
+bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& waves, int& ns, int& tiles)
+{
+    if (m < 2 || m > 16 || bits != 4 || (group != 64 && group != 128) || pqs || k % group)
+        return false;
+    if (Tactic const* t = current_tactic())
+        if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)
+            return false; // a tuned launch shape of the strip-group kernel
+    EnvOverrides const& env = env_overrides();
+    if (env.rows_mode == 0 || env.has_stream_shape || env.wide_mode == 1 || env.stream_splits > 0)
+        return false;
+    if (env.rows_mode == 1)
+    {
+        waves = env.rows_shape[0], ns = env.rows_shape[1], tiles = env.rows_shape[2];
+        return true;
+    }
+    // Measured on MI355X against the staged strip-group kernels (bf16, scales + zeros; 2 tile rows per
+    // wavefront and pass, 8 wavefronts; us, staged -> this kernel).  K = 4096, 256 strips, one strip per
+    // workgroup: 5 rows 5.64 -> 4.64, 8 6.11 -> 4.95, 12 6.60 -> 5.56, 16 7.25 -> 6.05 (g64: 6.54 -> 5.17 at 8 rows);
+    // 384 strips, two strips: 5 rows 6.19 -> 5.68, 8 6.56 -> 5.88, 16 7.68 -> 7.10 (g64 6.95 -> 6.59 at 8);
+    // 1792 strips, four strips (g128 only): 3 rows 14.73 -> 13.86, 4 15.31 -> 14.14, 8 15.17 -> 14.44, 10 15.14 ->
+    // 14.85, from 12 rows on slower.  K = 8192, 640 strips, four strips (g128): 5 rows 13.89 -> 12.91, 8 14.09 ->
+    // 13.31, 10 14.21 -> 13.78, slower below 5 and above 10 rows.  Elsewhere (K = 8192 with up to 512 strips:
+    // within 5 % either way; the widest matrices; K beyond 8192, where the staged kernel splits K across
+    // workgroups) the staged kernels stay.
+    int const k_tiles = (k + 127) / 128;
+    int const strips = n / 16;
+    waves = 8, tiles = 2;
+    if (k_tiles <= 32)
+    {
+        if (strips <= 256 && m >= 5)
+            return ns = 1, true;
+        if (strips <= 512 && m >= 5)
+            return ns = 2, true;
+        if (strips >= 1024 && group == 128 && m >= 3 && m <= 10)
+            return ns = 4, true;
+        return false;
+    }
+    if (k_tiles <= 64 && strips > 512 && strips <= 1024 && group == 128 && m >= 5 && m <= 10)
+        return ns = 4, true;
+    return false;
+}
+
 // The W4A8 row kernel (stream_row_w4a8.hip) for this problem and its launch shape; WOQ_ROW_SHAPE as above.
 bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles)
 {
@@ -403,6 +448,8 @@ EnvOverrides read_env()
         o.wide_mode = std::sscanf(e, "%d,%d,%d", &o.wide_shape[0], &o.wide_shape[1], &o.wide_shape[2]) == 3 ? 1 : 0;
     if (char const* e = std::getenv("WOQ_ROW_SHAPE"))
         o.row_mode = std::sscanf(e, "%d,%d", &o.row_shape[0], &o.row_shape[1]) == 2 ? 1 : 0;
+    if (char const* e = std::getenv("WOQ_ROWS_SHAPE"))
+        o.rows_mode = std::sscanf(e, "%d,%d,%d", &o.rows_shape[0], &o.rows_shape[1], &o.rows_shape[2]) == 3 ? 1 : 0;
     if (char const* e = std::getenv("WOQ_STREAM_SLOTS"))
         o.slots_off = e[0] == '0';
     if (char const* e = std::getenv("WOQ_GEMM_KERNEL"))

@@ -1,0 +1,227 @@
+// Decode of up to sixteen rows (int4 weights, group scales) without a staging pass.
+//
+// Counterpart of the reference's small-M kernel at batch 2 ... 16
+// (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernel.h:57-146) in purpose only.  The row kernel
+// (stream_row.hip) showed what a decode launch is made of on this part: a stream at the rate of a plain read
+// with fixed pieces around it, the largest of which - scalar loads of the arguments, a staging pass, a
+// barrier - a kernel can avoid.  This is the same skeleton for more rows than fit its (group, row) packing:
+//   * plain scalar arguments, the ones the requests need among the first fourteen dwords (preloaded into
+//     SGPRs when the wavefront starts);
+//   * a workgroup owns NS neighbouring strips of 16 columns, its wavefronts split K: wavefront w takes the TPW
+//     consecutive tile rows (pass * WAVES + w) * TPW .. of it and requests everything those need at once -
+//     the activation fragments (row c of the 16x16x32 instruction's A operand is row c of the problem; rows
+//     past m lie outside the descriptor, read zeros and cost no traffic), NS x TPW weight tiles, and the
+//     scales and zeros: lane (kg, c) fetches those of tile row kg for its column c, one two-byte load per strip
+//     and table for the whole pass, and hands them to the lanes that need them with a lane permute;
+//   * an activation fragment is read once per wavefront and used for all NS strips, which is what bounds the
+//     traffic from the L2 (per workgroup m rows of activations against NS x 8 bytes per k of weights);
+//   * P = A x (q + OFFSET) per group and strip, S = A x ones per group, out += s * P + (z - OFFSET * s) * S in
+//     float32, as in the other streaming kernels; the wavefronts are added through LDS in wavefront order:
+//     results are bit-reproducible.
+#include "stream_kernel.h"
+
+namespace woq
+{
+
+struct RowsTail
+{
+    void const* bias;
+    float alpha;
+    int m;
+};
+
+template <int DT, int GROUP, bool ZERO, int WAVES, int NS, int TPW>
+__global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* weight, void const* act, void const* scales,
+    void const* zeros, int k_tiles, int strips, int groups_per_xcd, int n, int k, int act_bytes, void* out, RowsTail tail)
+{
+    using E = Elem<DT>;
+    constexpr int TK = 128;
+    constexpr int SEGS = TK / GROUP, SEG_SLABS = GROUP / 32, SLABS = TK / 32;
+    static_assert(GROUP == 64 || GROUP == 128, "group scales of 64 or 128 rows");
+    static_assert(TPW >= 1 && TPW <= 4, "tile row kg of a pass has its scales fetched by the lanes kg");
+    constexpr float OFF = Offset<DT, 4>::value;
+    constexpr uint32_t kOob = 0x80000000u;
+
+    int const groups = (strips + NS - 1) / NS;
+    int const group = xcd_strip(blockIdx.x, groups_per_xcd);
+    if (group >= groups)
+        return; // whole workgroup leaves together
+    int const strip0 = group * NS;
+
+    int const lane = threadIdx.x & 63;
+    int const wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int const c = lane & 15, kg = lane >> 4;
+    int const KT = k_tiles;
+    auto const w_rsrc = make_rsrc(weight, (uint32_t) strips * (uint32_t) KT * 1024u);
+    auto const act_rsrc = make_rsrc(act, (uint32_t) act_bytes);
+    int const groups_k = k / GROUP;
+    uint32_t const sz_bytes = (uint32_t) groups_k * (uint32_t) n * 2u;
+    auto const sc_rsrc = make_rsrc(scales, sz_bytes);
+    auto const zr_rsrc = make_rsrc(ZERO ? zeros : scales, sz_bytes);
+    // lane (kg, c): A operand row c, k offset kg * 8 inside a slab; B operand column c
+    uint32_t const a_lane = ((uint32_t) c * (uint32_t) k + (uint32_t) (kg * 8)) * 2u;
+    uint32_t wlane[NS], sc_lane[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+    {
+        bool const ok = strip0 + s < strips;
+        wlane[s] = ok ? ((uint32_t) (strip0 + s) * (uint32_t) KT * 64u + (uint32_t) lane) * 16u : kOob;
+        sc_lane[s] = ok ? (uint32_t) ((strip0 + s) * 16 + c) * 2u : kOob;
+    }
+
+    u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
+    NibbleConsts const nib = nibble_consts<DT>();
+    f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 total[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        total[s] = zero4;
+
+    int const passes = (KT + WAVES * TPW - 1) / (WAVES * TPW);
+    for (int pass = 0; pass < passes; ++pass)
+    {
+        int const kt0 = (pass * WAVES + wave) * TPW;
+        // ---- every request of the pass ----
+        u32x4 a[TPW][SLABS], w[TPW][NS];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int j = 0; j < SLABS; ++j)
+                a[i][j] = buffer_load_x4(
+                    act_rsrc, (kt0 + i) * TK + j * 32 < k ? a_lane + (uint32_t) ((kt0 + i) * TK + j * 32) * 2u : kOob);
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+                w[i][s] = buffer_load_x4(w_rsrc, kt0 + i < KT ? wlane[s] + (uint32_t) (kt0 + i) * 1024u : (uint32_t) kOob);
+        // scale (low half) and zero (high half) of tile row kt0 + kg, segment seg, strip s, column c
+        uint32_t sz[NS][SEGS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                int const g = (kt0 + kg) * SEGS + seg;
+                uint32_t const off
+                    = kg < TPW && g < groups_k ? (uint32_t) g * (uint32_t) n * 2u + sc_lane[s] : (uint32_t) kOob;
+                uint32_t const sv = buffer_load_u16(sc_rsrc, off);
+                uint32_t const zv = ZERO ? (uint32_t) buffer_load_u16(zr_rsrc, off) : 0u;
+                sz[s][seg] = sv | (zv << 16);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- products and scale application, tile row by tile row ----
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+        {
+#pragma unroll
+            for (int seg = 0; seg < SEGS; ++seg)
+            {
+                f32x4 S = zero4;
+#pragma unroll
+                for (int js = 0; js < SEG_SLABS; ++js)
+                    S = E::mma(a[i][seg * SEG_SLABS + js], ones, S);
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                {
+                    f32x4 P = zero4;
+#pragma unroll
+                    for (int js = 0; js < SEG_SLABS; ++js)
+                        P = E::mma(a[i][seg * SEG_SLABS + js], expand_int4<DT>(w[i][s][seg * SEG_SLABS + js], nib), P);
+                    // the lanes (i, c) hold this tile row's scale and zero for column c
+                    uint32_t const got = (uint32_t) __shfl((int) sz[s][seg], i * 16 + c);
+                    float const sc = E::from_bits((uint16_t) (got & 0xFFFFu));
+                    float const cc = __builtin_fmaf(-OFF, sc, ZERO ? E::from_bits((uint16_t) (got >> 16)) : 0.f);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        total[s][r] = __builtin_fmaf(sc, P[r], __builtin_fmaf(cc, S[r], total[s][r]));
+                }
+            }
+        }
+    }
+
+    // ---- the wavefronts' sums, in wavefront order ----
+    __shared__ float red[WAVES][NS][16][16];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            red[wave][s][kg * 4 + r][c] = total[s][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < NS * 256; e += WAVES * 64)
+    {
+        int const s = e >> 8, row = (e >> 4) & 15, col = e & 15;
+        float sum = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2)
+            sum += red[w2][s][row][col];
+        if (row < tail.m && strip0 + s < strips)
+        {
+            int const ocol = (strip0 + s) * 16 + col;
+            float v = tail.alpha * sum;
+            if (tail.bias)
+                v += E::load(tail.bias, ocol);
+            static_cast<uint16_t*>(out)[(size_t) row * n + ocol] = E::store(v);
+        }
+    }
+}
+
+namespace
+{
+template <int DT, int GROUP, bool ZERO, int WAVES, int NS, int TPW>
+int launch_rows_variant(StreamParams sp, hipStream_t stream)
+{
+    sp.groups = (sp.strips + NS - 1) / NS;
+    sp.groups_per_xcd = (sp.groups + 7) / 8;
+    dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
+    note_launch("stream multirow waves=%d ns=%d tpw=%d passes=%d", WAVES, NS, TPW, (sp.k_tiles + WAVES * TPW - 1) / (WAVES * TPW));
+    RowsTail tail{sp.bias, sp.alpha, sp.m};
+    int const act_bytes = sp.m * sp.k * 2;
+    hipLaunchKernelGGL((stream_rows_kernel<DT, GROUP, ZERO, WAVES, NS, TPW>), grid, block, 0, stream, sp.weight, sp.act,
+        sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes, sp.out, tail);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        return fail(WOQ_ERR_RUNTIME, "rows stream kernel launch failed: %s", hipGetErrorString(err));
+    return WOQ_OK;
+}
+
+template <int DT, int GROUP, bool ZERO>
+int launch_rows_shaped(StreamParams const& sp, int waves, int ns, int tpw, hipStream_t s)
+{
+#define WOQ_ROWS(WAVES_, NS_, TPW_)                                                                                    \
+    if (waves == WAVES_ && ns == NS_ && tpw == TPW_)                                                                   \
+        return launch_rows_variant<DT, GROUP, ZERO, WAVES_, NS_, TPW_>(sp, s);
+    WOQ_ROWS(8, 1, 2)
+    WOQ_ROWS(8, 2, 2)
+    WOQ_ROWS(8, 4, 2)
+    WOQ_ROWS(16, 2, 2)
+    WOQ_ROWS(4, 1, 4)
+#undef WOQ_ROWS
+    return fail(WOQ_ERR_UNSUPPORTED, "rows stream shape waves=%d ns=%d tpw=%d is not instantiated", waves, ns, tpw);
+}
+
+template <int DT, int GROUP>
+int launch_rows_flags(StreamParams const& sp, bool zero, int waves, int ns, int tpw, hipStream_t s)
+{
+    return zero ? launch_rows_shaped<DT, GROUP, true>(sp, waves, ns, tpw, s)
+                : launch_rows_shaped<DT, GROUP, false>(sp, waves, ns, tpw, s);
+}
+} // namespace
+
+int launch_stream_rows(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream)
+{
+    auto s = static_cast<hipStream_t>(stream);
+    if (sp.m < 1 || sp.m > 16 || (group != 64 && group != 128) || sp.k % group || sp.pqs || sp.num_experts
+        || sp.activation != kActIdentity || sp.residual)
+        return fail(WOQ_ERR_UNSUPPORTED,
+            "rows stream kernel: up to sixteen rows, int4, group size 64 or 128, no smoothing vector, plain epilogue");
+    if ((uint64_t) sp.m * (uint64_t) sp.n * 2 >= ((uint64_t) 1 << 31) || (uint64_t) sp.m * (uint64_t) sp.k * 2 >= ((uint64_t) 1 << 31))
+        return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: operand beyond 2 GiB");
+    if (dtype == WOQ_BF16)
+        return group == 64 ? launch_rows_flags<WOQ_BF16, 64>(sp, zero, waves, ns, tpw, s)
+                           : launch_rows_flags<WOQ_BF16, 128>(sp, zero, waves, ns, tpw, s);
+    return group == 64 ? launch_rows_flags<WOQ_FP16, 64>(sp, zero, waves, ns, tpw, s)
+                       : launch_rows_flags<WOQ_FP16, 128>(sp, zero, waves, ns, tpw, s);
+}
+
+} // namespace woq

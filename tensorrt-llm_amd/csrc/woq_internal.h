@@ -30,7 +30,7 @@ inline int bits_of(int quant_type)
 //   WOQ_FORCE_REGIME=stream|gemm      WOQ_STREAM_SHAPE=ns,waves,pf,lds   WOQ_WIDE_SHAPE=ns,waves,pf | 0
 //   WOQ_STREAM_SLOTS=0                WOQ_GEMM_KERNEL=exact|skinny       WOQ_GEMM_RT=4|8|16
 //   WOQ_GEMM_SPLITS=<n>               WOQ_STREAM_SPLITS=<n>              WOQ_GEMM_PERSIST=0
-//   WOQ_GEMM_COLS=192|256             WOQ_ROW_SHAPE=waves,tiles | 0
+//   WOQ_GEMM_COLS=192|256             WOQ_ROW_SHAPE=waves,tiles | 0      WOQ_ROWS_SHAPE=waves,ns,tiles | 0
 struct EnvOverrides
 {
     int regime = 0;                // woq_regime; 0 = none
@@ -40,6 +40,8 @@ struct EnvOverrides
     int wide_shape[3] = {0, 0, 0};
     int row_mode = -1;             // single-row streaming kernel: -1 built-in rule, 0 off, 1 forced shape
     int row_shape[2] = {0, 0};     // wavefronts per workgroup, tiles per wavefront and pass
+    int rows_mode = -1;            // multi-row streaming kernel (stream_rows.hip): -1 built-in rule, 0 off, 1 forced shape
+    int rows_shape[3] = {0, 0, 0}; // wavefronts per workgroup, strips per workgroup, tile rows per wavefront and pass
     bool slots_off = false;        // no group-slot variants of the streaming kernel
     int gemm_kernel = 0;           // 0 any, 1 exact-dequantize, 2 deferred-scale
     int gemm_rt = 0;               // row tiles per wavefront of the exact-dequantize / fp8 kernel

@@ -272,6 +272,64 @@ def test_row_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype
             assert err < TOL, (shape, M, zero, bias, pqs, err)
 
 
+@pytest.mark.parametrize("shape", ["8,1,2", "8,2,2", "8,4,2", "16,2,2", "4,1,4"])
+@pytest.mark.parametrize("group,dtype,K,N", [(128, "bf16", 2176, 272), (64, "fp16", 2112, 1040), (128, "fp16", 128, 16),
+                                             (64, "bf16", 4160, 528), (128, "bf16", 14336, 48)])
+def test_multirow_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, K, N):
+    """The multi-row kernel without a staging pass (a workgroup owns a few strips, its wavefronts split K and
+    request everything of a pass at once), forced through WOQ_ROWS_SHAPE for 2 ... 16 rows: K that needs several
+    passes or leaves wavefronts without tile rows, a last tile that is only half inside K (g64), a strip count
+    that the strips per workgroup do not divide, with and without zeros and bias.  With a smoothing vector the
+    call falls through to the staged kernel."""
+    woq_env(WOQ_ROWS_SHAPE=shape, WOQ_ROW_SHAPE="0")
+    for M in (2, 5, 8, 13, 16):
+        for zero, bias in [(True, True), (False, False), (True, False)]:
+            p = random_problem(oracle, M, K, N, 4, group, dtype, zero=zero, bias=bias, seed=K + N + M)
+            err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+            assert "stream multirow" in _last_launch(pkg), (M, _last_launch(pkg))
+            assert err < TOL, (shape, M, zero, bias, err)
+    p = random_problem(oracle, 8, K, N, 4, group, dtype, zero=True, pqs=True, seed=K + N)
+    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+    assert "stream multirow" not in _last_launch(pkg) and err < TOL, (_last_launch(pkg), err)
+
+
+def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
+    """The built-in rule takes the multi-row kernel for 5 ... 16 rows on narrow matrices with K up to 4096 (one
+    strip per workgroup up to 256 strips, two up to 512) and not for int8 weights, per-channel scales, one row
+    or a smoothing vector; one-hot activation rows return the dequantized weight rows through it, row for row;
+    rows past m stay untouched in the output buffer's neighbours (the kernel stores rows below m only)."""
+    K, N = 4096, 4096
+    p = random_problem(oracle, 8, K, N, 4, 128, "bf16", zero=True, seed=91)
+    auto = run_product(pkg, oracle, dev, p, 0)
+    assert "stream multirow waves=8 ns=1 tpw=2 passes=2" in _last_launch(pkg), _last_launch(pkg)
+    assert parity_err(oracle, auto, p) < TOL
+    woq_env(WOQ_ROWS_SHAPE="0")
+    staged = run_product(pkg, oracle, dev, p, 0)
+    assert "stream multirow" not in _last_launch(pkg) and parity_err(oracle, staged, p) < TOL
+    woq_env(WOQ_ROWS_SHAPE=None)
+    p = random_problem(oracle, 12, 4096, 6144, 4, 64, "fp16", zero=False, seed=92)
+    assert parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p) < TOL
+    assert "stream multirow waves=8 ns=2 tpw=2" in _last_launch(pkg), _last_launch(pkg)
+    for kw in (dict(bits=8, group=128), dict(bits=4, group=0), dict(bits=4, group=128, M=1),
+               dict(bits=4, group=128, pqs=True)):
+        q = random_problem(oracle, kw.get("M", 8), 1024, 256, kw["bits"], kw["group"], "bf16", zero=kw["group"] != 0,
+                           pqs=kw.get("pqs", False), seed=93)
+        run_product(pkg, oracle, dev, q, 0)
+        assert "stream multirow" not in _last_launch(pkg), (kw, _last_launch(pkg))
+    M, K, N = 11, 2048, 272
+    p = random_problem(oracle, M, K, N, 4, 128, "bf16", zero=True, seed=94)
+    hot = [(997 * r + 127) % K for r in range(M)]
+    p["act"] = np.zeros((M, K), np.float32)
+    for r, h in enumerate(hot):
+        p["act"][r, h] = 1.0
+    woq_env(WOQ_ROWS_SHAPE="8,2,2", WOQ_ROW_SHAPE="0")
+    out = run_product(pkg, oracle, dev, p, STREAM)
+    assert "stream multirow" in _last_launch(pkg)
+    w = oracle.dequantize(p["q"], p["scales"], p["zeros"], 128, "bf16")
+    for r, h in enumerate(hot):
+        assert (np.abs(out[r] - w[h]) <= np.abs(w[h]) * 2.0 ** -7 + 2.5e-7).all(), r
+
+
 def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev, woq_env):
     """One row, int4 with group scales of 64 or 128: the built-in rule takes the row kernel, with one pass over
     K where sixteen wavefronts x eight tiles reach that far; two rows except at K = 8192 on narrow matrices;
