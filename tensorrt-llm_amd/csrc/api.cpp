@@ -285,7 +285,8 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
 // WOQ_ROWS_SHAPE="waves,ns,tiles" forces it, "0" switches it off.
 bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& waves, int& ns, int& tiles)
 {
-    if (m < 2 || m > 16 || bits != 4 || (group != 64 && group != 128) || pqs || k % group)
+    (void) pqs; // smoothed activations cost four more requests per tile row: same classes
+    if (m < 2 || m > 16 || bits != 4 || (group != 64 && group != 128) || k % group)
         return false;
     if (Tactic const* t = current_tactic())
         if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)

@@ -12,7 +12,8 @@
 //     the activation fragments (row c of the 16x16x32 instruction's A operand is row c of the problem; rows
 //     past m lie outside the descriptor, read zeros and cost no traffic), NS x TPW weight tiles, and the
 //     scales and zeros: lane (kg, c) fetches those of tile row kg for its column c, one two-byte load per strip
-//     and table for the whole pass, and hands them to the lanes that need them with a lane permute;
+//     and table for the whole pass, and hands them to the lanes that need them with a lane permute; a
+//     smoothing vector, if any, comes as the same 8 k-values per lane for every row and is multiplied in;
 //   * an activation fragment is read once per wavefront and used for all NS strips, which is what bounds the
 //     traffic from the L2 (per workgroup m rows of activations against NS x 8 bytes per k of weights);
 //   * P = A x (q + OFFSET) per group and strip, S = A x ones per group, out += s * P + (z - OFFSET * s) * S in
@@ -25,12 +26,13 @@ namespace woq
 
 struct RowsTail
 {
+    void const* pqs; // smoothing vector [k] in the activation type, or NULL (PQS variants only)
     void const* bias;
     float alpha;
     int m;
 };
 
-template <int DT, int GROUP, bool ZERO, int WAVES, int NS, int TPW>
+template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
 __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* weight, void const* act, void const* scales,
     void const* zeros, int k_tiles, int strips, int groups_per_xcd, int n, int k, int act_bytes, void* out, RowsTail tail)
 {
@@ -58,6 +60,9 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
     uint32_t const sz_bytes = (uint32_t) groups_k * (uint32_t) n * 2u;
     auto const sc_rsrc = make_rsrc(scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? zeros : scales, sz_bytes);
+    // (with a smoothing vector the first request waits for one more scalar load: its pointer lies past the
+    // preloaded arguments)
+    auto const pq_rsrc = make_rsrc(PQS ? tail.pqs : act, (uint32_t) k * 2u);
     // lane (kg, c): A operand row c, k offset kg * 8 inside a slab; B operand column c
     uint32_t const a_lane = ((uint32_t) c * (uint32_t) k + (uint32_t) (kg * 8)) * 2u;
     uint32_t wlane[NS], sc_lane[NS];
@@ -82,13 +87,17 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
     {
         int const kt0 = (pass * WAVES + wave) * TPW;
         // ---- every request of the pass ----
-        u32x4 a[TPW][SLABS], w[TPW][NS];
+        u32x4 a[TPW][SLABS], w[TPW][NS], pq[PQS ? TPW : 1][SLABS];
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
 #pragma unroll
             for (int j = 0; j < SLABS; ++j)
-                a[i][j] = buffer_load_x4(
-                    act_rsrc, (kt0 + i) * TK + j * 32 < k ? a_lane + (uint32_t) ((kt0 + i) * TK + j * 32) * 2u : kOob);
+            {
+                bool const in_k = (kt0 + i) * TK + j * 32 < k;
+                a[i][j] = buffer_load_x4(act_rsrc, in_k ? a_lane + (uint32_t) ((kt0 + i) * TK + j * 32) * 2u : kOob);
+                if constexpr (PQS) // the same 8 k-values for every row
+                    pq[i][j] = buffer_load_x4(pq_rsrc, in_k ? (uint32_t) ((kt0 + i) * TK + j * 32 + kg * 8) * 2u : kOob);
+            }
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
 #pragma unroll
@@ -114,6 +123,14 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
         {
+            if constexpr (PQS) // T(a * s), one rounding, as the separate smoothing pass does
+            {
+#pragma unroll
+                for (int j = 0; j < SLABS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        a[i][j][r] = E::mul2(a[i][j][r], pq[i][j][r]);
+            }
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
             {
@@ -168,16 +185,16 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
 
 namespace
 {
-template <int DT, int GROUP, bool ZERO, int WAVES, int NS, int TPW>
+template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
 int launch_rows_variant(StreamParams sp, hipStream_t stream)
 {
     sp.groups = (sp.strips + NS - 1) / NS;
     sp.groups_per_xcd = (sp.groups + 7) / 8;
     dim3 grid(sp.groups_per_xcd * 8), block(WAVES * 64);
     note_launch("stream multirow waves=%d ns=%d tpw=%d passes=%d", WAVES, NS, TPW, (sp.k_tiles + WAVES * TPW - 1) / (WAVES * TPW));
-    RowsTail tail{sp.bias, sp.alpha, sp.m};
+    RowsTail tail{sp.pqs, sp.bias, sp.alpha, sp.m};
     int const act_bytes = sp.m * sp.k * 2;
-    hipLaunchKernelGGL((stream_rows_kernel<DT, GROUP, ZERO, WAVES, NS, TPW>), grid, block, 0, stream, sp.weight, sp.act,
+    hipLaunchKernelGGL((stream_rows_kernel<DT, GROUP, PQS, ZERO, WAVES, NS, TPW>), grid, block, 0, stream, sp.weight, sp.act,
         sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes, sp.out, tail);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
@@ -185,12 +202,12 @@ int launch_rows_variant(StreamParams sp, hipStream_t stream)
     return WOQ_OK;
 }
 
-template <int DT, int GROUP, bool ZERO>
+template <int DT, int GROUP, bool PQS, bool ZERO>
 int launch_rows_shaped(StreamParams const& sp, int waves, int ns, int tpw, hipStream_t s)
 {
 #define WOQ_ROWS(WAVES_, NS_, TPW_)                                                                                    \
     if (waves == WAVES_ && ns == NS_ && tpw == TPW_)                                                                   \
-        return launch_rows_variant<DT, GROUP, ZERO, WAVES_, NS_, TPW_>(sp, s);
+        return launch_rows_variant<DT, GROUP, PQS, ZERO, WAVES_, NS_, TPW_>(sp, s);
     WOQ_ROWS(8, 1, 2)
     WOQ_ROWS(8, 2, 2)
     WOQ_ROWS(8, 4, 2)
@@ -203,18 +220,20 @@ int launch_rows_shaped(StreamParams const& sp, int waves, int ns, int tpw, hipSt
 template <int DT, int GROUP>
 int launch_rows_flags(StreamParams const& sp, bool zero, int waves, int ns, int tpw, hipStream_t s)
 {
-    return zero ? launch_rows_shaped<DT, GROUP, true>(sp, waves, ns, tpw, s)
-                : launch_rows_shaped<DT, GROUP, false>(sp, waves, ns, tpw, s);
+    if (sp.pqs)
+        return zero ? launch_rows_shaped<DT, GROUP, true, true>(sp, waves, ns, tpw, s)
+                    : launch_rows_shaped<DT, GROUP, true, false>(sp, waves, ns, tpw, s);
+    return zero ? launch_rows_shaped<DT, GROUP, false, true>(sp, waves, ns, tpw, s)
+                : launch_rows_shaped<DT, GROUP, false, false>(sp, waves, ns, tpw, s);
 }
 } // namespace
 
 int launch_stream_rows(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream)
 {
     auto s = static_cast<hipStream_t>(stream);
-    if (sp.m < 1 || sp.m > 16 || (group != 64 && group != 128) || sp.k % group || sp.pqs || sp.num_experts
+    if (sp.m < 1 || sp.m > 16 || (group != 64 && group != 128) || sp.k % group || sp.num_experts
         || sp.activation != kActIdentity || sp.residual)
-        return fail(WOQ_ERR_UNSUPPORTED,
-            "rows stream kernel: up to sixteen rows, int4, group size 64 or 128, no smoothing vector, plain epilogue");
+        return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: up to sixteen rows, int4, group size 64 or 128, plain epilogue");
     if ((uint64_t) sp.m * (uint64_t) sp.n * 2 >= ((uint64_t) 1 << 31) || (uint64_t) sp.m * (uint64_t) sp.k * 2 >= ((uint64_t) 1 << 31))
         return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: operand beyond 2 GiB");
     if (dtype == WOQ_BF16)

@@ -279,24 +279,20 @@ def test_multirow_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, 
     """The multi-row kernel without a staging pass (a workgroup owns a few strips, its wavefronts split K and
     request everything of a pass at once), forced through WOQ_ROWS_SHAPE for 2 ... 16 rows: K that needs several
     passes or leaves wavefronts without tile rows, a last tile that is only half inside K (g64), a strip count
-    that the strips per workgroup do not divide, with and without zeros and bias.  With a smoothing vector the
-    call falls through to the staged kernel."""
+    that the strips per workgroup do not divide; every optional input (zeros, bias, smoothing vector)."""
     woq_env(WOQ_ROWS_SHAPE=shape, WOQ_ROW_SHAPE="0")
     for M in (2, 5, 8, 13, 16):
-        for zero, bias in [(True, True), (False, False), (True, False)]:
-            p = random_problem(oracle, M, K, N, 4, group, dtype, zero=zero, bias=bias, seed=K + N + M)
+        for zero, bias, pqs in [(True, True, True), (False, False, False), (True, False, False), (False, True, True)]:
+            p = random_problem(oracle, M, K, N, 4, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + M)
             err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
             assert "stream multirow" in _last_launch(pkg), (M, _last_launch(pkg))
-            assert err < TOL, (shape, M, zero, bias, err)
-    p = random_problem(oracle, 8, K, N, 4, group, dtype, zero=True, pqs=True, seed=K + N)
-    err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
-    assert "stream multirow" not in _last_launch(pkg) and err < TOL, (_last_launch(pkg), err)
+            assert err < TOL, (shape, M, zero, bias, pqs, err)
 
 
 def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
     """The built-in rule takes the multi-row kernel for 5 ... 16 rows on narrow matrices with K up to 4096 (one
-    strip per workgroup up to 256 strips, two up to 512) and not for int8 weights, per-channel scales, one row
-    or a smoothing vector; one-hot activation rows return the dequantized weight rows through it, row for row;
+    strip per workgroup up to 256 strips, two up to 512), with or without a smoothing vector, and not for int8
+    weights, per-channel scales or one row; one-hot activation rows return the dequantized weight rows through it, row for row;
     rows past m stay untouched in the output buffer's neighbours (the kernel stores rows below m only)."""
     K, N = 4096, 4096
     p = random_problem(oracle, 8, K, N, 4, 128, "bf16", zero=True, seed=91)
@@ -310,10 +306,10 @@ def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
     p = random_problem(oracle, 12, 4096, 6144, 4, 64, "fp16", zero=False, seed=92)
     assert parity_err(oracle, run_product(pkg, oracle, dev, p, 0), p) < TOL
     assert "stream multirow waves=8 ns=2 tpw=2" in _last_launch(pkg), _last_launch(pkg)
-    for kw in (dict(bits=8, group=128), dict(bits=4, group=0), dict(bits=4, group=128, M=1),
-               dict(bits=4, group=128, pqs=True)):
-        q = random_problem(oracle, kw.get("M", 8), 1024, 256, kw["bits"], kw["group"], "bf16", zero=kw["group"] != 0,
-                           pqs=kw.get("pqs", False), seed=93)
+    q = random_problem(oracle, 8, 1024, 256, 4, 128, "bf16", zero=True, pqs=True, seed=93)
+    assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL and "stream multirow" in _last_launch(pkg)
+    for kw in (dict(bits=8, group=128), dict(bits=4, group=0), dict(bits=4, group=128, M=1)):
+        q = random_problem(oracle, kw.get("M", 8), 1024, 256, kw["bits"], kw["group"], "bf16", zero=kw["group"] != 0, seed=93)
         run_product(pkg, oracle, dev, q, 0)
         assert "stream multirow" not in _last_launch(pkg), (kw, _last_launch(pkg))
     M, K, N = 11, 2048, 272
