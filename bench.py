@@ -721,7 +721,7 @@ def main():
     ap.add_argument("--summarize-trace", default=None, metavar="CSV",
                     help="print per-kernel durations of a rocprofv3 kernel trace (no GPU needed) and exit")
     ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
-    ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
+    ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "gemm16", "gemm8", "gemm4", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings", "operands", "timeline"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
