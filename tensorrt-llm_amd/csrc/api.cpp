@@ -280,13 +280,13 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
     return true;
 }
 
-// The multi-row streaming kernel (stream_rows.hip: up to sixteen rows, no staging pass) for this problem, and
+// The multi-row streaming kernel (stream_rows_kernel.h: up to sixteen rows, no staging pass) for this problem, and
 // its launch shape: wavefronts per workgroup, strips per workgroup, tile rows per wavefront and pass.
 // WOQ_ROWS_SHAPE="waves,ns,tiles" forces it, "0" switches it off.
 bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& waves, int& ns, int& tiles)
 {
     (void) pqs; // smoothed activations cost four more requests per tile row: same classes
-    if (m < 2 || m > 16 || bits != 4 || (group != 64 && group != 128) || k % group)
+    if (m < 1 || m > 16 || (group != 0 && group != 64 && group != 128) || (group && k % group))
         return false;
     if (Tactic const* t = current_tactic())
         if (t->regime == WOQ_REGIME_STREAM && t->ns != 0)
@@ -308,9 +308,26 @@ bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& wa
     // 13.31, 10 14.21 -> 13.78, slower below 5 and above 10 rows.  Elsewhere (K = 8192 with up to 512 strips:
     // within 5 % either way; the widest matrices; K beyond 8192, where the staged kernel splits K across
     // workgroups) the staged kernels stay.
-    int const k_tiles = (k + 127) / 128;
     int const strips = n / 16;
     waves = 8, tiles = 2;
+    if (bits == 8 && group == 0)
+    {
+        // int8 per-channel (fp16 / bf16, no zeros), same comparison: K = 4096, 256 strips, one strip per
+        // workgroup: 8 rows 6.36 -> 5.90, 16 rows 7.51 -> 6.77 (one row: 5.37 -> 5.52, not taken); 384 strips, two
+        // strips: 8 rows 7.57 -> 7.09, 16 rows 8.70 -> 8.12; wide matrices, sixteen wavefronts x two strips: 8192 x
+        // 57344 at 1 / 4 / 8 rows 83.3 -> 75.4 / 82.4 -> 75.9 / 84.7 -> 78.0, 4096 x 28672 21.3 -> 21.0 / 22.4 -> 21.1 /
+        // 22.7 -> 22.3, slower at 16 rows; K = 14336 x 256 strips and 8192 x 640 strips: no gain.
+        if (k <= 4096 && strips <= 256 && m >= 5)
+            return ns = 1, true;
+        if (k <= 4096 && strips <= 512 && m >= 5)
+            return ns = 2, true;
+        if (k <= 8192 && strips >= 1024 && m <= 8)
+            return waves = 16, ns = 2, true;
+        return false;
+    }
+    if (bits != 4 || group == 0 || m < 2)
+        return false; // int8 with group scales, int4 per-channel: not measured, the staged kernels serve them
+    int const k_tiles = (k + 127) / 128;
     if (k_tiles <= 32)
     {
         if (strips <= 256 && m >= 5)

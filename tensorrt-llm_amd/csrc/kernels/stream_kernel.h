@@ -1057,8 +1057,9 @@ bool try_launch_stream_wide(MatmulProblem const& p, StreamParams const& sp, hipS
 // the single-row kernel (stream_row.hip) and the rule that picks it and its launch shape (api.cpp)
 int launch_stream_row(StreamParams const& sp, int dtype, int group, bool pqs, bool zero, int waves, int tpw, void* stream);
 bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& tiles);
-// the multi-row kernel without a staging pass (stream_rows.hip) and its rule (api.cpp)
-int launch_stream_rows(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream);
+// the multi-row kernel without a staging pass (stream_rows_kernel.h) and its rule (api.cpp)
+int launch_stream_rows_int4(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream);
+int launch_stream_rows_int8(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream);
 bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& waves, int& ns, int& tiles);
 
 template <int DT, int BITS>
@@ -1108,7 +1109,8 @@ int launch_stream_typed(MatmulProblem const& p, void* stream)
         int ns = 0;
         if (pick_rows_shape(p.m, p.n, p.k, p.group_size, BITS, pqs, waves, ns, tiles))
         {
-            int const rc = launch_stream_rows(sp, DT, p.group_size, zero, waves, ns, tiles, stream);
+            int const rc = BITS == 4 ? launch_stream_rows_int4(sp, DT, p.group_size, zero, waves, ns, tiles, stream)
+                                     : launch_stream_rows_int8(sp, DT, p.group_size, zero, waves, ns, tiles, stream);
             if (rc != WOQ_ERR_UNSUPPORTED)
                 return rc;
         }

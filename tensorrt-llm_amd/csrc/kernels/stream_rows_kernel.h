@@ -1,4 +1,5 @@
-// Decode of up to sixteen rows (int4 weights, group scales) without a staging pass.
+// Decode of up to sixteen rows without a staging pass (int4 or int8 weights; group scales of 64 or 128 rows, or
+// per-channel scales).
 //
 // Counterpart of the reference's small-M kernel at batch 2 ... 16
 // (cpp/tensorrt_llm/kernels/weightOnlyBatchedGemv/kernel.h:57-146) in purpose only.  The row kernel
@@ -18,7 +19,11 @@
 //     traffic from the L2 (per workgroup m rows of activations against NS x 8 bytes per k of weights);
 //   * P = A x (q + OFFSET) per group and strip, S = A x ones per group, out += s * P + (z - OFFSET * s) * S in
 //     float32, as in the other streaming kernels; the wavefronts are added through LDS in wavefront order:
-//     results are bit-reproducible.
+//     results are bit-reproducible.  With per-channel scales P and S run over all of K and the scale is applied
+//     once, after the wavefronts are added.
+// Instantiated per weight width in stream_rows_int4.hip / stream_rows_int8.hip.
+#pragma once
+
 #include "stream_kernel.h"
 
 namespace woq
@@ -32,16 +37,20 @@ struct RowsTail
     int m;
 };
 
-template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
 __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* weight, void const* act, void const* scales,
     void const* zeros, int k_tiles, int strips, int groups_per_xcd, int n, int k, int act_bytes, void* out, RowsTail tail)
 {
     using E = Elem<DT>;
-    constexpr int TK = 128;
-    constexpr int SEGS = TK / GROUP, SEG_SLABS = GROUP / 32, SLABS = TK / 32;
-    static_assert(GROUP == 64 || GROUP == 128, "group scales of 64 or 128 rows");
+    constexpr int TK = BITS == 4 ? 128 : 64; // rows of K in a 1 KiB tile
+    constexpr int SLABS = TK / 32;
+    constexpr bool PER_CHANNEL = GROUP == 0;
+    constexpr int SEGS = (!PER_CHANNEL && GROUP < TK) ? TK / GROUP : 1; // scale groups inside a tile row
+    constexpr int SEG_SLABS = SLABS / SEGS;
+    static_assert(GROUP == 0 || GROUP == 64 || GROUP == 128, "per-channel scales or group scales of 64 or 128 rows");
+    static_assert(!(PER_CHANNEL && ZERO), "per-channel scales come without zeros");
     static_assert(TPW >= 1 && TPW <= 4, "tile row kg of a pass has its scales fetched by the lanes kg");
-    constexpr float OFF = Offset<DT, 4>::value;
+    constexpr float OFF = Offset<DT, BITS>::value;
     constexpr uint32_t kOob = 0x80000000u;
 
     int const groups = (strips + NS - 1) / NS;
@@ -56,7 +65,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
     int const KT = k_tiles;
     auto const w_rsrc = make_rsrc(weight, (uint32_t) strips * (uint32_t) KT * 1024u);
     auto const act_rsrc = make_rsrc(act, (uint32_t) act_bytes);
-    int const groups_k = k / GROUP;
+    int const groups_k = PER_CHANNEL ? 1 : k / (PER_CHANNEL ? 1 : GROUP);
     uint32_t const sz_bytes = (uint32_t) groups_k * (uint32_t) n * 2u;
     auto const sc_rsrc = make_rsrc(scales, sz_bytes);
     auto const zr_rsrc = make_rsrc(ZERO ? zeros : scales, sz_bytes);
@@ -77,10 +86,19 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
     u32x4 const ones = {E::kOnes, E::kOnes, E::kOnes, E::kOnes};
     NibbleConsts const nib = nibble_consts<DT>();
     f32x4 const zero4 = {0.f, 0.f, 0.f, 0.f};
-    f32x4 total[NS];
+    f32x4 total[NS];     // finished sums (group scales) / running P (per-channel)
+    f32x4 s_all = zero4; // running S of the per-channel mode
 #pragma unroll
     for (int s = 0; s < NS; ++s)
         total[s] = zero4;
+    // one slab's B operand from a lane's 16 packed bytes
+    auto expand = [&](u32x4 const& wv, int j) -> u32x4
+    {
+        if constexpr (BITS == 4)
+            return expand_int4<DT>(wv[j], nib);
+        else
+            return expand_int8<DT>(wv[2 * j], wv[2 * j + 1]);
+    };
 
     int const passes = (KT + WAVES * TPW - 1) / (WAVES * TPW);
     for (int pass = 0; pass < passes; ++pass)
@@ -105,18 +123,21 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
                 w[i][s] = buffer_load_x4(w_rsrc, kt0 + i < KT ? wlane[s] + (uint32_t) (kt0 + i) * 1024u : (uint32_t) kOob);
         // scale (low half) and zero (high half) of tile row kt0 + kg, segment seg, strip s, column c
         uint32_t sz[NS][SEGS];
+        if constexpr (!PER_CHANNEL)
+        {
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
+            for (int s = 0; s < NS; ++s)
 #pragma unroll
-            for (int seg = 0; seg < SEGS; ++seg)
-            {
-                int const g = (kt0 + kg) * SEGS + seg;
-                uint32_t const off
-                    = kg < TPW && g < groups_k ? (uint32_t) g * (uint32_t) n * 2u + sc_lane[s] : (uint32_t) kOob;
-                uint32_t const sv = buffer_load_u16(sc_rsrc, off);
-                uint32_t const zv = ZERO ? (uint32_t) buffer_load_u16(zr_rsrc, off) : 0u;
-                sz[s][seg] = sv | (zv << 16);
-            }
+                for (int seg = 0; seg < SEGS; ++seg)
+                {
+                    int const g = ((kt0 + kg) * TK + seg * (TK / SEGS)) / (PER_CHANNEL ? 1 : GROUP);
+                    uint32_t const off
+                        = kg < TPW && g < groups_k ? (uint32_t) g * (uint32_t) n * 2u + sc_lane[s] : (uint32_t) kOob;
+                    uint32_t const sv = buffer_load_u16(sc_rsrc, off);
+                    uint32_t const zv = ZERO ? (uint32_t) buffer_load_u16(zr_rsrc, off) : 0u;
+                    sz[s][seg] = sv | (zv << 16);
+                }
+        }
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- products and scale application, tile row by tile row ----
@@ -134,6 +155,18 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
 #pragma unroll
             for (int seg = 0; seg < SEGS; ++seg)
             {
+                if constexpr (PER_CHANNEL)
+                {
+#pragma unroll
+                    for (int js = 0; js < SLABS; ++js)
+                    {
+                        s_all = E::mma(a[i][js], ones, s_all);
+#pragma unroll
+                        for (int s = 0; s < NS; ++s)
+                            total[s] = E::mma(a[i][js], expand(w[i][s], js), total[s]);
+                    }
+                    continue;
+                }
                 f32x4 S = zero4;
 #pragma unroll
                 for (int js = 0; js < SEG_SLABS; ++js)
@@ -144,7 +177,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
                     f32x4 P = zero4;
 #pragma unroll
                     for (int js = 0; js < SEG_SLABS; ++js)
-                        P = E::mma(a[i][seg * SEG_SLABS + js], expand_int4<DT>(w[i][s][seg * SEG_SLABS + js], nib), P);
+                        P = E::mma(a[i][seg * SEG_SLABS + js], expand(w[i][s], seg * SEG_SLABS + js), P);
                     // the lanes (i, c) hold this tile row's scale and zero for column c
                     uint32_t const got = (uint32_t) __shfl((int) sz[s][seg], i * 16 + c);
                     float const sc = E::from_bits((uint16_t) (got & 0xFFFFu));
@@ -162,8 +195,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            red[wave][s][kg * 4 + r][c] = total[s][r];
+        for (int r = 0; r < 4; ++r) // per-channel: sum a * q = P - OFFSET * S; the column's scale follows below
+            red[wave][s][kg * 4 + r][c] = PER_CHANNEL ? __builtin_fmaf(-OFF, s_all[r], total[s][r]) : total[s][r];
     __syncthreads();
     for (int e = threadIdx.x; e < NS * 256; e += WAVES * 64)
     {
@@ -175,6 +208,8 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
         if (row < tail.m && strip0 + s < strips)
         {
             int const ocol = (strip0 + s) * 16 + col;
+            if constexpr (PER_CHANNEL)
+                sum *= E::load(scales, ocol);
             float v = tail.alpha * sum;
             if (tail.bias)
                 v += E::load(tail.bias, ocol);
@@ -183,9 +218,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_kernel(void const* wei
     }
 }
 
-namespace
-{
-template <int DT, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO, int WAVES, int NS, int TPW>
 int launch_rows_variant(StreamParams sp, hipStream_t stream)
 {
     sp.groups = (sp.strips + NS - 1) / NS;
@@ -194,20 +227,20 @@ int launch_rows_variant(StreamParams sp, hipStream_t stream)
     note_launch("stream multirow waves=%d ns=%d tpw=%d passes=%d", WAVES, NS, TPW, (sp.k_tiles + WAVES * TPW - 1) / (WAVES * TPW));
     RowsTail tail{sp.pqs, sp.bias, sp.alpha, sp.m};
     int const act_bytes = sp.m * sp.k * 2;
-    hipLaunchKernelGGL((stream_rows_kernel<DT, GROUP, PQS, ZERO, WAVES, NS, TPW>), grid, block, 0, stream, sp.weight, sp.act,
-        sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes, sp.out, tail);
+    hipLaunchKernelGGL((stream_rows_kernel<DT, BITS, GROUP, PQS, ZERO, WAVES, NS, TPW>), grid, block, 0, stream, sp.weight,
+        sp.act, sp.scales, sp.zeros, sp.k_tiles, sp.strips, sp.groups_per_xcd, sp.n, sp.k, act_bytes, sp.out, tail);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess)
         return fail(WOQ_ERR_RUNTIME, "rows stream kernel launch failed: %s", hipGetErrorString(err));
     return WOQ_OK;
 }
 
-template <int DT, int GROUP, bool PQS, bool ZERO>
+template <int DT, int BITS, int GROUP, bool PQS, bool ZERO>
 int launch_rows_shaped(StreamParams const& sp, int waves, int ns, int tpw, hipStream_t s)
 {
 #define WOQ_ROWS(WAVES_, NS_, TPW_)                                                                                    \
     if (waves == WAVES_ && ns == NS_ && tpw == TPW_)                                                                   \
-        return launch_rows_variant<DT, GROUP, PQS, ZERO, WAVES_, NS_, TPW_>(sp, s);
+        return launch_rows_variant<DT, BITS, GROUP, PQS, ZERO, WAVES_, NS_, TPW_>(sp, s);
     WOQ_ROWS(8, 1, 2)
     WOQ_ROWS(8, 2, 2)
     WOQ_ROWS(8, 4, 2)
@@ -217,30 +250,44 @@ int launch_rows_shaped(StreamParams const& sp, int waves, int ns, int tpw, hipSt
     return fail(WOQ_ERR_UNSUPPORTED, "rows stream shape waves=%d ns=%d tpw=%d is not instantiated", waves, ns, tpw);
 }
 
-template <int DT, int GROUP>
+template <int DT, int BITS, int GROUP>
 int launch_rows_flags(StreamParams const& sp, bool zero, int waves, int ns, int tpw, hipStream_t s)
 {
-    if (sp.pqs)
-        return zero ? launch_rows_shaped<DT, GROUP, true, true>(sp, waves, ns, tpw, s)
-                    : launch_rows_shaped<DT, GROUP, true, false>(sp, waves, ns, tpw, s);
-    return zero ? launch_rows_shaped<DT, GROUP, false, true>(sp, waves, ns, tpw, s)
-                : launch_rows_shaped<DT, GROUP, false, false>(sp, waves, ns, tpw, s);
+    if constexpr (GROUP == 0)
+    {
+        if (zero)
+            return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: per-channel scales come without zeros");
+        return sp.pqs ? launch_rows_shaped<DT, BITS, 0, true, false>(sp, waves, ns, tpw, s)
+                      : launch_rows_shaped<DT, BITS, 0, false, false>(sp, waves, ns, tpw, s);
+    }
+    else
+    {
+        if (sp.pqs)
+            return zero ? launch_rows_shaped<DT, BITS, GROUP, true, true>(sp, waves, ns, tpw, s)
+                        : launch_rows_shaped<DT, BITS, GROUP, true, false>(sp, waves, ns, tpw, s);
+        return zero ? launch_rows_shaped<DT, BITS, GROUP, false, true>(sp, waves, ns, tpw, s)
+                    : launch_rows_shaped<DT, BITS, GROUP, false, false>(sp, waves, ns, tpw, s);
+    }
 }
-} // namespace
 
-int launch_stream_rows(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream)
+// the launcher of one weight width (its translation unit instantiates every kernel of that width)
+template <int BITS>
+int launch_stream_rows_bits(StreamParams const& sp, int dtype, int group, bool zero, int waves, int ns, int tpw, void* stream)
 {
     auto s = static_cast<hipStream_t>(stream);
-    if (sp.m < 1 || sp.m > 16 || (group != 64 && group != 128) || sp.k % group || sp.num_experts
+    if (sp.m < 1 || sp.m > 16 || (group != 0 && group != 64 && group != 128) || (group && sp.k % group) || sp.num_experts
         || sp.activation != kActIdentity || sp.residual)
-        return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: up to sixteen rows, int4, group size 64 or 128, plain epilogue");
+        return fail(WOQ_ERR_UNSUPPORTED,
+            "rows stream kernel: up to sixteen rows, per-channel scales or group size 64 or 128, plain epilogue");
     if ((uint64_t) sp.m * (uint64_t) sp.n * 2 >= ((uint64_t) 1 << 31) || (uint64_t) sp.m * (uint64_t) sp.k * 2 >= ((uint64_t) 1 << 31))
         return fail(WOQ_ERR_UNSUPPORTED, "rows stream kernel: operand beyond 2 GiB");
     if (dtype == WOQ_BF16)
-        return group == 64 ? launch_rows_flags<WOQ_BF16, 64>(sp, zero, waves, ns, tpw, s)
-                           : launch_rows_flags<WOQ_BF16, 128>(sp, zero, waves, ns, tpw, s);
-    return group == 64 ? launch_rows_flags<WOQ_FP16, 64>(sp, zero, waves, ns, tpw, s)
-                       : launch_rows_flags<WOQ_FP16, 128>(sp, zero, waves, ns, tpw, s);
+        return group == 0 ? launch_rows_flags<WOQ_BF16, BITS, 0>(sp, zero, waves, ns, tpw, s)
+                          : (group == 64 ? launch_rows_flags<WOQ_BF16, BITS, 64>(sp, zero, waves, ns, tpw, s)
+                                         : launch_rows_flags<WOQ_BF16, BITS, 128>(sp, zero, waves, ns, tpw, s));
+    return group == 0 ? launch_rows_flags<WOQ_FP16, BITS, 0>(sp, zero, waves, ns, tpw, s)
+                      : (group == 64 ? launch_rows_flags<WOQ_FP16, BITS, 64>(sp, zero, waves, ns, tpw, s)
+                                     : launch_rows_flags<WOQ_FP16, BITS, 128>(sp, zero, waves, ns, tpw, s));
 }
 
 } // namespace woq

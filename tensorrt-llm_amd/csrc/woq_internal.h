@@ -40,7 +40,7 @@ struct EnvOverrides
     int wide_shape[3] = {0, 0, 0};
     int row_mode = -1;             // single-row streaming kernel: -1 built-in rule, 0 off, 1 forced shape
     int row_shape[2] = {0, 0};     // wavefronts per workgroup, tiles per wavefront and pass
-    int rows_mode = -1;            // multi-row streaming kernel (stream_rows.hip): -1 built-in rule, 0 off, 1 forced shape
+    int rows_mode = -1;            // multi-row streaming kernel (stream_rows_kernel.h): -1 built-in rule, 0 off, 1 forced shape
     int rows_shape[3] = {0, 0, 0}; // wavefronts per workgroup, strips per workgroup, tile rows per wavefront and pass
     bool slots_off = false;        // no group-slot variants of the streaming kernel
     int gemm_kernel = 0;           // 0 any, 1 exact-dequantize, 2 deferred-scale

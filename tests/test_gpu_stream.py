@@ -289,10 +289,26 @@ def test_multirow_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, 
             assert err < TOL, (shape, M, zero, bias, pqs, err)
 
 
+@pytest.mark.parametrize("shape", ["8,1,2", "8,4,2", "16,2,2"])
+@pytest.mark.parametrize("bits,group,dtype,K,N", [(8, 0, "fp16", 2112, 272), (8, 0, "bf16", 4160, 528), (8, 64, "bf16", 2112, 272),
+                                                 (8, 128, "fp16", 1408, 1040), (4, 0, "bf16", 2176, 272), (4, 0, "fp16", 128, 16)])
+def test_multirow_kernel_forced_int8_and_per_channel(pkg, oracle, dev, woq_env, shape, bits, group, dtype, K, N):
+    """The multi-row kernel's other weight formats, forced through WOQ_ROWS_SHAPE: int8 (64 rows of K per tile)
+    with per-channel scales or group scales of 64 / 128 rows (a group of 128 spans two tile rows), int4 with
+    per-channel scales; 1 ... 16 rows, zeros where the format has them, bias, smoothing vector."""
+    woq_env(WOQ_ROWS_SHAPE=shape, WOQ_ROW_SHAPE="0")
+    for M in (1, 3, 8, 16):
+        for zero, bias, pqs in [(group != 0, True, True), (False, False, False)]:
+            p = random_problem(oracle, M, K, N, bits, group, dtype, zero=zero, bias=bias, pqs=pqs, seed=K + N + M + bits)
+            err = parity_err(oracle, run_product(pkg, oracle, dev, p, STREAM), p)
+            assert "stream multirow" in _last_launch(pkg), (M, _last_launch(pkg))
+            assert err < TOL, (shape, M, zero, bias, pqs, err)
+
+
 def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
     """The built-in rule takes the multi-row kernel for 5 ... 16 rows on narrow matrices with K up to 4096 (one
-    strip per workgroup up to 256 strips, two up to 512), with or without a smoothing vector, and not for int8
-    weights, per-channel scales or one row; one-hot activation rows return the dequantized weight rows through it, row for row;
+    strip per workgroup up to 256 strips, two up to 512), with or without a smoothing vector, and for int8
+    per-channel weights on the same matrices; not for int8 with group scales, int4 per-channel or one row; one-hot activation rows return the dequantized weight rows through it, row for row;
     rows past m stay untouched in the output buffer's neighbours (the kernel stores rows below m only)."""
     K, N = 4096, 4096
     p = random_problem(oracle, 8, K, N, 4, 128, "bf16", zero=True, seed=91)
@@ -308,7 +324,10 @@ def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
     assert "stream multirow waves=8 ns=2 tpw=2" in _last_launch(pkg), _last_launch(pkg)
     q = random_problem(oracle, 8, 1024, 256, 4, 128, "bf16", zero=True, pqs=True, seed=93)
     assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL and "stream multirow" in _last_launch(pkg)
-    for kw in (dict(bits=8, group=128), dict(bits=4, group=0), dict(bits=4, group=128, M=1)):
+    q = random_problem(oracle, 8, 4096, 4096, 8, 0, "fp16", seed=95)  # int8 per-channel on a narrow matrix
+    assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL
+    assert "stream multirow waves=8 ns=1 tpw=2" in _last_launch(pkg), _last_launch(pkg)
+    for kw in (dict(bits=8, group=128), dict(bits=4, group=0), dict(bits=4, group=128, M=1), dict(bits=8, group=0, M=1)):
         q = random_problem(oracle, kw.get("M", 8), 1024, 256, kw["bits"], kw["group"], "bf16", zero=kw["group"] != 0, seed=93)
         run_product(pkg, oracle, dev, q, 0)
         assert "stream multirow" not in _last_launch(pkg), (kw, _last_launch(pkg))
