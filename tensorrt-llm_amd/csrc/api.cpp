@@ -343,6 +343,46 @@ bool pick_rows_shape(int m, int n, int k, int group, int bits, bool pqs, int& wa
     return false;
 }
 
+// The W4A8 multi-row kernel (stream_rows_w4a8.hip) for this problem and its launch shape; WOQ_ROWS_SHAPE as above.
+bool pick_rows_w4a8_shape(int m, int n, int k, int& waves, int& ns, int& tiles)
+{
+    if (m < 1 || m > 16)
+        return false;
+    EnvOverrides const& env = env_overrides();
+    if (env.rows_mode == 0 || env.has_stream_shape)
+        return false;
+    if (env.rows_mode == 1)
+    {
+        waves = env.rows_shape[0], ns = env.rows_shape[1], tiles = env.rows_shape[2];
+        return true;
+    }
+    // Measured on MI355X against the staged W4A8 streaming kernel (bf16 output, symmetric g128; us, staged ->
+    // this kernel; eight wavefronts, two tile rows per wavefront and pass).  K = 4096: 256 strips, one strip per
+    // workgroup, 5 rows 5.48 -> 5.23, 10 5.98 -> 5.50, 16 6.99 -> 6.52; 384 strips, two strips, 5 rows 7.43 -> 6.46,
+    // 8 7.78 -> 6.65, 10 7.96 -> 6.72, 16 7.95 -> 7.25; 1792 strips, two strips up to 8 rows (5 rows 16.3 -> 15.2,
+    // 8 19.7 -> 16.1), four strips at 9 ... 11 (10 rows 20.4 -> 16.4), slower from 12 rows on.  K = 8192, 640 strips,
+    // four strips from 10 rows on: 10 rows 16.8 -> 15.8, 12 18.4 -> 15.7, 16 20.8 -> 16.2; slower below.  Elsewhere
+    // (K = 8192 with up to 512 strips, the widest matrices, K beyond 8192) the staged kernel stays.
+    int const k_tiles = k / 128;
+    int const strips = n / 16;
+    waves = 8, tiles = 2;
+    if (m < 5)
+        return false;
+    if (k_tiles <= 32)
+    {
+        if (strips <= 256)
+            return ns = 1, true;
+        if (strips <= 512)
+            return ns = 2, true;
+        if (strips >= 1024 && m <= 11)
+            return ns = m <= 8 ? 2 : 4, true;
+        return false;
+    }
+    if (k_tiles <= 64 && strips > 512 && strips <= 1024 && m >= 10)
+        return ns = 4, true;
+    return false;
+}
+
 // The W4A8 row kernel (stream_row_w4a8.hip) for this problem and its launch shape; WOQ_ROW_SHAPE as above.
 bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles)
 {

@@ -482,6 +482,8 @@ int launch_shaped(StreamParams const& sp, hipStream_t s)
 
 int launch_stream_row_w4a8(StreamParams const& sp, int out_dtype, int waves, int tpw, void* stream);
 bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles);
+int launch_stream_rows_w4a8(StreamParams const& sp, int out_dtype, int waves, int ns, int tpw, void* stream);
+bool pick_rows_w4a8_shape(int m, int n, int k, int& waves, int& ns, int& tiles);
 
 int launch_stream_w4a8(MatmulProblem const& p, void* stream)
 {
@@ -516,6 +518,14 @@ int launch_stream_w4a8(MatmulProblem const& p, void* stream)
         if (pick_row_w4a8_shape(p.m, p.n, p.k, waves, tiles))
         {
             int const rc = launch_stream_row_w4a8(sp, p.out_dtype, waves, tiles, stream);
+            if (rc != WOQ_ERR_UNSUPPORTED)
+                return rc;
+        }
+        // up to sixteen rows: the multi-row kernel (stream_rows_w4a8.hip), where its rule (or WOQ_ROWS_SHAPE) picks it
+        int ns = 0;
+        if (pick_rows_w4a8_shape(p.m, p.n, p.k, waves, ns, tiles))
+        {
+            int const rc = launch_stream_rows_w4a8(sp, p.out_dtype, waves, ns, tiles, stream);
             if (rc != WOQ_ERR_UNSUPPORTED)
                 return rc;
         }

@@ -372,3 +372,59 @@ def test_w4a8_row_kernel_rule_and_exact_rows(pkg, oracle, dev):
             w8 = oracle.dequantize(q, s, z, G, "fp8")
             assert np.abs(w8).max() == 448.0
             assert (out == oracle.round_f16(w8[hot])).all(), (M, K, N, z is not None)
+
+
+@pytest.mark.parametrize("shape", ["8,1,2", "8,2,2", "8,4,2", "16,2,2", "4,1,4"])
+@pytest.mark.parametrize("K,N,G", [(2048, 272, 128), (1408, 1040, 128), (128, 16, 128), (4096 + 128, 528, 256)])
+def test_w4a8_multirow_kernel_forced(pkg, oracle, dev, woq_env, shape, K, N, G):
+    """The W4A8 multi-row kernel (a workgroup owns a few strips, its wavefronts split K and request a pass at
+    once, no staging), forced through WOQ_ROWS_SHAPE for 1 ... 16 rows: several passes, wavefronts without tile
+    rows, a strip count the strips per workgroup do not divide, groups of two tile rows with a shorter last one;
+    zeros and bias; 16-bit activations through the smoothing pass and e4m3 activations handed over directly give
+    the same bits, and the staged kernel agrees."""
+    rows_g = -(-K // G)
+    for M in (1, 3, 8, 13, 16):
+        prob = oracle.make_w4a8_problem(M, K, N, seed=K + N + M, out_dtype="bf16")
+        rng = np.random.default_rng(M + K)
+        prob["scales"] = oracle.round_f16(np.exp(rng.uniform(-3, 0, (rows_g, N))).astype(np.float32))
+        zeros = oracle.round_f16((rng.standard_normal((rows_g, N)) * 2).astype(np.float32))
+        bias = oracle.round_bf16(rng.standard_normal(N).astype(np.float32))
+        for z, b in ((None, None), (zeros, bias)):
+            woq_env(WOQ_ROWS_SHAPE=shape, WOQ_ROW_SHAPE="0")
+            out, ref = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, regime=STREAM, group=G)
+            assert "stream multirow w4a8" in _launch(pkg), (M, _launch(pkg))
+            assert _perr(oracle, out, ref, prob) < TOL, (shape, M, z is not None)
+            direct, _ = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, direct_fp8=True, regime=STREAM, group=G)
+            assert (direct == out).all()
+            woq_env(WOQ_ROWS_SHAPE="0", WOQ_ROW_SHAPE="0")
+            other, _ = _run(pkg, oracle, dev, prob, M, K, N, "bf16", zeros=z, bias=b, regime=STREAM, group=G)
+            assert "stream w4a8" in _launch(pkg), _launch(pkg)
+            assert oracle.max_rel_err(other, out) < 2e-3
+
+
+def test_w4a8_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev):
+    """From five rows on, matrices with K up to 4096 (and mid-width ones with K up to 8192 from ten rows) run on
+    the multi-row kernel; one-hot rows and saturating scales come back as the e4m3-rounded dequantized weight
+    rows, bit for bit, in fp16 output."""
+    rng = np.random.default_rng(37)
+    for M, K, N, G, want in ((8, 4096, 4096, 128, "waves=8 ns=1 tpw=2"), (16, 2048, 6144 + 16, 128, "waves=8 ns=2 tpw=2"),
+                             (6, 1024, 16384, 128, "waves=8 ns=2 tpw=2"), (10, 1024, 16384 + 48, 256, "waves=8 ns=4 tpw=2"),
+                             (12, 8192, 10240, 128, "waves=8 ns=4 tpw=2"), (12, 1024, 16384, 128, None),
+                             (8, 8192, 10240, 128, None), (4, 4096, 4096, 128, None), (16, 8192 + 128, 256, 128, None)):
+        rows_g = -(-K // G)
+        q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
+        s = oracle.round_f16(np.exp(rng.uniform(-2, 4.5, (rows_g, N))).astype(np.float32))  # up to 90: saturates
+        zeros = oracle.round_f16((rng.standard_normal((rows_g, N)) * 100).astype(np.float32))
+        hot = rng.choice(K, size=M, replace=False)
+        act = np.zeros((M, K), np.float32)
+        act[np.arange(M), hot] = 1.0
+        prob = dict(q=q, scales=s, act=act, pre_quant_scale=np.ones(K, np.float32), alpha=1.0)
+        for z in (None, zeros):
+            out, _ = _run(pkg, oracle, dev, prob, M, K, N, "fp16", zeros=z, direct_fp8=True, group=G)
+            if want is None:
+                assert "stream multirow w4a8" not in _launch(pkg), (M, K, N, _launch(pkg))
+            else:
+                assert "stream multirow w4a8 " + want in _launch(pkg), (M, K, N, _launch(pkg))
+            w8 = oracle.dequantize(q, s, z, G, "fp8")
+            assert np.abs(w8).max() == 448.0
+            assert (out == oracle.round_f16(w8[hot])).all(), (M, K, N, z is not None)
