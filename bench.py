@@ -385,18 +385,21 @@ def run_for_counters(pkg, dev, mode, reps=20, shape=None, replay_ms=0):
                                         "32 rows (16 tokens, top-2)", "algorithmic_bytes_per_launch": by})
         return
     _, k, n = SHAPES_8B[2]
+    shapes = dict([("8b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_8B] + [("70b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_70B])
     if mode.startswith("w4a8_") and mode[5:].isdigit():
         m = int(mode[5:])
-        run = w4a8_setup(pkg, dev, m, k, n)
-        run()
-        finish(lambda r: run(), {"mode": mode, "kernel": "%s on gate_up K=4096 N=28672 M=%d" % (last_launch(pkg), m),
-                                 "flop_per_launch": 2.0 * m * n * k})
+        if shape:
+            k, n = shapes[shape]
+        copies = copies_beyond_cache(k * n // 2) if m <= 256 else 1
+        run = w4a8_setup(pkg, dev, m, k, n, copies=copies)
+        run(0)
+        finish(run, {"mode": mode, "kernel": "%s on %s K=%d N=%d M=%d" % (last_launch(pkg), shape or "gate_up", k, n, m),
+                     "flop_per_launch": 2.0 * m * n * k})
         return
     if mode.startswith("gemm"):
         m = int(mode[4:] or 4096)
         if shape:  # another layer shape than the 8B gate_up: "70b_qkv", "8b_down", ...
-            k, n = dict([("8b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_8B]
-                        + [("70b_" + nm, (kk, nn)) for nm, kk, nn in SHAPES_70B])[shape]
+            k, n = shapes[shape]
         # weights rotate over copies beyond the last-level cache while they matter (M <= 256), as in the sweeps
         copies = min(copies_beyond_cache(k * n // 2), 64) if m <= 256 else 1
         layers = rotated_copies(make_layer(pkg, dev, k, n, 2002), copies)
@@ -720,8 +723,8 @@ def main():
                     help="counter / trace modes: afterwards replay the launches from a HIP graph for this long")
     ap.add_argument("--summarize-trace", default=None, metavar="CSV",
                     help="print per-kernel durations of a rocprofv3 kernel trace (no GPU needed) and exit")
-    ap.add_argument("--shape", default=None, help="gemm<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
-    ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "gemm16", "gemm8", "gemm4", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_decode", "moe_decode",
+    ap.add_argument("--shape", default=None, help="gemm<M> and w4a8_<M> modes: the layer shape (8b_qkv ... 70b_down; default 8b_gate_up)")
+    ap.add_argument("--mode", choices=["bench", "dominant", "dominant70b", "copy", "gemm4096", "gemm256", "gemm128", "gemm64", "gemm32", "gemm16", "gemm8", "gemm4", "w4a8_4096", "w4a8_256", "w4a8_64", "w4a8_16", "w4a8_8", "w4a8_decode", "moe_decode",
                                        "sweep", "ceilings", "operands", "timeline"],
                     default="bench", help="dominant / copy / gemm<M>: launch only that kernel, for rocprofv3 runs; "
                                           "sweep: the table named by --sweep")
