@@ -259,10 +259,16 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
     int const k_tiles = (k + 127) / 128;
     int const strips = n / 16;
     int const segs = 128 / group;
+    // K = 14336 (112 tiles) does not fill sixteen wavefronts x eight tiles - two wavefronts idle, the others with
+    // the longest share - and takes shapes that divide it instead: one row, two passes of eight wavefronts x seven
+    // tiles, 7.78 -> 7.28 us; four rows (g128), four passes of seven wavefronts x four tiles, 9.03 -> 8.63
+    // (two and three rows: within the noise).
     if (m == 1)
     {
         tiles = 8;
         waves = k_tiles <= 32 ? 4 : (k_tiles <= 64 ? 8 : (k_tiles <= 128 ? 16 : 4));
+        if (k_tiles > 64 && k_tiles <= 128 && k_tiles % 56 == 0)
+            waves = 8, tiles = 7;
         return true;
     }
     if (m == 2)
@@ -277,6 +283,8 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
         return false;
     tiles = 4 / segs;
     waves = segs == 1 ? 8 : 16;
+    if (m == 4 && segs == 1 && k_tiles > 64 && k_tiles % 28 == 0)
+        waves = 7;
     return true;
 }
 

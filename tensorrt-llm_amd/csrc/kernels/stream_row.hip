@@ -306,6 +306,8 @@ int launch_row_shaped(StreamParams const& sp, int waves, int tpw, hipStream_t s)
     WOQ_ROW(4, 4)
     WOQ_ROW(8, 4)
     WOQ_ROW(16, 2)
+    WOQ_ROW(8, 7) // K = 14336 is 112 tiles: passes that K divides evenly, every wavefront with a full share
+    WOQ_ROW(7, 4)
 #undef WOQ_ROW
     return fail(WOQ_ERR_UNSUPPORTED, "row stream shape waves=%d tpw=%d is not instantiated", waves, tpw);
 }

@@ -252,7 +252,7 @@ def test_wide_decode_kernel_is_what_wide_single_row_int8_problems_run_on(pkg, or
     assert (np.abs(out[0] - w) <= np.abs(w) * 2.0 ** -7 + 2.5e-7).all()
 
 
-@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,2"])
+@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,2", "8,7", "7,4"])
 @pytest.mark.parametrize("group,dtype,K,N", [(128, "bf16", 2176, 272), (64, "fp16", 1408, 1040), (128, "fp16", 128, 16),
                                              (64, "bf16", 4160, 528), (128, "bf16", 14336, 48)])
 def test_row_decode_kernel_forced(pkg, oracle, dev, woq_env, shape, group, dtype, K, N):
@@ -371,7 +371,8 @@ def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev
     assert "stream mt=1" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, other, p) < TOL
     woq_env(WOQ_ROW_SHAPE=None)
-    for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=8 passes=1 rows=1"), (1, 14336, 128, "waves=16 tpw=8 passes=1 rows=1"),
+    for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=8 passes=1 rows=1"), (1, 14336, 128, "waves=8 tpw=7 passes=2 rows=1"), (1, 12288, 128, "waves=16 tpw=8 passes=1 rows=1"),
+                               (4, 14336, 128, "waves=7 tpw=4 passes=4 rows=4"),
                                (1, 28672, 128, "waves=4 tpw=8 passes=7 rows=1"), (1, 128, 64, "waves=4 tpw=8 passes=1 rows=1"),
                                (2, 4096, 128, "waves=8 tpw=4 passes=1 rows=2"), (2, 28672, 64, "waves=4 tpw=4 passes=14 rows=2"),
                                (3, 4096, 128, "waves=8 tpw=4 passes=1 rows=4"), (4, 14336, 64, "waves=16 tpw=2 passes=4 rows=4")):
