@@ -411,7 +411,15 @@ bool pick_row_w4a8_shape(int m, int n, int k, int& waves, int& tiles)
     // 11.6 -> 10.8; 8192 x 10240 at four rows 14.6 -> 13.4).  The conversion, not the memory system, bounds
     // this kernel (about 80 VALU instructions per KiB of weights), so the wide and long matrices, where the
     // strip-group kernel's deeper pipeline keeps more of it under the loads, stay there.
+    // K = 14336 (112 tiles) on a narrow matrix, with shapes that divide it: 14336 x 4096 at two rows, sixteen
+    // wavefronts x seven tiles, 9.21 -> 8.74 us; at four rows, two passes of fourteen x four, 10.77 -> 9.80
+    // (one row: level with the strip-group kernel, which keeps it).
     int const k_tiles = (k + 127) / 128;
+    if (k_tiles > 64 && k_tiles <= 128 && k_tiles % 56 == 0 && n <= 256 * 16 && m >= 2)
+    {
+        waves = m == 2 ? 16 : 14, tiles = m == 2 ? 7 : 4;
+        return true;
+    }
     if (k_tiles <= 32)
         waves = 8;
     else if (k_tiles <= 64 && n <= 1024 * 16)

@@ -164,6 +164,9 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_w4a8_kernel(void const*
             compute(st[0]);
         }
     }
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+        before_mode_change(total[i]);
     fp8_saturation_off();
 
     // ---- rows (lanes kg) of a wavefront, then the wavefronts, in fixed order ----
@@ -233,6 +236,8 @@ int launch_row_w4a8_shaped(StreamParams const& sp, int waves, int tpw, hipStream
     WOQ_ROW(4, 4)
     WOQ_ROW(8, 4)
     WOQ_ROW(16, 4)
+    WOQ_ROW(14, 4) // K = 14336 is 112 tiles: shapes that divide it
+    WOQ_ROW(16, 7)
 #undef WOQ_ROW
     return fail(WOQ_ERR_UNSUPPORTED, "W4A8 row stream shape waves=%d tpw=%d is not instantiated", waves, tpw);
 }

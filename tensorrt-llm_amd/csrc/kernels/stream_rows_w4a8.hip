@@ -146,6 +146,9 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_w4a8_kernel(void const
             }
         }
     }
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        before_mode_change(total[s]);
     fp8_saturation_off();
 
     // ---- the wavefronts' sums, in wavefront order ----

@@ -316,6 +316,11 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
     }
 
     // ---- cross-wavefront reduction (fixed order) and epilogue: out = T(alpha * sum + bias) ----
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            before_mode_change(acc[s][mt]);
     fp8_saturation_off();
     constexpr int SLOTS = NS * MT * 4;
     __shared__ float red[WAVES][SLOTS][64];

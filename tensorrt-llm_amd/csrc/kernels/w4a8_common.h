@@ -193,6 +193,21 @@ __device__ __forceinline__ T after_mode_change(T v)
     return v;
 }
 
+// The other side of the switch: pass every sum that the conversions feed through before_mode_change()
+// in front of fp8_saturation_off().  The statement needs the finished sum, so everything the sum depends on
+// - the matrix instructions and, through them, the conversions - stays in front of it, and volatile asm
+// statements keep their order: no conversion can be scheduled behind the switch.  (In straight-line code
+// nothing else holds them there: the one-pass row kernel with seven tiles per wavefront had its last
+// conversions moved behind the switch and returned NaN for saturating scales.)
+__device__ __forceinline__ void before_mode_change(float& v)
+{
+    asm volatile("" : "+v"(v));
+}
+__device__ __forceinline__ void before_mode_change(f32x4& v)
+{
+    asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]));
+}
+
 // Row of the [ceil(k / group_size), n] scale / zero tables that the 128-row tile row kt reads.  Groups
 // are multiples of 128 (the reference's Hopper kernels take any multiple of their K tile for e4m3
 // activations, launchers/fpA_intB_launcher_sm90.inl:190-198; the last group may be shorter): `magic` is 0

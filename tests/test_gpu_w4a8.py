@@ -319,7 +319,7 @@ def test_w4a8_flexible_groups_one_hot_rows(pkg, oracle, dev):
             assert (out == oracle.round_f16(w8[rows])).all(), (regime, z is not None)
 
 
-@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,4"])
+@pytest.mark.parametrize("shape", ["4,8", "8,8", "16,8", "4,4", "8,4", "16,4", "14,4", "16,7"])
 @pytest.mark.parametrize("K,N", [(2176, 272), (128, 16), (8192, 48), (14336, 32)])
 def test_w4a8_row_kernel_forced(pkg, oracle, dev, woq_env, shape, K, N):
     """The W4A8 row kernel (one workgroup per strip, no staging pass, weights converted through the table of
@@ -348,13 +348,15 @@ def test_w4a8_row_kernel_forced(pkg, oracle, dev, woq_env, shape, K, N):
 
 
 def test_w4a8_row_kernel_rule_and_exact_rows(pkg, oracle, dev):
-    """One to four rows with K up to 4096, or up to 8192 on at most 1024 strips, run on the row kernel; one-hot
+    """One to four rows with K up to 4096, or up to 8192 on at most 1024 strips (and two to four rows of a narrow
+    matrix with K = 14336), run on the row kernel; one-hot
     rows and saturating scales come back as the e4m3-rounded dequantized weight rows, bit for bit (the table is
     built with the arithmetic form's own FMA and saturating conversion), also with groups of 256."""
     rng = np.random.default_rng(31)
     for M, K, N, G, want in ((1, 4096, 272, 128, "waves=8 tpw=4 passes=1 rows=1"), (4, 1024, 64, 128, "waves=8 tpw=4 passes=1 rows=4"),
                              (2, 8192, 48, 256, "waves=16 tpw=4 passes=1 rows=2"), (3, 8192, 16400, 128, None),
-                             (1, 14336, 32, 128, None), (5, 1024, 64, 128, None)):
+                             (1, 14336, 32, 128, None), (5, 1024, 64, 128, None),
+                             (2, 14336, 32, 128, "waves=16 tpw=7 passes=1 rows=2"), (4, 14336, 32, 256, "waves=14 tpw=4 passes=2 rows=4")):
         rows_g = -(-K // G)
         q = rng.integers(-8, 8, size=(K, N)).astype(np.int8)
         s = oracle.round_f16(np.exp(rng.uniform(-2, 4.5, (rows_g, N))).astype(np.float32))  # up to 90: saturates
