@@ -267,6 +267,15 @@ __device__ __forceinline__ u32x4 buffer_load_x4(__amdgpu_buffer_rsrc_t rsrc, uin
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) byte_offset, 0, 0);
 }
 
+// The same load with the non-temporal hint, for data a launch reads exactly once - the packed weights of the
+// streaming kernels.  Lines fetched this way are not kept in the caches at the expense of what is reused
+// (activations, scales) and the fetch itself is cheaper: measured on MI355X, one row, 8192 x 57344 42.9 ->
+// 39.0 us (0.80 of 8 TB/s, above what a plain read with ordinary loads reaches), 4096 x 28672 12.5 -> 12.0.
+__device__ __forceinline__ u32x4 buffer_load_x4_once(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int) byte_offset, 0, 2 /* nt */);
+}
+
 __device__ __forceinline__ u32x2 buffer_load_x2(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_offset)
 {
     return __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int) byte_offset, 0, 0);

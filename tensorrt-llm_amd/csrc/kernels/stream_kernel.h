@@ -209,7 +209,7 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         uint32_t const tile_off = kt < KT ? (uint32_t) kt * 1024u : 0x80000000u; // scalar select
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
+            st.w[s] = buffer_load_x4_once(w_rsrc, wlane[s] + tile_off);
         if constexpr (!ALDS)
         {
 #pragma unroll

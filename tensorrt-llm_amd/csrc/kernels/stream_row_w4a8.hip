@@ -74,7 +74,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_row_w4a8_kernel(void const*
             st.a[j] = buffer_load_x2(act_rsrc, a_ok ? a_lane + (uint32_t) (kt_mine * 128 + j * 32) : kOob);
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
-            st.w[i] = buffer_load_x4(w_rsrc, kt0 + i < KT ? wlane + (uint32_t) (kt0 + i) * 1024u : kOob);
+            st.w[i] = buffer_load_x4_once(w_rsrc, kt0 + i < KT ? wlane + (uint32_t) (kt0 + i) * 1024u : kOob);
     };
     auto kt_of = [&](int pass) { return (pass * WAVES + wave) * TPW; };
     Stage st[1];

@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_rows_w4a8_kernel(void const
         for (int i = 0; i < TPW; ++i)
 #pragma unroll
             for (int s = 0; s < NS; ++s)
-                w[i][s] = buffer_load_x4(w_rsrc, kt0 + i < KT ? wlane[s] + (uint32_t) (kt0 + i) * 1024u : (uint32_t) kOob);
+                w[i][s] = buffer_load_x4_once(w_rsrc, kt0 + i < KT ? wlane[s] + (uint32_t) (kt0 + i) * 1024u : (uint32_t) kOob);
         // scale (low half) and zero (high half) of tile row kt0 + kg, strip s, column c
         uint32_t sz[NS];
         uint32_t const magic = tail.group_magic;

@@ -102,7 +102,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_w4a8_kernel(StreamParams p)
         uint32_t const past = kt < KT ? 0u : kPast; // scalar select: a tile row past K reads zeros everywhere
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            st.w[s] = buffer_load_x4(w_rsrc, (wlane[s] + (uint32_t) kt * 1024u) | past);
+            st.w[s] = buffer_load_x4_once(w_rsrc, (wlane[s] + (uint32_t) kt * 1024u) | past);
         if constexpr (!ALDS)
         {
 #pragma unroll

@@ -101,7 +101,7 @@ __global__ void __launch_bounds__(WAVES * 64) stream_wide_kernel(StreamParams p)
         uint32_t const tile_off = (kt < KT && has_work) ? (uint32_t) kt * 1024u : 0x80000000u;
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            st.w[s] = buffer_load_x4(w_rsrc, wlane[s] + tile_off);
+            st.w[s] = buffer_load_x4_once(w_rsrc, wlane[s] + tile_off);
     };
     // chunk `ch` of window `wnd`: row (slot) ch / (NS*2) of the scales, or of the zeros behind them
     auto window_fetch = [&](u32x4 (&wv)[WLOADS], int wnd)
