@@ -565,21 +565,26 @@ def run_ceilings(pkg, dev):
                           ("8b_gate_up 62.5 MB", 62455808), ("70b_gate_up 250 MB", 250478592)]:
         nbytes = nbytes // 65536 * 65536
         copies = (1 << 30) // nbytes
-        best = None
-        for kib, u in [(4, 4), (8, 8), (16, 8), (32, 4), (64, 8)]:
-            def body(reps=40):
-                for r in range(reps):
-                    pkg._lib.check(lib.woq_probe_read(ctypes.c_void_p(pool.data_ptr() + (r % copies) * nbytes), nbytes, kib, u,
-                                                      ctypes.c_void_p(sink.data_ptr()), stream_of()))
-            body(3)
-            torch.cuda.synchronize()
-            _, sec, launches = time_graph(body, 40, repeats=3)
-            us = sec / launches * 1e6
-            if best is None or us < best[0]:
-                best = (us, kib, u)
-        out["reads"].append({"like": label, "bytes": nbytes, "us": round(best[0], 2), "gbs": round(nbytes / best[0] / 1e3, 1),
-                             "frac_of_peak": round(nbytes / best[0] / 1e3 / HBM_PEAK_GBS, 4),
-                             "kib_per_wave": best[1], "loads_in_flight": best[2]})
+        entry = {"like": label, "bytes": nbytes}
+        for nt in (0, 1):  # ordinary loads / loads with the non-temporal hint (the streaming kernels' weight loads)
+            best = None
+            for kib, u in [(4, 4), (8, 8), (16, 8), (32, 4), (64, 8)]:
+                def body(reps=40):
+                    for r in range(reps):
+                        pkg._lib.check(lib.woq_probe_read(ctypes.c_void_p(pool.data_ptr() + (r % copies) * nbytes),
+                                                          ctypes.c_size_t(nbytes), kib, u, nt,
+                                                          ctypes.c_void_p(sink.data_ptr()), stream_of()))
+                body(3)
+                torch.cuda.synchronize()
+                _, sec, launches = time_graph(body, 40, repeats=3)
+                us = sec / launches * 1e6
+                if best is None or us < best[0]:
+                    best = (us, kib, u)
+            tag = "nontemporal_" if nt else ""
+            entry.update({tag + "us": round(best[0], 2), tag + "gbs": round(nbytes / best[0] / 1e3, 1),
+                          tag + "frac_of_peak": round(nbytes / best[0] / 1e3 / HBM_PEAK_GBS, 4),
+                          tag + "kib_per_wave": best[1], tag + "loads_in_flight": best[2]})
+        out["reads"].append(entry)
 
     def empty(reps=200):
         for _ in range(reps):

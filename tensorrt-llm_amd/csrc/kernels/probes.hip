@@ -1,8 +1,9 @@
 // Measurement probes: what the hardware allows, measured with the same harness as the kernels
 // (bench.py --mode ceilings).  No counterpart in the reference.
 //   woq_probe_read   plain streaming read of a buffer: every lane one 16-byte load per KiB, a wavefront
-//                    reads `kib_per_wave` contiguous KiB with `U` loads in flight - the HBM ceiling
-//                    the weight-streaming kernels are measured against
+//                    reads `kib_per_wave` contiguous KiB with `U` loads in flight, ordinary loads or loads
+//                    with the non-temporal hint (what the streaming kernels read their weights with) - the
+//                    HBM ceiling the weight-streaming kernels are measured against
 //   woq_probe_empty  a kernel that does nothing: the cost of a launch
 //   woq_probe_mfma   nothing but matrix instructions on every SIMD: the matrix-core ceiling, with
 //                    constant or with pseudo-random operands
@@ -15,7 +16,7 @@ namespace woq
 {
 namespace
 {
-template <int U>
+template <int U, bool NT>
 __global__ void __launch_bounds__(256) probe_read_kernel(u32x4 const* __restrict__ src, size_t kib_per_wave, size_t waves,
     unsigned* sink)
 {
@@ -29,7 +30,7 @@ __global__ void __launch_bounds__(256) probe_read_kernel(u32x4 const* __restrict
         u32x4 v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            v[u] = q[(i + u) * 64];
+            v[u] = NT ? __builtin_nontemporal_load(q + (i + u) * 64) : q[(i + u) * 64];
 #pragma unroll
         for (int u = 0; u < U; ++u)
             acc ^= v[u];
@@ -145,7 +146,8 @@ __global__ void __launch_bounds__(256) probe_mfma_kernel(float* sink, int iters)
 
 using namespace woq;
 
-extern "C" int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, void* sink, void* stream)
+extern "C" int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, int loads_in_flight, int nontemporal, void* sink,
+    void* stream)
 {
     if (!src || !sink || kib_per_wave <= 0 || bytes < (size_t) kib_per_wave * 1024)
         return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: src, sink and a buffer of at least one wavefront's share");
@@ -158,14 +160,22 @@ extern "C" int woq_probe_read(const void* src, size_t bytes, int kib_per_wave, i
     auto s = static_cast<hipStream_t>(stream);
     auto const* p = static_cast<u32x4 const*>(src);
     auto* k = static_cast<unsigned*>(sink);
+#define WOQ_PROBE(U_)                                                                                                  \
+    case U_:                                                                                                           \
+        if (nontemporal)                                                                                               \
+            hipLaunchKernelGGL((probe_read_kernel<U_, true>), grid, block, 0, s, p, (size_t) kib_per_wave, waves, k);   \
+        else                                                                                                           \
+            hipLaunchKernelGGL((probe_read_kernel<U_, false>), grid, block, 0, s, p, (size_t) kib_per_wave, waves, k);  \
+        break;
     switch (loads_in_flight)
     {
-    case 1: hipLaunchKernelGGL(probe_read_kernel<1>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
-    case 2: hipLaunchKernelGGL(probe_read_kernel<2>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
-    case 4: hipLaunchKernelGGL(probe_read_kernel<4>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
-    case 8: hipLaunchKernelGGL(probe_read_kernel<8>, grid, block, 0, s, p, (size_t) kib_per_wave, waves, k); break;
+        WOQ_PROBE(1)
+        WOQ_PROBE(2)
+        WOQ_PROBE(4)
+        WOQ_PROBE(8)
     default: return fail(WOQ_ERR_INVALID_ARGUMENT, "woq_probe_read: loads_in_flight must be 1, 2, 4 or 8");
     }
+#undef WOQ_PROBE
     hipError_t const err = hipGetLastError();
     return err == hipSuccess ? WOQ_OK : fail(WOQ_ERR_RUNTIME, "probe launch failed: %s", hipGetErrorString(err));
 }
