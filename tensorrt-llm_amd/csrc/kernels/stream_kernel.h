@@ -209,7 +209,14 @@ __device__ __forceinline__ void stream_body(StreamParams const& p)
         uint32_t const tile_off = kt < KT ? (uint32_t) kt * 1024u : 0x80000000u; // scalar select
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            st.w[s] = buffer_load_x4_once(w_rsrc, wlane[s] + tile_off);
+        {
+            // The non-temporal hint, except in the grouped kernel (ACT): a launch with few active experts on a
+            // long K is bound by latency, not bandwidth (two experts' 14336 x 4096 at one token: 20.9 us with
+            // ordinary loads, 24.4 with the hint), and an expert with more than sixteen rows reads its weights
+            // again; with 1 ... 8 rows in every expert the hint would gain 5-7 % there.
+            uint32_t const off = wlane[s] + tile_off;
+            st.w[s] = ACT ? buffer_load_x4(w_rsrc, off) : buffer_load_x4_once(w_rsrc, off);
+        }
         if constexpr (!ALDS)
         {
 #pragma unroll
