@@ -263,12 +263,20 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
     // the longest share - and takes shapes that divide it instead: one row, two passes of eight wavefronts x seven
     // tiles, 7.78 -> 7.28 us; four rows (g128), four passes of seven wavefronts x four tiles, 9.03 -> 8.63
     // (two and three rows: within the noise).
+    // With the weights read non-temporally, smaller requests per wavefront win on three classes (one row): K = 4096 on
+    // wide matrices, eight wavefronts x four tiles (4096 x 28672 11.85 -> 11.47 us; level on 384 strips, 3.7 -> 4.1 on
+    // 256); K = 8192 on up to 512 strips, two passes of eight x four (8192 x 8192 8.0 -> 7.75; level on 640 strips
+    // and on 3584); K beyond 16384, passes of four x four (28672 x 8192 21.7 -> 21.0).
     if (m == 1)
     {
         tiles = 8;
         waves = k_tiles <= 32 ? 4 : (k_tiles <= 64 ? 8 : (k_tiles <= 128 ? 16 : 4));
         if (k_tiles > 64 && k_tiles <= 128 && k_tiles % 56 == 0)
             waves = 8, tiles = 7;
+        else if ((k_tiles <= 32 && strips >= 1024) || (k_tiles > 32 && k_tiles <= 64 && strips <= 512))
+            waves = 8, tiles = 4;
+        else if (k_tiles > 128)
+            waves = 4, tiles = 4;
         return true;
     }
     if (m == 2)

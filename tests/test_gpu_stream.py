@@ -371,9 +371,9 @@ def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev
     assert "stream mt=1" in _last_launch(pkg), _last_launch(pkg)
     assert parity_err(oracle, other, p) < TOL
     woq_env(WOQ_ROW_SHAPE=None)
-    for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=8 passes=1 rows=1"), (1, 14336, 128, "waves=8 tpw=7 passes=2 rows=1"), (1, 12288, 128, "waves=16 tpw=8 passes=1 rows=1"),
+    for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=4 passes=2 rows=1"), (1, 14336, 128, "waves=8 tpw=7 passes=2 rows=1"), (1, 12288, 128, "waves=16 tpw=8 passes=1 rows=1"),
                                (4, 14336, 128, "waves=7 tpw=4 passes=4 rows=4"),
-                               (1, 28672, 128, "waves=4 tpw=8 passes=7 rows=1"), (1, 128, 64, "waves=4 tpw=8 passes=1 rows=1"),
+                               (1, 28672, 128, "waves=4 tpw=4 passes=14 rows=1"), (1, 128, 64, "waves=4 tpw=8 passes=1 rows=1"),
                                (2, 4096, 128, "waves=8 tpw=4 passes=1 rows=2"), (2, 28672, 64, "waves=4 tpw=4 passes=14 rows=2"),
                                (3, 4096, 128, "waves=8 tpw=4 passes=1 rows=4"), (4, 14336, 64, "waves=16 tpw=2 passes=4 rows=4")):
         q = random_problem(oracle, M, K2, 48, 4, group, "fp16", zero=True, bias=True, pqs=True, seed=K2 + M)
