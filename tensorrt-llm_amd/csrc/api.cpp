@@ -377,7 +377,8 @@ bool pick_rows_w4a8_shape(int m, int n, int k, int& waves, int& ns, int& tiles)
     // workgroup, 5 rows 5.48 -> 5.23, 10 5.98 -> 5.50, 16 6.99 -> 6.52; 384 strips, two strips, 5 rows 7.43 -> 6.46,
     // 8 7.78 -> 6.65, 10 7.96 -> 6.72, 16 7.95 -> 7.25; 1792 strips, two strips up to 8 rows (5 rows 16.3 -> 15.2,
     // 8 19.7 -> 16.1), four strips at 9 ... 11 (10 rows 20.4 -> 16.4), slower from 12 rows on.  K = 8192, 640 strips,
-    // four strips from 10 rows on: 10 rows 16.8 -> 15.8, 12 18.4 -> 15.7, 16 20.8 -> 16.2; slower below.  Elsewhere
+    // four strips from 12 rows on: 12 rows 17.6 -> 16.9, 16 20.2 -> 17.2 (10 rows: 16.1 -> 16.7 since the staged
+    // kernel reads its weights non-temporally); slower below.  Elsewhere
     // (K = 8192 with up to 512 strips, the widest matrices, K beyond 8192) the staged kernel stays.
     int const k_tiles = k / 128;
     int const strips = n / 16;
@@ -394,7 +395,7 @@ bool pick_rows_w4a8_shape(int m, int n, int k, int& waves, int& ns, int& tiles)
             return ns = m <= 8 ? 2 : 4, true;
         return false;
     }
-    if (k_tiles <= 64 && strips > 512 && strips <= 1024 && m >= 10)
+    if (k_tiles <= 64 && strips > 512 && strips <= 1024 && m >= 12)
         return ns = 4, true;
     return false;
 }
