@@ -208,7 +208,9 @@ def bench_decode(pkg, dev, steps, warmup, m=1):
     # dominant kernel on its own: the gate_up GEMV
     gi = 2
     _, gk, gn = SHAPES_8B[gi]
-    reps = max(steps, 50)
+    # (a graph launch costs about 40 us before its first kernel starts, whatever its length: 400 launches per
+    # replay keep that below 1 % of a launch; the step's own timing above is exactly `steps` steps, as asked)
+    reps = max(steps, 400)
     _, dom_s, dom_launches = time_graph(
         lambda: [launch(pkg, acts[gk], layers[gi][r % len(layers[gi])], outs[gi]) for r in range(reps)], reps)
     dom_launch = last_launch(pkg)  # the kernel and launch shape the timed launches ran on
