@@ -279,12 +279,18 @@ bool pick_row_shape(int m, int n, int k, int group, int bits, int& waves, int& t
             waves = 4, tiles = 4;
         return true;
     }
+    // (two rows, with the weights read non-temporally: 4096 x 4096 with four wavefronts x eight tiles 4.22 -> 3.96 us;
+    // 8192 x 8192 in passes of four x four 8.74 (strip-group kernel) -> 8.05; level on 8192 x 10240)
     if (m == 2)
     {
+        if (k_tiles > 32 && k_tiles <= 64 && strips <= 512)
+            return waves = 4, tiles = 4, true;
         if (k_tiles > 32 && k_tiles <= 64 && strips < 2048)
             return false;
         tiles = 4;
         waves = k_tiles <= 128 ? 8 : 4;
+        if (k_tiles <= 32 && strips <= 256 && segs == 1)
+            waves = 4, tiles = 8;
         return true;
     }
     if (strips > 512 || k_tiles > 128 || (k_tiles > 32 && k_tiles <= 64))

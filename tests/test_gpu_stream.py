@@ -347,7 +347,7 @@ def test_multirow_kernel_rule_and_exact_rows(pkg, oracle, dev, woq_env):
 
 def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev, woq_env):
     """One row, int4 with group scales of 64 or 128: the built-in rule takes the row kernel, with one pass over
-    K where sixteen wavefronts x eight tiles reach that far; two rows except at K = 8192 on narrow matrices;
+    K where sixteen wavefronts x eight tiles reach that far; two rows except at K = 8192 on matrices of 513 ... 2047 strips;
     three and four rows on narrow matrices with K up to 4096 or beyond 8192.  int8 weights, more rows,
     per-channel scales or larger groups do not.  Every one-hot activation returns the dequantized weight row
     through it; switched off, the strip-group kernel meets the same bar."""
@@ -374,12 +374,12 @@ def test_row_decode_kernel_is_what_few_row_int4_problems_run_on(pkg, oracle, dev
     for M, K2, group, want in ((1, 8192, 64, "waves=8 tpw=4 passes=2 rows=1"), (1, 14336, 128, "waves=8 tpw=7 passes=2 rows=1"), (1, 12288, 128, "waves=16 tpw=8 passes=1 rows=1"),
                                (4, 14336, 128, "waves=7 tpw=4 passes=4 rows=4"),
                                (1, 28672, 128, "waves=4 tpw=4 passes=14 rows=1"), (1, 128, 64, "waves=4 tpw=8 passes=1 rows=1"),
-                               (2, 4096, 128, "waves=8 tpw=4 passes=1 rows=2"), (2, 28672, 64, "waves=4 tpw=4 passes=14 rows=2"),
+                               (2, 4096, 128, "waves=4 tpw=8 passes=1 rows=2"), (2, 8192, 128, "waves=4 tpw=4 passes=4 rows=2"), (2, 28672, 64, "waves=4 tpw=4 passes=14 rows=2"),
                                (3, 4096, 128, "waves=8 tpw=4 passes=1 rows=4"), (4, 14336, 64, "waves=16 tpw=2 passes=4 rows=4")):
         q = random_problem(oracle, M, K2, 48, 4, group, "fp16", zero=True, bias=True, pqs=True, seed=K2 + M)
         assert parity_err(oracle, run_product(pkg, oracle, dev, q, 0), q) < TOL
         assert "stream row " + want in _last_launch(pkg), (M, K2, _last_launch(pkg))
-    for kw in (dict(M=5), dict(M=2, K=8192), dict(M=4, K=8192), dict(M=4, N=513 * 16), dict(bits=8, group=64),
+    for kw in (dict(M=5), dict(M=2, K=8192, N=640 * 16), dict(M=4, K=8192), dict(M=4, N=513 * 16), dict(bits=8, group=64),
                dict(group=0), dict(group=256)):
         a = dict(M=1, K=K, N=N, bits=4, group=128)
         a.update(kw)
