@@ -141,9 +141,11 @@ inline double gemm_cost_us(bool skinny, int rt, long tiles, int m, int n, int k,
     int const k_tiles = (k + tk - 1) / tk;
     double c;
     if (skinny)
-        // (two row tiles: 0.79 before the A fragments were read a step ahead; four row tiles read half a set
-        // ahead at group size 128 only - `group` is -1 where the caller does not know it)
-        c = bits == 4 ? (rt == 2 ? 0.73 : (group == 128 ? 1.19 : 1.29)) : 0.565;
+        // (two row tiles: 0.79 before the A fragments were read a step ahead; four row tiles at group size 128:
+        // 1.19 before the fragments were read just in time and placed free of LDS bank conflicts, re-measured
+        // against the exact-dequantize kernel at 48 ... 128 rows since - `group` is -1 where the caller does not
+        // know it)
+        c = bits == 4 ? (rt == 2 ? 0.73 : (group == 128 ? 1.03 : 1.29)) : 0.565;
     else
         c = bits == 4 ? 0.807 + 0.108 * rt : 0.642 + 0.0404 * rt;
     // the tiles are dealt to the 8 XCDs (32 CUs each) in equal contiguous runs: the fullest XCD
