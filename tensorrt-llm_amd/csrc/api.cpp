@@ -708,13 +708,15 @@ extern "C" int woq_select_regime(int32_t m, int32_t n, int32_t k, int32_t quant_
     // W4A8: the streaming kernel converts every weight to e4m3 in registers and still runs at
     // memory speed for one 16-row tile; with two tiles per wavefront (17..32 rows) it still beats the
     // fp8 GEMM kernel, whose 64-row tiles convert the same weights for a quarter of the rows, by 8-39 %
-    // on the Llama-3-8B / 70B shapes - except on the long-K, narrow-N ones beyond 24 rows (70B down at
-    // M = 32: 59 against 53 us); beyond that the GEMM kernel
+    // on the Llama-3-8B / 70B shapes - except on the long-K, narrow-N ones from some row count on (below);
+    // beyond that the GEMM kernel
     if (quant_algo & WOQ_ALGO_FP8_ALPHA)
     {
         if (m <= kStreamW4a8AutoMaxM)
             return WOQ_REGIME_STREAM;
-        if (m <= kStreamW4a8MaxM && !(m > 24 && k >= 2 * n))
+        // (long K on few columns: 28672 x 8192 streams up to 30 rows - 28 rows 52.2 against 57.0 us - 14336 x 4096
+        // up to 19: 24 rows 25.8 against 22.7)
+        if (m <= kStreamW4a8MaxM && !(m > (n <= 4096 ? 19 : 30) && k >= 2 * n))
             return WOQ_REGIME_STREAM;
         return WOQ_REGIME_GEMM;
     }

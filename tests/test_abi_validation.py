@@ -134,13 +134,15 @@ def test_regime_table(pkg):
         for n, k in ((4096, 4096), (6144, 4096), (8192, 8192), (2048, 4096), (5120, 8192)):
             picks = [sel(m, n, k, algo) for m in range(17, 130)]
             assert picks == sorted(picks, key=lambda r: r != L.REGIME_STREAM), (n, k, algo)
-    # W4A8: streaming kernel up to two 16-row tiles (24 rows on long-K / narrow-N shapes), the fp8 GEMM above
+    # W4A8: streaming kernel up to two 16-row tiles (30 / 19 rows on long-K shapes of 8192 / 4096 columns), the fp8 GEMM above
     assert sel(1, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
     assert sel(16, 57344, 8192, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
     assert sel(17, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
     assert sel(32, 57344, 8192, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
-    assert sel(24, 8192, 28672, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
-    assert sel(25, 8192, 28672, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
+    assert sel(30, 8192, 28672, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
+    assert sel(31, 8192, 28672, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
+    assert sel(19, 4096, 14336, L.ALGO_FP8_ALPHA) == L.REGIME_STREAM
+    assert sel(20, 4096, 14336, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
     assert sel(33, 4096, 4096, L.ALGO_FP8_ALPHA) == L.REGIME_GEMM
     rc, msg = status(pkg, m=33, quant_algo=L.ALGO_FP8_ALPHA, act_dtype=L.FP8_E4M3, regime=1)
     assert rc == -3 and "unsupported m" in msg
