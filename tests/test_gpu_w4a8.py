@@ -235,7 +235,7 @@ def test_w4a8_streaming_two_row_tiles(pkg, oracle, dev, out_dtype, M, K, N):
         gemm, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=z, bias=b, regime=GEMM)
         assert oracle.max_rel_err(gemm, out) < 2e-3
     auto, _ = _run(pkg, oracle, dev, prob, M, K, N, out_dtype, zeros=zeros, bias=bias)
-    expect_stream = not (M > 24 and K >= 2 * N)
+    expect_stream = not (M > (19 if N <= 4096 else 30) and K >= 2 * N)
     assert ("stream w4a8 mt=2" in _launch(pkg)) == expect_stream, _launch(pkg)
     if expect_stream:
         assert (auto == out).all()
